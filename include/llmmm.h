@@ -1,0 +1,122 @@
+/*
+ * llmmm.h -- C ABI of the MI355X (gfx950) implementation of LLMMM's matrix-multiplication core.
+ *
+ * Every entry point takes plain device pointers and sizes, allocates nothing, never
+ * synchronises the device and enqueues its work on the caller's HIP stream (passed as void*,
+ * NULL = default stream), exactly like the reference's host launchers.  All functions return
+ * LLMMM_OK or one of the LLMMM_ERR_* codes below; argument errors are detected before any
+ * device work is enqueued.  The C++ drop-in shims in include/llmmm/mm/ turn non-zero codes into
+ * the std::runtime_error the reference throws.
+ *
+ * Data layouts (row-major everywhere, as in the reference):
+ *   FP16/BF16 GEMM  A[m*K+k], B[k*N+n] (or Bt[n*K+k]), C[m*N+n]      src/mm/fp16/mm.cuh:102,103,236
+ *   FP8 GEMM        A[m*K+k] e4m3, As[(k/128)*M+m], Bt[n*K+k] e4m3,
+ *                   Bs[(n/128)*(K/128)+k/128], C[m*N+n], Cs[(n/128)*M+m]
+ *                                                                    examples/005.fp8.mm.cu:131,157,168,212,774,2698
+ *   e4m3 = OCP FP8 E4M3 (bias 7, max 448, no inf, NaN 0x7F/0xFF), the format of __nv_fp8_e4m3.
+ */
+#ifndef LLMMM_H
+#define LLMMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LLMMM_API __attribute__((visibility("default")))
+
+/* ---- status codes ---------------------------------------------------------------------- */
+#define LLMMM_OK 0
+#define LLMMM_ERR_NOT_ALIGNED 1      /* "M or N or K are not aligned."   src/mm/fp16/mm.cu:19-21 */
+#define LLMMM_ERR_UNSUPPORTED_TYPE 2 /* "T is not supported."            src/mm/fp16/mm.cu:15-17 */
+#define LLMMM_ERR_INVALID_ARGUMENT 3 /* null / misaligned pointer, non-positive size, bad enum    */
+#define LLMMM_ERR_WORKSPACE 4        /* workspace missing or too small for the chosen split-K     */
+#define LLMMM_ERR_RUNTIME 5          /* a HIP call failed (the reference prints and exits,        */
+                                     /* src/util/macro.h:26-33; here the caller decides)          */
+
+/* ---- enums ----------------------------------------------------------------------------- */
+#define LLMMM_DTYPE_F16 0  /* half            src/mm/fp16/mm.cu:44 */
+#define LLMMM_DTYPE_BF16 1 /* __nv_bfloat16   src/mm/fp16/mm.cu:45-46 */
+
+#define LLMMM_B_ROW_MAJOR 0  /* B[K,N], the reference layout (src/mm/fp16/mm.cuh:103) */
+#define LLMMM_B_TRANSPOSED 1 /* Bt[N,K]; an extension, same arithmetic */
+
+#define LLMMM_OUT_F32 0  /* ...__output_fp32              examples/005.fp8.mm.cu:217-225 */
+#define LLMMM_OUT_BF16 1 /* same result rounded to bf16 (no reference kernel; RNE cast of the fp32 result) */
+#define LLMMM_OUT_FP8Q 2 /* ...__C_1x128__output_fp8      examples/005.fp8.mm.cu:2467-2476 */
+
+#define LLMMM_QUANT_1x128_T 0   /* <1,128,true>    activations: scale[(n/128)*M + m]           examples/005.fp8.mm.cu:2686 */
+#define LLMMM_QUANT_128x128 1   /* <128,128,false> weights:     scale[(m/128)*ceil(N/128)+n/128] examples/005.fp8.mm.cu:2739 */
+#define LLMMM_QUANT_1x128 2     /* <1,128,false>                scale[m*ceil(N/128) + n/128] */
+#define LLMMM_QUANT_128x128_T 3 /* <128,128,true>               scale[(n/128)*M + m/128] */
+
+/* Kernel selection for llmmm_fp8_gemm_ex / llmmm_fp16_gemm_ex (the auto-tune driver's knobs).
+ * tile: LLMMM_TILE_AUTO or one of the explicit ids; split_k: 0 = auto, >= 1 explicit
+ * (only the skinny kernel splits K). */
+#define LLMMM_TILE_AUTO (-1)
+#define LLMMM_TILE_256x256 0
+#define LLMMM_TILE_128x256 1
+#define LLMMM_TILE_256x128 2
+#define LLMMM_TILE_128x128 3
+#define LLMMM_TILE_SKINNY 8 /* M <= 64 weight-streaming kernel */
+
+typedef struct llmmm_gemm_cfg {
+  int tile;
+  int split_k;
+} llmmm_gemm_cfg;
+
+/* ---- FP16 / BF16 GEMM -------------------------------------------------------------------
+ * Replaces  template<T> void LLMMM::fp16_mm(const T* A, const T* B, T* C, int M, int N, int K,
+ *                                           cudaStream_t)      src/mm/fp16/mm.h:9-10, mm.cu:6-42.
+ * C = A * B with fp32 accumulation, result rounded (nearest even) to the input type.
+ * Requires M % 128 == 0, N % 128 == 0, K % 16 == 0 (the reference: M,N % 256, K % 16; the C++
+ * shim enforces the reference's stricter rule).  Pointers must be 16-byte aligned. */
+LLMMM_API int llmmm_fp16_gemm(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int b_layout, void* stream);
+LLMMM_API int llmmm_fp16_gemm_ex(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int b_layout,
+                                 const llmmm_gemm_cfg* cfg, void* stream);
+
+/* ---- FP8 blockwise GEMM -----------------------------------------------------------------
+ * Replaces  fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(A, A_scale_transposed,
+ *             B_transposed, B_scale_transposed, C, M, N, K, stream)   examples/005.fp8.mm.cu:217-246
+ * and       fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(..., C,
+ *             C_scale_transposed, M, N, K, stream)                    examples/005.fp8.mm.cu:2467-2500,
+ *                                                                     examples/005.fp8.mm.opt.cu:468-508.
+ * C is float* (OUT_F32), bf16* (OUT_BF16) or e4m3 uint8_t* (OUT_FP8Q); Cs is only used (and
+ * required) for OUT_FP8Q.  N % 128 == 0 and K % 128 == 0 are required.  M % 128 == 0 runs the
+ * MFMA tile kernels (the reference's domain); 1 <= M <= 64 runs the weight-streaming kernel,
+ * which may split K: then `workspace` must hold llmmm_fp8_gemm_workspace() bytes, prepared once
+ * with llmmm_workspace_init().  With workspace == NULL no split is used.  Other M are rejected
+ * as not aligned.  Calls that share a workspace must be ordered on one stream. */
+LLMMM_API int llmmm_fp8_gemm(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
+                             int M, int N, int K, void* workspace, size_t workspace_bytes, void* stream);
+LLMMM_API int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
+                                int M, int N, int K, void* workspace, size_t workspace_bytes, const llmmm_gemm_cfg* cfg,
+                                void* stream);
+/* Bytes of workspace that any configuration the library may pick for this shape needs
+ * (0 when the shape never splits K).  No reference counterpart: split-K is "still to do" there
+ * (README.md:22). */
+LLMMM_API size_t llmmm_fp8_gemm_workspace(int out_kind, int M, int N, int K);
+/* Zeroes the arrival counters at the head of a workspace (a small fill kernel, safe to capture
+ * in a HIP graph).  Call once after allocating it; the kernels leave the counters at zero. */
+LLMMM_API int llmmm_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+/* The configuration llmmm_fp8_gemm would use for this shape (tune table, then heuristic). */
+LLMMM_API int llmmm_fp8_gemm_query(int out_kind, int M, int N, int K, llmmm_gemm_cfg* cfg);
+
+/* ---- FP8 blockwise quantiser ------------------------------------------------------------
+ * Replaces  template<int QUANT_M, int QUANT_N, bool SCALE_TRANSPOSE>
+ *           void fp8_blockwise_symmetric_quantization(const float* x, __nv_fp8_e4m3* q,
+ *                float* scale, int M, int N, cudaStream_t)             examples/005.fp8.mm.cu:547-563.
+ * x [M,N] fp32 -> q [M,N] e4m3 + scales (layout per `kind`).  Any M; N % 4 == 0. */
+LLMMM_API int llmmm_quant_fp8(int kind, const float* x, void* q, float* scale, int M, int N, void* stream);
+
+/* ---- misc ------------------------------------------------------------------------------- */
+LLMMM_API const char* llmmm_error_string(int code); /* the reference's exception texts for codes 1 and 2 */
+LLMMM_API const char* llmmm_last_error(void);       /* thread-local detail of the last failure */
+LLMMM_API int         llmmm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLMMM_H */

@@ -1,0 +1,19 @@
+"""llmmm_amd: MI355X (gfx950) implementation of LLMMM's matrix-multiplication core.
+
+``llmmm_amd.mm`` mirrors the reference's host entry points on torch CUDA tensors;
+``llmmm_amd._lib`` is the raw ctypes view of the C ABI in ``include/llmmm.h``.
+"""
+from . import _lib  # noqa: F401  (raises if libllmmm.so has not been built)
+from .mm import (  # noqa: F401
+    fp16_gemm,
+    fp16_mm,
+    fp8_blockwise_symmetric_quantization,
+    fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8,
+    fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16,
+    fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32,
+    make_workspace,
+    quantize_activation,
+    quantize_weight,
+    query_config,
+    workspace_bytes,
+)

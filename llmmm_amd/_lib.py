@@ -1,0 +1,67 @@
+"""ctypes binding of ``libllmmm.so`` (the C ABI declared in ``include/llmmm.h``).
+
+The library is the product: there is no Python or CPU fallback.  If it is missing, importing
+this module raises, so nothing can silently run on another path.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libllmmm.so")
+
+OK, ERR_NOT_ALIGNED, ERR_UNSUPPORTED_TYPE, ERR_INVALID_ARGUMENT, ERR_WORKSPACE, ERR_RUNTIME = range(6)
+DTYPE_F16, DTYPE_BF16 = 0, 1
+B_ROW_MAJOR, B_TRANSPOSED = 0, 1
+OUT_F32, OUT_BF16, OUT_FP8Q = 0, 1, 2
+QUANT_1x128_T, QUANT_128x128, QUANT_1x128, QUANT_128x128_T = 0, 1, 2, 3
+TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_SKINNY = -1, 0, 1, 2, 3, 8
+
+
+class GemmCfg(ctypes.Structure):
+    _fields_ = [("tile", ctypes.c_int), ("split_k", ctypes.c_int)]
+
+
+# name -> (restype, argtypes); must list every symbol include/llmmm.h declares
+_c = ctypes
+_vp, _fp, _i, _sz = _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_size_t
+SIGNATURES = {
+    "llmmm_fp16_gemm": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "llmmm_fp16_gemm_ex": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _c.POINTER(GemmCfg), _vp]),
+    "llmmm_fp8_gemm": (_i, [_i, _vp, _fp, _vp, _fp, _vp, _fp, _i, _i, _i, _vp, _sz, _vp]),
+    "llmmm_fp8_gemm_ex": (_i, [_i, _vp, _fp, _vp, _fp, _vp, _fp, _i, _i, _i, _vp, _sz, _c.POINTER(GemmCfg), _vp]),
+    "llmmm_fp8_gemm_workspace": (_sz, [_i, _i, _i, _i]),
+    "llmmm_workspace_init": (_i, [_vp, _sz, _vp]),
+    "llmmm_fp8_gemm_query": (_i, [_i, _i, _i, _i, _c.POINTER(GemmCfg)]),
+    "llmmm_quant_fp8": (_i, [_i, _fp, _vp, _fp, _i, _i, _vp]),
+    "llmmm_error_string": (_c.c_char_p, [_i]),
+    "llmmm_last_error": (_c.c_char_p, []),
+    "llmmm_version": (_i, []),
+}
+
+
+def load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "%s is missing: build it with `python -m llmmm_amd.build` (hipcc, gfx950). "
+            "There is no fallback path." % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = res, args
+    return lib
+
+
+lib = load()
+
+
+def check(code):
+    """Turn a status code into the exception the reference's launchers throw.
+
+    Codes 1 and 2 carry the reference's own texts (src/mm/fp16/mm.cu:15-21)."""
+    if code == OK:
+        return
+    text = lib.llmmm_error_string(code).decode()
+    detail = lib.llmmm_last_error().decode()
+    if code in (ERR_NOT_ALIGNED, ERR_UNSUPPORTED_TYPE):
+        raise RuntimeError(text)
+    raise RuntimeError("%s: %s" % (text, detail) if detail else text)

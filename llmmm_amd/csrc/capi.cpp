@@ -1,0 +1,256 @@
+// C-ABI layer: argument validation, kernel selection (tune table, then heuristic) and launch.
+// Mirrors the reference's host launchers: no allocation, no synchronisation, work enqueued on
+// the caller's stream (src/mm/fp16/mm.cu:6-42, examples/005.fp8.mm.cu:2466-2500).
+#include "../../include/llmmm.h"
+#include "kernels.h"
+#include "tune_table.h"
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+namespace {
+
+thread_local char g_last_error[256] = "";
+
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail(int code, const char* fmt, ...)
+{
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+constexpr size_t WS_HEADER_BYTES = 4096;  // arrival counters: one uint32 per 128-column group
+constexpr int    MAX_SPLIT_K     = 32;
+constexpr int    NUM_CUS         = 256;   // MI355X
+
+int max_split_for(int K) { return (K / 128) < MAX_SPLIT_K ? (K / 128) : MAX_SPLIT_K; }
+
+// Split count for the weight-streaming kernel: enough workgroups (one per 128 columns x split)
+// to cover the chip about twice, every split at least two 128-K slices long.
+int heuristic_split(int N, int K)
+{
+  const int groups = N / 128, kb = K / 128;
+  int       s      = (2 * NUM_CUS + groups - 1) / groups;
+  if (s > kb / 2) s = kb / 2;
+  if (s > MAX_SPLIT_K) s = MAX_SPLIT_K;
+  if (s < 1) s = 1;
+  return s;
+}
+
+// Tile for the MFMA kernels: fewest "waves" of workgroups over the 256 CUs, weighted by tile
+// area and a mild efficiency penalty for the smaller tiles (less operand reuse per byte of LDS).
+int heuristic_tile(int M, int N)
+{
+  static const struct {
+    int   id, bm, bn, per_cu;
+    float eff;
+  } cand[] = {{LLMMM_TILE_256x256, 256, 256, 1, 1.00f},
+              {LLMMM_TILE_128x256, 128, 256, 1, 0.88f},
+              {LLMMM_TILE_256x128, 256, 128, 1, 0.88f},
+              {LLMMM_TILE_128x128, 128, 128, 2, 0.75f}};
+  int   best      = -1;
+  float best_cost = 0.f;
+  for (const auto& c : cand) {
+    if (M % c.bm || N % c.bn) continue;
+    const long  tiles = (long)(M / c.bm) * (N / c.bn);
+    const long  slots = (long)NUM_CUS * c.per_cu;
+    const long  waves = (tiles + slots - 1) / slots;
+    const float cost  = (float)waves * c.per_cu * c.bm * c.bn / c.eff;
+    if (best < 0 || cost < best_cost) {
+      best      = c.id;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
+bool tile_dims(int tile, int& bm, int& bn)
+{
+  switch (tile) {
+    case LLMMM_TILE_256x256: bm = 256; bn = 256; return true;
+    case LLMMM_TILE_128x256: bm = 128; bn = 256; return true;
+    case LLMMM_TILE_256x128: bm = 256; bn = 128; return true;
+    case LLMMM_TILE_128x128: bm = 128; bn = 128; return true;
+    default: return false;
+  }
+}
+
+int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
+{
+  if (M <= 0 || N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "M, N and K must be positive (got %d, %d, %d)", M, N, K);
+  if (N % 128 || K % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+  if (M <= 64) {
+    cfg->tile    = LLMMM_TILE_SKINNY;
+    cfg->split_k = 0;
+    for (const auto& e : llmmm::kSkinnyTune)
+      if (e.N == N && e.K == K && M <= e.m_max) {
+        cfg->split_k = e.split_k;
+        break;
+      }
+    if (cfg->split_k == 0) cfg->split_k = heuristic_split(N, K);
+    return LLMMM_OK;
+  }
+  if (M % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+  cfg->tile    = -1;
+  cfg->split_k = 1;
+  for (const auto& e : llmmm::kTileTune)
+    if (e.M == M && e.N == N && e.K == K) {
+      cfg->tile = e.tile;
+      break;
+    }
+  if (cfg->tile < 0) cfg->tile = heuristic_tile(M, N);
+  return LLMMM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* llmmm_error_string(int code)
+{
+  switch (code) {
+    case LLMMM_OK: return "ok";
+    case LLMMM_ERR_NOT_ALIGNED: return "M or N or K are not aligned.";
+    case LLMMM_ERR_UNSUPPORTED_TYPE: return "T is not supported.";
+    case LLMMM_ERR_INVALID_ARGUMENT: return "invalid argument";
+    case LLMMM_ERR_WORKSPACE: return "workspace missing or too small";
+    case LLMMM_ERR_RUNTIME: return "HIP runtime error";
+    default: return "unknown error";
+  }
+}
+
+const char* llmmm_last_error(void) { return g_last_error; }
+
+int llmmm_version(void) { return 100; }
+
+int llmmm_fp16_gemm_ex(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int b_layout,
+                       const llmmm_gemm_cfg* cfg, void* stream)
+{
+  if (dtype != LLMMM_DTYPE_F16 && dtype != LLMMM_DTYPE_BF16) return fail(LLMMM_ERR_UNSUPPORTED_TYPE, "T is not supported.");
+  if (b_layout != LLMMM_B_ROW_MAJOR && b_layout != LLMMM_B_TRANSPOSED)
+    return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown B layout %d", b_layout);
+  if (M <= 0 || N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "M, N and K must be positive (got %d, %d, %d)", M, N, K);
+  if (M % 128 || N % 128 || K % 16) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+  if (!A || !B || !C) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (!aligned16(A) || !aligned16(B) || !aligned16(C)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+  if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
+    return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
+  int tile = cfg ? cfg->tile : LLMMM_TILE_AUTO;
+  if (tile == LLMMM_TILE_AUTO) {
+    for (const auto& e : llmmm::kFp16TileTune)
+      if (e.M == M && e.N == N && e.K == K) {
+        tile = e.tile;
+        break;
+      }
+    if (tile == LLMMM_TILE_AUTO) tile = heuristic_tile(M, N);
+  }
+  int bm, bn;
+  if (!tile_dims(tile, bm, bn)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown tile id %d", tile);
+  if (M % bm || N % bn) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+  const hipError_t e = llmmm::fp16_gemm_launch(dtype, b_layout, tile, A, B, C, M, N, K, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "fp16 gemm launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
+int llmmm_fp16_gemm(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int b_layout, void* stream)
+{
+  return llmmm_fp16_gemm_ex(dtype, A, B, C, M, N, K, b_layout, nullptr, stream);
+}
+
+int llmmm_fp8_gemm_query(int out_kind, int M, int N, int K, llmmm_gemm_cfg* cfg)
+{
+  if (out_kind < LLMMM_OUT_F32 || out_kind > LLMMM_OUT_FP8Q) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown output kind %d", out_kind);
+  if (!cfg) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null cfg");
+  return choose_fp8(M, N, K, cfg);
+}
+
+size_t llmmm_fp8_gemm_workspace(int out_kind, int M, int N, int K)
+{
+  (void)out_kind;
+  if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128 || M > 64) return 0;
+  return WS_HEADER_BYTES + (size_t)max_split_for(K) * M * N * sizeof(float);
+}
+
+int llmmm_workspace_init(void* workspace, size_t workspace_bytes, void* stream)
+{
+  if (!workspace || workspace_bytes < WS_HEADER_BYTES) return fail(LLMMM_ERR_WORKSPACE, "workspace must hold at least %zu bytes", WS_HEADER_BYTES);
+  if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+  const hipError_t e = llmmm::fill_u32_launch((uint32_t*)workspace, 0u, WS_HEADER_BYTES / 4, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "workspace init: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
+int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
+                      int N, int K, void* workspace, size_t workspace_bytes, const llmmm_gemm_cfg* user, void* stream)
+{
+  if (out_kind < LLMMM_OUT_F32 || out_kind > LLMMM_OUT_FP8Q) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown output kind %d", out_kind);
+  llmmm_gemm_cfg cfg;
+  const int      rc = choose_fp8(M, N, K, &cfg);
+  if (rc) return rc;
+  if (!A || !As || !Bt || !Bs || !C) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (out_kind == LLMMM_OUT_FP8Q && !Cs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "C_scale_transposed is required for fp8 output");
+  if (!aligned16(A) || !aligned16(Bt) || !aligned16(C)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+  if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
+    return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
+  if (N / 128 > (int)(WS_HEADER_BYTES / 4)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "N too large");
+  if (user) {
+    if (user->tile != LLMMM_TILE_AUTO) cfg.tile = user->tile;
+    if (user->split_k > 0) cfg.split_k = user->split_k;
+  }
+  hipError_t e;
+  if (cfg.tile == LLMMM_TILE_SKINNY) {
+    if (M > 64) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the skinny kernel handles M <= 64");
+    int split = cfg.split_k;
+    if (split > max_split_for(K)) split = max_split_for(K);
+    if (split < 1) split = 1;
+    if (!workspace) split = 1;  // documented: no workspace, no split
+    float*    partial  = nullptr;
+    unsigned* counters = nullptr;
+    if (split > 1) {
+      const size_t need = WS_HEADER_BYTES + (size_t)split * M * N * sizeof(float);
+      if (workspace_bytes < need) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace_bytes, split, need);
+      if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+      counters = (unsigned*)workspace;
+      partial  = (float*)((char*)workspace + WS_HEADER_BYTES);
+    }
+    e = llmmm::fp8_skinny_launch(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, split, partial, counters, (hipStream_t)stream);
+  }
+  else {
+    int bm, bn;
+    if (!tile_dims(cfg.tile, bm, bn)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown tile id %d", cfg.tile);
+    if (M % bm || N % bn) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+    e = llmmm::fp8_gemm_launch(out_kind, cfg.tile, A, As, Bt, Bs, C, Cs, M, N, K, (hipStream_t)stream);
+  }
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "fp8 gemm launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
+int llmmm_fp8_gemm(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N,
+                   int K, void* workspace, size_t workspace_bytes, void* stream)
+{
+  return llmmm_fp8_gemm_ex(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, workspace, workspace_bytes, nullptr, stream);
+}
+
+int llmmm_quant_fp8(int kind, const float* x, void* q, float* scale, int M, int N, void* stream)
+{
+  if (kind < LLMMM_QUANT_1x128_T || kind > LLMMM_QUANT_128x128_T) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown quantiser kind %d", kind);
+  if (M <= 0 || N <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "M and N must be positive (got %d, %d)", M, N);
+  if (N % 4) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+  if (!x || !q || !scale) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (!aligned16(x) || (reinterpret_cast<uintptr_t>(q) & 3u)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "x must be 16-byte and q 4-byte aligned");
+  if ((long)M * N >= (1L << 31)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
+  const int quant_m   = (kind == LLMMM_QUANT_1x128_T || kind == LLMMM_QUANT_1x128) ? 1 : 128;
+  const int transpose = (kind == LLMMM_QUANT_1x128_T || kind == LLMMM_QUANT_128x128_T) ? 1 : 0;
+  const hipError_t e  = llmmm::quant_fp8_launch(quant_m, transpose, x, q, scale, M, N, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "quantiser launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,305 @@
+// FP8 (OCP e4m3) blockwise-scaled GEMM for gfx950 with fp32 / bf16 output or the fused
+// per-1x128 re-quantisation of C.
+//
+//   C[m,n] = sum_kb ( sum_{k in 128-slice kb} Aq[m,k] * Bq[n,k] ) * As[kb,m] * Bs[n/128,kb]
+//
+// Replaces the reference kernels fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32
+// (examples/005.fp8.mm.cu:51-246) and ...__C_1x128__output_fp8 (canonical form
+// examples/005.fp8.mm.opt.cu:177-465).  Layouts as there: A [M,K] e4m3, A_scale_transposed
+// [K/128,M], B_transposed [N,K] e4m3, B_scale [N/128,K/128], C [M,N], C_scale_transposed
+// [N/128,M] (examples/005.fp8.mm.cu:131,157,168,212,774).
+//
+// Design:
+//  * v_mfma_f32_16x16x128_f8f6f4 (both operands e4m3): one instruction covers one 128-wide
+//    quantisation slice of a 16x16 output block, started from C = 0, so the slice's partial sum
+//    comes back as 4 fp32 registers per lane;
+//  * the slice scale As[kb,m]*Bs[nb,kb] is applied with one v_fma_f32 per accumulator
+//    (promotion once per 128-K slice, the order of examples/005.fp8.mm.cu:885-902); Bt is the
+//    row operand and A the column operand, so a lane owns one row m and its scale is a single
+//    register per 16-row fragment;
+//  * one stage = one slice: a BM x 128 B tile of A and a BN x 128 B tile of Bt, both K-major,
+//    land in LDS by LDS-direct loads (two stages in flight) and are read with ds_read_b128
+//    through the SWZ_ROWS16 placement;
+//  * fused epilogue (examples/005.fp8.mm.opt.cu:401-462): a wavefront owns 64 rows x one whole
+//    128-column quantisation group, so the row amax needs the lane's 32 values and two
+//    cross-lane steps; scale = amax/448, codes = e4m3(C * (448/amax)), saturating.
+//    A group of zeros yields scale 0 and codes 0 (the reference's unguarded 0*inf gives NaN codes).
+#include "device_common.hip.h"
+#include "kernels.h"
+
+namespace llmmm {
+
+enum { OUT_F32 = 0, OUT_BF16 = 1, OUT_FP8Q = 2 };
+
+__device__ __forceinline__ f32x4 mfma_fp8_k128(i32x8 x, i32x8 y)
+{
+  const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, z, 0, 0, 0, 0, 0, 0);
+}
+
+__device__ __forceinline__ void fp8_tile_coords(int wg, int tiles_m, int tiles_n, int& tm, int& tn)
+{
+  const int tiles = tiles_m * tiles_n;
+  int       L     = wg;
+  if ((tiles & 7) == 0) L = (wg & 7) * (tiles >> 3) + (wg >> 3);
+  constexpr int GROUP_M = 4;
+  const int     per     = GROUP_M * tiles_n;
+  const int     group   = L / per;
+  const int     first   = group * GROUP_M;
+  const int     gm      = (tiles_m - first) < GROUP_M ? (tiles_m - first) : GROUP_M;
+  const int     in      = L - group * per;
+  tm                    = first + in % gm;
+  tn                    = in / gm;
+}
+
+template <int BM, int BN>
+struct Fp8Tile {
+  static constexpr int WAVES_M = BM / 64;
+  static constexpr int WAVES_N = BN / 128;
+  static constexpr int NW      = WAVES_M * WAVES_N;
+  static constexpr int NT      = NW * 64;
+  static constexpr int A_BYTES = BM * 128;
+  static constexpr int B_BYTES = BN * 128;
+  static constexpr int STAGE   = A_BYTES + B_BYTES;
+  static constexpr int A_LOADS = (BM / 8) / NW;
+  static constexpr int B_LOADS = (BN / 8) / NW;
+};
+
+template <int BM, int BN>
+__device__ __forceinline__ void fp8_issue_stage(char LLMMM_LDS* lds, const uint8_t* __restrict__ Ag,
+                                                const uint8_t* __restrict__ Bg, const int (&a_off)[Fp8Tile<BM, BN>::A_LOADS],
+                                                const int (&b_off)[Fp8Tile<BM, BN>::B_LOADS], int wave)
+{
+  typedef Fp8Tile<BM, BN> TC;
+#pragma unroll
+  for (int i = 0; i < TC::A_LOADS; ++i) load_lds_16B(Ag + a_off[i], lds + (wave + i * TC::NW) * 1024);
+#pragma unroll
+  for (int i = 0; i < TC::B_LOADS; ++i) load_lds_16B(Bg + b_off[i], lds + TC::A_BYTES + (wave + i * TC::NW) * 1024);
+}
+
+__device__ __forceinline__ i32x8 fp8_read_frag(const char LLMMM_LDS* tile, int rd)
+{
+  union {
+    i32x4 h[2];
+    i32x8 v;
+  } u;
+  u.h[0] = *(const i32x4 LLMMM_LDS*)(tile + rd);
+  u.h[1] = *(const i32x4 LLMMM_LDS*)(tile + (rd ^ 16));
+  return u.v;
+}
+
+// One 128-K slice of the wave's 64 x 128 sub-tile.  s[mf] = As[kb, row] * Bs[nb, kb].
+template <int BM, int BN>
+__device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, const int (&a_rd)[4], const int (&b_rd)[8],
+                                                  const float (&s)[4], f32x4 (&acc)[8][4])
+{
+  typedef Fp8Tile<BM, BN> TC;
+  const char LLMMM_LDS*   ldsA = lds;
+  const char LLMMM_LDS*   ldsB = lds + TC::A_BYTES;
+  i32x8                   a[4], b[2];
+  f32x4                   p[2][4];
+#pragma unroll
+  for (int mf = 0; mf < 4; ++mf) a[mf] = fp8_read_frag(ldsA, a_rd[mf]);
+  b[0] = fp8_read_frag(ldsB, b_rd[0]);
+#pragma unroll
+  for (int nf = 0; nf < 8; ++nf) {
+    const int cur = nf & 1;
+    if (nf + 1 < 8) b[cur ^ 1] = fp8_read_frag(ldsB, b_rd[nf + 1]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int mf = 0; mf < 4; ++mf) p[cur][mf] = mfma_fp8_k128(b[cur], a[mf]);
+    if (nf > 0) {
+#pragma unroll
+      for (int mf = 0; mf < 4; ++mf)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[nf - 1][mf][r] = __builtin_fmaf(p[cur ^ 1][mf][r], s[mf], acc[nf - 1][mf][r]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int mf = 0; mf < 4; ++mf)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[7][mf][r] = __builtin_fmaf(p[1][mf][r], s[mf], acc[7][mf][r]);
+}
+
+__device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float d)
+{
+  // v_cvt_pk_fp8_f32 rounds to nearest even but turns |x| > 464 into NaN: clamp first, which
+  // gives the saturate-to-finite behaviour of the reference's __nv_fp8_e4m3(float).
+  a     = __builtin_amdgcn_fmed3f(a, -448.f, 448.f);
+  b     = __builtin_amdgcn_fmed3f(b, -448.f, 448.f);
+  c     = __builtin_amdgcn_fmed3f(c, -448.f, 448.f);
+  d     = __builtin_amdgcn_fmed3f(d, -448.f, 448.f);
+  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  v     = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+  return (uint32_t)v;
+}
+
+template <int BM, int BN, int OUT>
+__global__ void __launch_bounds__((BM / 64) * (BN / 128) * 64)
+fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
+                const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int tiles_m,
+                int tiles_n)
+{
+  typedef Fp8Tile<BM, BN> TC;
+  __shared__ __attribute__((aligned(1024))) char lds0[TC::STAGE];
+  __shared__ __attribute__((aligned(1024))) char lds1[TC::STAGE];
+
+  const int tid  = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm   = wave % TC::WAVES_M;
+  const int wn   = wave / TC::WAVES_M;
+  int       tm, tn;
+  fp8_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int KB = K >> 7;
+
+  int a_off[TC::A_LOADS], b_off[TC::B_LOADS];
+#pragma unroll
+  for (int i = 0; i < TC::A_LOADS; ++i) {
+    const KMajorLane p = kmajor_lane<SWZ_ROWS16>(wave + i * TC::NW, lane);
+    a_off[i]           = p.row * K + p.chunk * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < TC::B_LOADS; ++i) {
+    const KMajorLane p = kmajor_lane<SWZ_ROWS16>(wave + i * TC::NW, lane);
+    b_off[i]           = p.row * K + p.chunk * 16;
+  }
+  const uint8_t* Ag = A + (size_t)m0 * K;
+  const uint8_t* Bg = Bt + (size_t)n0 * K;
+
+  // operand reads: lane = (g = lane/16, i = lane%16) takes row i of a 16-row fragment and the
+  // 32 bytes k = 32g .. 32g+31 (chunks 2g and 2g+1; the second one sits at offset ^ 16)
+  int       a_rd[4], b_rd[8];
+  const int g = lane >> 4;
+#pragma unroll
+  for (int mf = 0; mf < 4; ++mf) a_rd[mf] = kmajor_offset<SWZ_ROWS16>(wm * 64 + mf * 16 + (lane & 15), 2 * g);
+#pragma unroll
+  for (int nf = 0; nf < 8; ++nf) b_rd[nf] = kmajor_offset<SWZ_ROWS16>(wn * 128 + nf * 16 + (lane & 15), 2 * g);
+
+  f32x4 acc[8][4];
+#pragma unroll
+  for (int nf = 0; nf < 8; ++nf)
+#pragma unroll
+    for (int mf = 0; mf < 4; ++mf) acc[nf][mf] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // scales: As[kb*M + m] for the lane's 4 rows, Bs[(n/128)*KB + kb] for the wave's column group
+  const int    mrow = m0 + wm * 64 + (lane & 15);
+  const float* Asp  = As + mrow;
+  const float* Bsp  = Bs + (size_t)((n0 >> 7) + wn) * KB;
+  float        sa[4], sa_next[4], sb, sb_next;
+#pragma unroll
+  for (int mf = 0; mf < 4; ++mf) sa_next[mf] = Asp[mf * 16];
+  sb_next = Bsp[0];
+
+  char LLMMM_LDS* const s0 = (char LLMMM_LDS*)lds0;
+  char LLMMM_LDS* const s1 = (char LLMMM_LDS*)lds1;
+
+  fp8_issue_stage<BM, BN>(s0, Ag, Bg, a_off, b_off, wave);
+  for (int kb = 0; kb < KB; kb += 2) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int kc = kb + half;
+      if (kc < KB) {
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): this wave's LDS-direct loads have landed
+        __syncthreads();
+        float s[4];
+#pragma unroll
+        for (int mf = 0; mf < 4; ++mf) s[mf] = sa_next[mf] * sb_next;
+        if (kc + 1 < KB) {
+          fp8_issue_stage<BM, BN>(half ? s0 : s1, Ag + (size_t)(kc + 1) * 128, Bg + (size_t)(kc + 1) * 128, a_off, b_off, wave);
+#pragma unroll
+          for (int mf = 0; mf < 4; ++mf) sa_next[mf] = Asp[(size_t)(kc + 1) * M + mf * 16];
+          sb_next = Bsp[kc + 1];
+        }
+        fp8_compute_stage<BM, BN>(half ? s1 : s0, a_rd, b_rd, s, acc);
+      }
+    }
+  }
+  (void)sa;
+  (void)sb;
+
+  // ---- epilogue.  lane (g, i): row m = .. + mf*16 + i, columns n = nf*16 + 4g + r
+  const int ncol = n0 + wn * 128 + 4 * g;
+  if constexpr (OUT == OUT_F32) {
+    float* C = (float*)Cv;
+#pragma unroll
+    for (int mf = 0; mf < 4; ++mf)
+#pragma unroll
+      for (int nf = 0; nf < 8; ++nf) *(f32x4*)(C + (size_t)(mrow + mf * 16) * N + ncol + nf * 16) = acc[nf][mf];
+  }
+  else if constexpr (OUT == OUT_BF16) {
+    __bf16* C = (__bf16*)Cv;
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int mf = 0; mf < 4; ++mf)
+#pragma unroll
+      for (int nf = 0; nf < 8; ++nf) {
+        bf16x4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[nf][mf][r];
+        *(bf16x4*)(C + (size_t)(mrow + mf * 16) * N + ncol + nf * 16) = o;
+      }
+  }
+  else {
+    uint8_t* C = (uint8_t*)Cv;
+#pragma unroll
+    for (int mf = 0; mf < 4; ++mf) {
+      float amax = 0.f;
+#pragma unroll
+      for (int nf = 0; nf < 8; ++nf)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) amax = fmaxf(amax, __builtin_fabsf(acc[nf][mf][r]));
+      amax              = wave_xor_max(amax, 16);
+      amax              = wave_xor_max(amax, 32);
+      const float scale = amax / 448.f;
+      const float inv   = amax > 0.f ? 448.f / amax : 0.f;
+      uint8_t*    crow  = C + (size_t)(mrow + mf * 16) * N + ncol;
+#pragma unroll
+      for (int nf = 0; nf < 8; ++nf) {
+        const f32x4 v                   = acc[nf][mf];
+        *(uint32_t*)(crow + nf * 16) = pack_e4m3x4(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+      }
+      if (g == 0) Cs[(size_t)((n0 >> 7) + wn) * M + mrow + mf * 16] = scale;
+    }
+  }
+}
+
+// --------------------------------------------------------------------------------------------- host
+template <int BM, int BN, int OUT>
+static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N,
+                             int K, hipStream_t stream)
+{
+  typedef Fp8Tile<BM, BN> TC;
+  const int tiles_m = M / BM, tiles_n = N / BN;
+  hipLaunchKernelGGL((fp8_gemm_kernel<BM, BN, OUT>), dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As,
+                     (const uint8_t*)Bt, Bs, C, Cs, M, N, K, tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
+template <int OUT>
+static hipError_t dispatch_fp8(int tile, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
+                               int M, int N, int K, hipStream_t stream)
+{
+  switch (tile) {
+    case LLMMM_TILE_256x256: return launch_fp8<256, 256, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, stream);
+    case LLMMM_TILE_128x256: return launch_fp8<128, 256, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, stream);
+    case LLMMM_TILE_256x128: return launch_fp8<256, 128, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, stream);
+    case LLMMM_TILE_128x128: return launch_fp8<128, 128, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t fp8_gemm_launch(int out_kind, int tile, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
+                           float* Cs, int M, int N, int K, hipStream_t stream)
+{
+  switch (out_kind) {
+    case OUT_F32: return dispatch_fp8<OUT_F32>(tile, A, As, Bt, Bs, C, Cs, M, N, K, stream);
+    case OUT_BF16: return dispatch_fp8<OUT_BF16>(tile, A, As, Bt, Bs, C, Cs, M, N, K, stream);
+    case OUT_FP8Q: return dispatch_fp8<OUT_FP8Q>(tile, A, As, Bt, Bs, C, Cs, M, N, K, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace llmmm

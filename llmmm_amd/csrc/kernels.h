@@ -1,0 +1,28 @@
+// Internal interface between the C-ABI layer (capi.cpp) and the gfx950 kernel files.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+// Tile ids (LLMMM_TILE_*) and enum values are those of the public header.
+#include "../../include/llmmm.h"
+
+namespace llmmm {
+
+// dtype: 0 = fp16, 1 = bf16.  b_layout: 0 = B[K,N] row-major, 1 = Bt[N,K].
+hipError_t fp16_gemm_launch(int dtype, int b_layout, int tile, const void* A, const void* B, void* C, int M, int N, int K,
+                            hipStream_t stream);
+
+// out_kind: 0 = fp32, 1 = bf16, 2 = e4m3 codes + per-1x128 scales.
+hipError_t fp8_gemm_launch(int out_kind, int tile, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
+                           float* Cs, int M, int N, int K, hipStream_t stream);
+
+// M <= 64; S splits of K; partial [S][M][N] fp32 and counters [N/128] are only touched when S > 1.
+hipError_t fp8_skinny_launch(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
+                             int M, int N, int K, int S, float* partial, unsigned* counters, hipStream_t stream);
+
+hipError_t quant_fp8_launch(int quant_m, int transpose, const float* x, void* q, float* scale, int M, int N, hipStream_t stream);
+
+hipError_t fill_u32_launch(uint32_t* p, uint32_t value, size_t n, hipStream_t stream);
+
+}  // namespace llmmm

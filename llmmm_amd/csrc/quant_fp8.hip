@@ -1,0 +1,154 @@
+// Blockwise symmetric FP8 (OCP e4m3) quantiser for gfx950.
+//
+// Replaces fp8_blockwise_symmetric_quantization<QUANT_M, 128, SCALE_TRANSPOSE>
+// (reference: examples/005.fp8.mm.cu:439-563): per block amax -> s = amax / 448.f ->
+// q = e4m3(s ? x / s : 0) with an IEEE-correct fp32 division, round-to-nearest-even and
+// saturation to +-448; a block of zeros gives s = 0 and q = 0.  Scale layouts:
+//   QUANT_M == 1:   transposed s[(n/128)*M + m]      plain s[m*ceil(N/128) + n/128]
+//   QUANT_M == 128: transposed s[(n/128)*M + m/128]  plain s[(m/128)*ceil(N/128) + n/128]
+// (row stride M in both transposed forms, as written at :494 and :532).
+// HBM-bound: x is read once (4 B/element) and q written once (1 B/element); the 128x128 form
+// keeps its block in registers between the amax pass and the conversion.
+// Rows may be ragged (any M); N must be a multiple of 4 (float4 accesses, as in the reference).
+#include "device_common.hip.h"
+#include "kernels.h"
+
+namespace llmmm {
+
+__device__ __forceinline__ uint32_t q_pack_e4m3x4(float a, float b, float c, float d)
+{
+  a     = __builtin_amdgcn_fmed3f(a, -448.f, 448.f);
+  b     = __builtin_amdgcn_fmed3f(b, -448.f, 448.f);
+  c     = __builtin_amdgcn_fmed3f(c, -448.f, 448.f);
+  d     = __builtin_amdgcn_fmed3f(d, -448.f, 448.f);
+  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  v     = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+  return (uint32_t)v;
+}
+
+__device__ __forceinline__ float amax4(float m, f32x4 v)
+{
+  return fmaxf(fmaxf(m, fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1]))), fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
+}
+
+// 1 x 128 blocks.  Half a wavefront (32 lanes x float4) owns one block; a workgroup of 256
+// threads covers 8 consecutive rows of one 128-column group per step and strides over rows.
+template <bool TRANSPOSE>
+__global__ void __launch_bounds__(256) quant_1x128_kernel(const float* __restrict__ x, uint8_t* __restrict__ q,
+                                                          float* __restrict__ scale, int M, int N, int rows_per_wg)
+{
+  const int tid   = threadIdx.x;
+  const int sub   = tid >> 5;        // which of the 8 rows of a step
+  const int l32   = tid & 31;
+  const int nb    = blockIdx.x;      // 128-column group
+  const int n     = nb * 128 + l32 * 4;
+  const int nbn   = (N + 127) >> 7;
+  const int mbeg  = blockIdx.y * rows_per_wg;
+  const int mend  = min(M, mbeg + rows_per_wg);
+  const bool live = n < N;
+  for (int m = mbeg + sub; m < mend; m += 8) {
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    if (live) v = __builtin_nontemporal_load((const f32x4*)(x + (size_t)m * N + n));
+    float a = amax4(0.f, v);
+    a       = wave_xor_max(a, 1);
+    a       = wave_xor_max(a, 2);
+    a       = wave_xor_max(a, 4);
+    a       = wave_xor_max(a, 8);
+    a       = wave_xor_max(a, 16);
+    const float s = a / 448.f;
+    uint32_t    c = 0;
+    if (s != 0.f) c = q_pack_e4m3x4(v[0] / s, v[1] / s, v[2] / s, v[3] / s);
+    if (live) *(uint32_t*)(q + (size_t)m * N + n) = c;
+    if (l32 == 0) {
+      if (TRANSPOSE)
+        scale[(size_t)nb * M + m] = s;
+      else
+        scale[(size_t)m * nbn + nb] = s;
+    }
+  }
+}
+
+// 128 x 128 blocks: one workgroup of 256 threads per block, 16 float4 per thread in registers.
+template <bool TRANSPOSE>
+__global__ void __launch_bounds__(256) quant_128x128_kernel(const float* __restrict__ x, uint8_t* __restrict__ q,
+                                                            float* __restrict__ scale, int M, int N)
+{
+  __shared__ float wmax[4];
+  const int tid  = threadIdx.x;
+  const int l32  = tid & 31;
+  const int sub  = tid >> 5;
+  const int nb   = blockIdx.x;
+  const int mb   = blockIdx.y;
+  const int n    = nb * 128 + l32 * 4;
+  const int nbn  = (N + 127) >> 7;
+  const bool live = n < N;
+  f32x4     v[16];
+  float     a = 0.f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int m = mb * 128 + r * 8 + sub;
+    v[r]        = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (live && m < M) v[r] = __builtin_nontemporal_load((const f32x4*)(x + (size_t)m * N + n));
+    a = amax4(a, v[r]);
+  }
+  a = wave_xor_max(a, 1);
+  a = wave_xor_max(a, 2);
+  a = wave_xor_max(a, 4);
+  a = wave_xor_max(a, 8);
+  a = wave_xor_max(a, 16);
+  a = wave_xor_max(a, 32);
+  if ((tid & 63) == 0) wmax[tid >> 6] = a;
+  __syncthreads();
+  a             = fmaxf(fmaxf(wmax[0], wmax[1]), fmaxf(wmax[2], wmax[3]));
+  const float s = a / 448.f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int m = mb * 128 + r * 8 + sub;
+    uint32_t  c = 0;
+    if (s != 0.f) c = q_pack_e4m3x4(v[r][0] / s, v[r][1] / s, v[r][2] / s, v[r][3] / s);
+    if (live && m < M) *(uint32_t*)(q + (size_t)m * N + n) = c;
+  }
+  if (tid == 0) {
+    if (TRANSPOSE)
+      scale[(size_t)nb * M + mb] = s;
+    else
+      scale[(size_t)mb * nbn + nb] = s;
+  }
+}
+
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t value, size_t n)
+{
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = value;
+}
+
+hipError_t fill_u32_launch(uint32_t* p, uint32_t value, size_t n, hipStream_t stream)
+{
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p, value, n);
+  return hipGetLastError();
+}
+
+hipError_t quant_fp8_launch(int quant_m, int transpose, const float* x, void* q, float* scale, int M, int N, hipStream_t stream)
+{
+  const int nbn = (N + 127) / 128;
+  if (quant_m == 1) {
+    // enough workgroups to fill the chip, at least 8 rows each
+    int rows_per_wg = 64;
+    while (rows_per_wg > 8 && (long)nbn * ((M + rows_per_wg - 1) / rows_per_wg) < 2048) rows_per_wg >>= 1;
+    dim3 grid(nbn, (M + rows_per_wg - 1) / rows_per_wg);
+    if (transpose)
+      hipLaunchKernelGGL(quant_1x128_kernel<true>, grid, dim3(256), 0, stream, x, (uint8_t*)q, scale, M, N, rows_per_wg);
+    else
+      hipLaunchKernelGGL(quant_1x128_kernel<false>, grid, dim3(256), 0, stream, x, (uint8_t*)q, scale, M, N, rows_per_wg);
+  }
+  else {
+    dim3 grid(nbn, (M + 127) / 128);
+    if (transpose)
+      hipLaunchKernelGGL(quant_128x128_kernel<true>, grid, dim3(256), 0, stream, x, (uint8_t*)q, scale, M, N);
+    else
+      hipLaunchKernelGGL(quant_128x128_kernel<false>, grid, dim3(256), 0, stream, x, (uint8_t*)q, scale, M, N);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace llmmm

@@ -1,0 +1,165 @@
+"""Host entry points of the matrix-multiplication path, mirroring the reference's launchers.
+
+Same names, argument order and error behaviour as the reference's C++ functions
+(``LLMMM::fp16_mm`` src/mm/fp16/mm.h:9-10; the FP8 launchers examples/005.fp8.mm.cu:217-225,
+:547-549, :2467-2476), taking torch CUDA tensors where the reference takes raw device pointers.
+Everything goes through the C ABI of ``libllmmm.so``; torch only owns the memory and the stream.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import GemmCfg, check, lib
+
+_FP8_DTYPES = (torch.uint8, torch.float8_e4m3fn)
+
+
+def _stream(stream):
+    if stream is None:
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    if isinstance(stream, torch.cuda.Stream):
+        return ctypes.c_void_p(stream.cuda_stream)
+    return ctypes.c_void_p(int(stream))
+
+
+def _ptr(t, what, dtypes=None, numel=None):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise TypeError("%s must be a CUDA tensor" % what)
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % what)
+    if dtypes is not None and t.dtype not in dtypes:
+        raise RuntimeError("T is not supported.")
+    if numel is not None and t.numel() < numel:
+        raise ValueError("%s holds %d elements, %d needed" % (what, t.numel(), numel))
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _dtype_code(t):
+    if t.dtype == torch.float16:
+        return _lib.DTYPE_F16
+    if t.dtype == torch.bfloat16:
+        return _lib.DTYPE_BF16
+    raise RuntimeError("T is not supported.")  # src/mm/fp16/mm.cu:15-17
+
+
+# ------------------------------------------------------------------------------------- FP16 / BF16
+def fp16_mm(A, B, C, M, N, K, stream=None):
+    """``LLMMM::fp16_mm<T>(A, B, C, M, N, K, stream)`` (src/mm/fp16/mm.cu:6-42).
+
+    A [M,K], B [K,N], C [M,N] row-major, T = float16 or bfloat16, fp32 accumulation.
+    Raises RuntimeError("M or N or K are not aligned.") unless M % 256 == 0, N % 256 == 0 and
+    K % 16 == 0 (the reference's rule, mm.cu:19-21) and RuntimeError("T is not supported.")
+    for other element types.  Asynchronous on ``stream`` (default: torch's current stream)."""
+    code = _dtype_code(A)
+    if B.dtype != A.dtype or C.dtype != A.dtype:
+        raise RuntimeError("T is not supported.")
+    if not (M % 256 == 0 and N % 256 == 0 and K % 16 == 0):
+        raise RuntimeError("M or N or K are not aligned.")
+    check(lib.llmmm_fp16_gemm(code, _ptr(A, "A", numel=M * K), _ptr(B, "B", numel=K * N), _ptr(C, "C", numel=M * N), M, N, K,
+                              _lib.B_ROW_MAJOR, _stream(stream)))
+
+
+def fp16_gemm(A, B, C=None, b_transposed=False, tile=_lib.TILE_AUTO, stream=None):
+    """C = A @ B (or A @ Bt.T when ``b_transposed``) through ``llmmm_fp16_gemm_ex``.
+
+    The library's own (wider) shape rule applies: M, N multiples of 128, K of 16."""
+    code = _dtype_code(A)
+    M, K = A.shape
+    N = B.shape[0] if b_transposed else B.shape[1]
+    if (B.shape[1] if b_transposed else B.shape[0]) != K or B.dtype != A.dtype:
+        raise ValueError("shape or dtype mismatch between A and B")
+    if C is None:
+        C = torch.empty((M, N), dtype=A.dtype, device=A.device)
+    cfg = GemmCfg(tile, 0)
+    check(lib.llmmm_fp16_gemm_ex(code, _ptr(A, "A"), _ptr(B, "B"), _ptr(C, "C", (A.dtype,), M * N), M, N, K,
+                                 _lib.B_TRANSPOSED if b_transposed else _lib.B_ROW_MAJOR, ctypes.byref(cfg), _stream(stream)))
+    return C
+
+
+# ------------------------------------------------------------------------------------- FP8 quantiser
+def fp8_blockwise_symmetric_quantization(x, q, scale, M, N, quant_m, quant_n=128, scale_transpose=False, stream=None):
+    """``fp8_blockwise_symmetric_quantization<QUANT_M, QUANT_N, SCALE_TRANSPOSE>(x, q, scale, M, N, stream)``
+    (examples/005.fp8.mm.cu:547-563).  quant_m in {1, 128}, quant_n == 128 (its static_asserts)."""
+    if quant_m not in (1, 128) or quant_n != 128:
+        raise ValueError("QUANT_M must be 1 or 128 and QUANT_N 128")
+    kind = {(1, True): _lib.QUANT_1x128_T, (128, False): _lib.QUANT_128x128, (1, False): _lib.QUANT_1x128,
+            (128, True): _lib.QUANT_128x128_T}[(quant_m, bool(scale_transpose))]
+    nb = (N + 127) // 128
+    n_scale = nb * M if scale_transpose else ((M + quant_m - 1) // quant_m) * nb
+    check(lib.llmmm_quant_fp8(kind, _ptr(x, "x", (torch.float32,), M * N), _ptr(q, "q", _FP8_DTYPES, M * N),
+                              _ptr(scale, "scale", (torch.float32,), n_scale), M, N, _stream(stream)))
+
+
+def quantize_activation(x, stream=None):
+    """1x128 quantisation with transposed scales: returns (codes uint8 [M,K], scales [K/128... ceil, M])."""
+    M, K = x.shape
+    q = torch.empty((M, K), dtype=torch.uint8, device=x.device)
+    s = torch.empty(((K + 127) // 128, M), dtype=torch.float32, device=x.device)
+    fp8_blockwise_symmetric_quantization(x, q, s, M, K, 1, 128, True, stream)
+    return q, s
+
+
+def quantize_weight(wt, stream=None):
+    """128x128 quantisation of a transposed weight Wt [N,K]: (codes [N,K], scales [ceil(N/128), ceil(K/128)])."""
+    N, K = wt.shape
+    q = torch.empty((N, K), dtype=torch.uint8, device=wt.device)
+    s = torch.empty(((N + 127) // 128, (K + 127) // 128), dtype=torch.float32, device=wt.device)
+    fp8_blockwise_symmetric_quantization(wt, q, s, N, K, 128, 128, False, stream)
+    return q, s
+
+
+# ------------------------------------------------------------------------------------- FP8 GEMM
+def workspace_bytes(out_kind, M, N, K):
+    return int(lib.llmmm_fp8_gemm_workspace(out_kind, M, N, K))
+
+
+def make_workspace(out_kind, M, N, K, device="cuda", stream=None):
+    """Allocate and initialise a split-K workspace for this shape (None when none is needed)."""
+    n = workspace_bytes(out_kind, M, N, K)
+    if n == 0:
+        return None
+    ws = torch.empty(n, dtype=torch.uint8, device=device)
+    check(lib.llmmm_workspace_init(ctypes.c_void_p(ws.data_ptr()), n, _stream(stream)))
+    return ws
+
+
+def query_config(out_kind, M, N, K):
+    cfg = GemmCfg()
+    check(lib.llmmm_fp8_gemm_query(out_kind, M, N, K, ctypes.byref(cfg)))
+    return cfg.tile, cfg.split_k
+
+
+def _fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, workspace, tile, split_k, stream):
+    kb = K // 128 if K % 128 == 0 else 0
+    c_dtypes = {_lib.OUT_F32: (torch.float32,), _lib.OUT_BF16: (torch.bfloat16,), _lib.OUT_FP8Q: _FP8_DTYPES}[out_kind]
+    a_p = _ptr(A, "A", _FP8_DTYPES, M * K)
+    as_p = _ptr(As, "A_scale_transposed", (torch.float32,), kb * M)
+    b_p = _ptr(Bt, "B_transposed", _FP8_DTYPES, N * K)
+    bs_p = _ptr(Bs, "B_scale_transposed", (torch.float32,), ((N + 127) // 128) * kb)
+    c_p = _ptr(C, "C", c_dtypes, M * N)
+    cs_p = _ptr(Cs, "C_scale_transposed", (torch.float32,), ((N + 127) // 128) * M) if out_kind == _lib.OUT_FP8Q else None
+    ws_p, ws_n = (ctypes.c_void_p(workspace.data_ptr()), workspace.numel() * workspace.element_size()) if workspace is not None else (None, 0)
+    cfg = GemmCfg(tile, split_k)
+    check(lib.llmmm_fp8_gemm_ex(out_kind, a_p, as_p, b_p, bs_p, c_p, cs_p, M, N, K, ws_p, ws_n, ctypes.byref(cfg), _stream(stream)))
+
+
+def fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(A, A_scale_transposed, B_transposed, B_scale_transposed, C, M, N, K,
+                                                             stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0):
+    """examples/005.fp8.mm.cu:217-246.  C [M,N] float32."""
+    _fp8_gemm(_lib.OUT_F32, A, A_scale_transposed, B_transposed, B_scale_transposed, C, None, M, N, K, workspace, tile, split_k, stream)
+
+
+def fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(A, A_scale_transposed, B_transposed, B_scale_transposed, C, M, N, K,
+                                                             stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0):
+    """The fp32 variant's result rounded to bfloat16 (no reference kernel; same signature)."""
+    _fp8_gemm(_lib.OUT_BF16, A, A_scale_transposed, B_transposed, B_scale_transposed, C, None, M, N, K, workspace, tile, split_k, stream)
+
+
+def fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(A, A_scale_transposed, B_transposed, B_scale_transposed, C,
+                                                                     C_scale_transposed, M, N, K, stream=None, workspace=None,
+                                                                     tile=_lib.TILE_AUTO, split_k=0):
+    """examples/005.fp8.mm.cu:2467-2500 / examples/005.fp8.mm.opt.cu:468-508.  C e4m3 codes [M,N],
+    C_scale_transposed float32 [N/128, M]."""
+    _fp8_gemm(_lib.OUT_FP8Q, A, A_scale_transposed, B_transposed, B_scale_transposed, C, C_scale_transposed, M, N, K, workspace, tile,
+              split_k, stream)

@@ -1,0 +1,232 @@
+"""CPU oracle for the LLMMM matrix-multiplication path: numpy front-end of ``oracle.c``.
+
+TEST INFRASTRUCTURE ONLY.  Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline``
+leg of ``bench.py`` may import this package; the product library (``llmmm_amd``) never does.
+
+Every function restates a piece of the reference (file:line given at the C definition in
+``oracle.c``); what pins each of them is listed in the header of that file.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+
+def build(force=False):
+    """Compile ``oracle.c`` with gcc (OpenMP, no contraction, no fast-math)."""
+    src = os.path.join(_HERE, "oracle.c")
+    if force or not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liboracle.so"], stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = ctypes.CDLL(_LIB_PATH)
+    c = ctypes
+    f32p, u8p, u16p = c.POINTER(c.c_float), c.POINTER(c.c_uint8), c.POINTER(c.c_uint16)
+    sig = {
+        "oracle_num_threads": (c.c_int, []),
+        "oracle_set_num_threads": (None, [c.c_int]),
+        "oracle_f16_to_f32": (c.c_float, [c.c_uint16]),
+        "oracle_f32_to_f16": (c.c_uint16, [c.c_float]),
+        "oracle_bf16_to_f32": (c.c_float, [c.c_uint16]),
+        "oracle_f32_to_bf16": (c.c_uint16, [c.c_float]),
+        "oracle_e4m3_decode": (c.c_float, [c.c_uint8]),
+        "oracle_e4m3_encode": (c.c_uint8, [c.c_float]),
+        "oracle_kahan_gemm": (None, [f32p, f32p, f32p, c.c_int, c.c_int, c.c_int, c.c_int]),
+        "oracle_kahan_gemm_bt": (None, [f32p, f32p, f32p, c.c_int, c.c_int, c.c_int, c.c_int]),
+        "oracle_double_gemm": (None, [f32p, f32p, f32p, c.c_int, c.c_int, c.c_int]),
+        "oracle_quant_fp8": (None, [f32p, u8p, f32p, c.c_int, c.c_int, c.c_int, c.c_int]),
+        "oracle_dequant_fp8": (None, [u8p, f32p, f32p, c.c_int, c.c_int, c.c_int, c.c_int]),
+        "oracle_fp8_gemm": (c.c_int, [u8p, f32p, u8p, f32p, f32p, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int]),
+        "oracle_requant_c_1x128": (None, [f32p, u8p, f32p, c.c_int, c.c_int, c.c_int, c.c_int]),
+        "oracle_e4m3_encode_n": (None, [f32p, u8p, c.c_size_t]),
+        "oracle_e4m3_decode_n": (None, [u8p, f32p, c.c_size_t]),
+        "oracle_f32_to_f16_n": (None, [f32p, u16p, c.c_size_t]),
+        "oracle_f16_to_f32_n": (None, [u16p, f32p, c.c_size_t]),
+        "oracle_f32_to_bf16_n": (None, [f32p, u16p, c.c_size_t]),
+        "oracle_bf16_to_f32_n": (None, [u16p, f32p, c.c_size_t]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = res, args
+    return lib
+
+
+_lib = _load()
+
+
+def _p(a, ct):
+    return a.ctypes.data_as(ctypes.POINTER(ct))
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _u8(a):
+    a = np.ascontiguousarray(a)
+    assert a.dtype == np.uint8, a.dtype
+    return a
+
+
+def num_threads():
+    return int(_lib.oracle_num_threads())
+
+
+def set_num_threads(n):
+    _lib.oracle_set_num_threads(int(n))
+
+
+# ----------------------------------------------------------------------------- scalar formats
+def e4m3_decode(codes):
+    """uint8 e4m3 codes -> float32 (NaN for 0x7F / 0xFF)."""
+    q = _u8(codes)
+    out = np.empty(q.shape, np.float32)
+    _lib.oracle_e4m3_decode_n(_p(q, ctypes.c_uint8), _p(out, ctypes.c_float), q.size)
+    return out
+
+
+def e4m3_encode(x):
+    """float32 -> e4m3 codes, RNE, saturate-to-finite, NaN -> 0x7F."""
+    x = _f32(x)
+    out = np.empty(x.shape, np.uint8)
+    _lib.oracle_e4m3_encode_n(_p(x, ctypes.c_float), _p(out, ctypes.c_uint8), x.size)
+    return out
+
+
+def f32_to_f16_bits(x):
+    x = _f32(x)
+    out = np.empty(x.shape, np.uint16)
+    _lib.oracle_f32_to_f16_n(_p(x, ctypes.c_float), _p(out, ctypes.c_uint16), x.size)
+    return out
+
+
+def f16_bits_to_f32(h):
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    out = np.empty(h.shape, np.float32)
+    _lib.oracle_f16_to_f32_n(_p(h, ctypes.c_uint16), _p(out, ctypes.c_float), h.size)
+    return out
+
+
+def f32_to_bf16_bits(x):
+    x = _f32(x)
+    out = np.empty(x.shape, np.uint16)
+    _lib.oracle_f32_to_bf16_n(_p(x, ctypes.c_float), _p(out, ctypes.c_uint16), x.size)
+    return out
+
+
+def bf16_bits_to_f32(h):
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    out = np.empty(h.shape, np.float32)
+    _lib.oracle_bf16_to_f32_n(_p(h, ctypes.c_uint16), _p(out, ctypes.c_float), h.size)
+    return out
+
+
+def e4m3_code_index(codes):
+    """Monotone integer order of e4m3 values: index(a) < index(b) <=> value(a) < value(b).
+
+    +0 and -0 share index 0; NaN codes map to +-127 (outside the finite range +-126)."""
+    c = np.asarray(codes, dtype=np.uint8).astype(np.int32)
+    mag = c & 0x7F
+    return np.where(c & 0x80, -mag, mag)
+
+
+# ----------------------------------------------------------------------------- GEMM references
+def kahan_gemm(A, B, fused=True):
+    """fp32 Kahan-compensated C = A[M,K] @ B[K,N] (test/kahan.cu:16-26)."""
+    A, B = _f32(A), _f32(B)
+    M, K = A.shape
+    K2, N = B.shape
+    assert K == K2
+    C = np.empty((M, N), np.float32)
+    _lib.oracle_kahan_gemm(_p(A, ctypes.c_float), _p(B, ctypes.c_float), _p(C, ctypes.c_float), M, N, K, int(fused))
+    return C
+
+
+def kahan_gemm_bt(A, Bt, fused=True):
+    """Same arithmetic with B given as Bt[N,K]."""
+    A, Bt = _f32(A), _f32(Bt)
+    M, K = A.shape
+    N, K2 = Bt.shape
+    assert K == K2
+    C = np.empty((M, N), np.float32)
+    _lib.oracle_kahan_gemm_bt(_p(A, ctypes.c_float), _p(Bt, ctypes.c_float), _p(C, ctypes.c_float), M, N, K, int(fused))
+    return C
+
+
+def double_gemm(A, B):
+    """fp32 products accumulated in double (test/kahan.cu:48-55)."""
+    A, B = _f32(A), _f32(B)
+    M, K = A.shape
+    K2, N = B.shape
+    assert K == K2
+    C = np.empty((M, N), np.float32)
+    _lib.oracle_double_gemm(_p(A, ctypes.c_float), _p(B, ctypes.c_float), _p(C, ctypes.c_float), M, N, K)
+    return C
+
+
+# ----------------------------------------------------------------------------- FP8 path
+def scale_shape(M, N, quant_m, scale_transpose):
+    nb = (N + 127) // 128
+    mb = (M + quant_m - 1) // quant_m
+    if scale_transpose:
+        # the reference strides the transposed layout by M also for 128-row blocks
+        # (examples/005.fp8.mm.cu:532-533), so the buffer is [nb, M] with only M/128 used per row
+        return (nb, M)
+    return (mb, nb)
+
+
+def quant_fp8(x, quant_m, scale_transpose):
+    """examples/005.fp8.mm.cu:439-545.  Returns (codes uint8 [M,N], scales float32)."""
+    x = _f32(x)
+    M, N = x.shape
+    assert quant_m in (1, 128)
+    q = np.empty((M, N), np.uint8)
+    s = np.zeros(scale_shape(M, N, quant_m, scale_transpose), np.float32)
+    _lib.oracle_quant_fp8(_p(x, ctypes.c_float), _p(q, ctypes.c_uint8), _p(s, ctypes.c_float), M, N, quant_m,
+                          int(scale_transpose))
+    return q, s
+
+
+def dequant_fp8(q, s, quant_m, scale_transpose):
+    q = _u8(q)
+    s = _f32(s)
+    M, N = q.shape
+    x = np.empty((M, N), np.float32)
+    _lib.oracle_dequant_fp8(_p(q, ctypes.c_uint8), _p(s, ctypes.c_float), _p(x, ctypes.c_float), M, N, quant_m,
+                            int(scale_transpose))
+    return x
+
+
+def fp8_gemm(Aq, As, Bt, Bs, promote=128, assoc=1):
+    """Blockwise-scaled GEMM, fp32 result (examples/005.fp8.mm.cu:176-199 / :885-902).
+
+    Aq [M,K] codes, As [K/128,M], Bt [N,K] codes, Bs [ceil(N/128),K/128]."""
+    Aq, Bt, As, Bs = _u8(Aq), _u8(Bt), _f32(As), _f32(Bs)
+    M, K = Aq.shape
+    N, K2 = Bt.shape
+    assert K == K2 and As.shape == (K // 128, M) and Bs.shape == ((N + 127) // 128, K // 128), (As.shape, Bs.shape)
+    C = np.empty((M, N), np.float32)
+    rc = _lib.oracle_fp8_gemm(_p(Aq, ctypes.c_uint8), _p(As, ctypes.c_float), _p(Bt, ctypes.c_uint8),
+                              _p(Bs, ctypes.c_float), _p(C, ctypes.c_float), M, N, K, promote, assoc)
+    if rc:
+        raise RuntimeError("M or N or K are not aligned.")
+    return C
+
+
+def requant_c_1x128(C, reciprocal=True, zero_guard=True):
+    """Fused-epilogue arithmetic (examples/005.fp8.mm.opt.cu:401-462): (Cq [M,N], Cs [ceil(N/128), M])."""
+    C = _f32(C)
+    M, N = C.shape
+    Cq = np.empty((M, N), np.uint8)
+    Cs = np.empty(((N + 127) // 128, M), np.float32)
+    _lib.oracle_requant_c_1x128(_p(C, ctypes.c_float), _p(Cq, ctypes.c_uint8), _p(Cs, ctypes.c_float), M, N,
+                                int(reciprocal), int(zero_guard))
+    return Cq, Cs
