@@ -1,0 +1,262 @@
+#!/usr/bin/env python3
+"""Benchmark of the matrix-multiplication hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-shapes]
+
+A "step" is one GEMM launch through the C ABI (``libllmmm.so``) on inputs already resident in
+HBM.  The headline workload is the FP16 GEMM at M=N=K=4096 (A ~ N(0,1), B ~ N(0,0.02), seed 2,
+fp32 accumulation, fp16 output, one kernel, no split-K); ``value`` is its TFLOP/s
+(2*M*N*K / time).  One JSON line is printed, carrying as well
+  * ``roofline``: the dominant kernel against MI355X's published dense MFMA peak (or HBM peak
+    for the decode shapes), from HIP events recorded on the launch stream around the timed
+    region;
+  * ``cpu_baseline``: the CPU oracle (a port of the reference's Kahan GEMM, test/kahan.cu:16-26)
+    timed on this host's cores on a bounded sample of the same workload;
+  * ``shapes``: TFLOP/s (and GB/s for M <= 16) of the other BASELINE shapes, measured the same way.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "fp8": 5000.0}  # MI355X dense MFMA, published
+PEAK_HBM_GBS = 8000.0
+
+QWEN3_4B = {"qkv": (6144, 2560), "o": (2560, 4096), "gate_up": (19456, 2560), "down": (2560, 9728)}
+
+
+def _events_ms(fn, steps, warmup, graph=False):
+    """Average duration of one call of fn, HIP events on torch's current stream (the stream
+    every launch below is enqueued on).  With graph=True the `steps` launches are captured into
+    one HIP graph and replayed, so that microsecond kernels are timed back-to-back on the GPU
+    instead of at the pace of the Python launch loop."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    if graph:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(steps):
+                fn()
+        g.replay()  # untimed replay: graph upload
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+    else:
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_time(e1) / steps, wall_ms / steps
+
+
+def fp16_inputs(M, N, K, dtype=torch.float16, seed=2):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    A = torch.randn((M, K), generator=g, device="cuda", dtype=torch.float32).to(dtype)
+    B = (torch.randn((K, N), generator=g, device="cuda", dtype=torch.float32) * 0.02).to(dtype)
+    return A, B
+
+
+def fp8_inputs(M, N, K, seed=3, copies=1):
+    """Activations N(0,1) with 1% of the K channels x20, weights N(0,0.02); quantised on the GPU by
+    the library's own quantiser (1x128 for A, 128x128 for Bt).  `copies` distinct weight buffers."""
+    import llmmm_amd
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    A = torch.randn((M, K), generator=g, device="cuda", dtype=torch.float32)
+    nout = max(1, (K + 99) // 100)
+    cols = torch.randperm(K, generator=g, device="cuda")[:nout]
+    A[:, cols] *= 20.0
+    Aq, As = llmmm_amd.quantize_activation(A)
+    weights = []
+    for c in range(copies):
+        Wt = torch.randn((N, K), generator=g, device="cuda", dtype=torch.float32) * 0.02
+        weights.append(llmmm_amd.quantize_weight(Wt))
+        del Wt
+    return Aq, As, weights
+
+
+def bench_fp16(M, N, K, steps, warmup, dtype=torch.float16, b_transposed=False):
+    import llmmm_amd
+    A, B = fp16_inputs(M, N, K, dtype)
+    if b_transposed:
+        B = B.t().contiguous()
+    C = torch.empty((M, N), dtype=dtype, device="cuda")
+    ms, wall = _events_ms(lambda: llmmm_amd.fp16_gemm(A, B, C, b_transposed=b_transposed), steps, warmup)
+    flops = 2.0 * M * N * K
+    return {"ms": ms, "wall_ms": wall, "tflops": flops / ms * 1e-9, "bytes": 2.0 * (M * K + K * N + M * N)}, (A, B, C)
+
+
+def fp8_bytes(M, N, K, out):
+    b = M * K + N * K + 4.0 * (M * K / 128 + (N / 128) * (K / 128))
+    if out == "fp8q":
+        b += M * N + 4.0 * M * N / 128
+    elif out == "bf16":
+        b += 2.0 * M * N
+    else:
+        b += 4.0 * M * N
+    return b
+
+
+def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0):
+    """out in {"f32","bf16","fp8q"}.  With rotate_bytes > 0 the launches cycle through enough
+    distinct weight copies to exceed that many bytes, so weights stream from HBM, not from cache."""
+    import llmmm_amd
+    from llmmm_amd import _lib
+    copies = 1
+    if rotate_bytes:
+        copies = max(2, int(np.ceil(rotate_bytes / float(N * K))))
+    Aq, As, weights = fp8_inputs(M, N, K, copies=copies)
+    kind = {"f32": _lib.OUT_F32, "bf16": _lib.OUT_BF16, "fp8q": _lib.OUT_FP8Q}[out]
+    cdt = {"f32": torch.float32, "bf16": torch.bfloat16, "fp8q": torch.uint8}[out]
+    C = torch.empty((M, N), dtype=cdt, device="cuda")
+    Cs = torch.empty((N // 128, M), dtype=torch.float32, device="cuda")
+    ws = llmmm_amd.make_workspace(kind, M, N, K)
+    fns = {"f32": llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32,
+           "bf16": llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16}
+    state = {"i": 0}
+
+    def step():
+        Bq, Bs = weights[state["i"] % copies]
+        state["i"] += 1
+        if out == "fp8q":
+            llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(Aq, As, Bq, Bs, C, Cs, M, N, K, workspace=ws)
+        else:
+            fns[out](Aq, As, Bq, Bs, C, M, N, K, workspace=ws)
+
+    ms, wall = _events_ms(step, steps, warmup, graph=(M <= 128))
+    flops = 2.0 * M * N * K
+    nbytes = fp8_bytes(M, N, K, out)
+    tile, split = llmmm_amd.query_config(kind, M, N, K)
+    return {"ms": ms, "wall_ms": wall, "tflops": flops / ms * 1e-9, "gbs": nbytes / ms * 1e-6, "bytes": nbytes, "tile": tile,
+            "split_k": split, "weight_copies": copies}
+
+
+def cpu_baseline_fp16(M, N, K, rows):
+    """Oracle Kahan GEMM on the first `rows` rows of the headline workload, all host threads."""
+    import oracle
+    rng = np.random.default_rng(2)
+    A = rng.standard_normal((rows, K), dtype=np.float32).astype(np.float16).astype(np.float32)
+    B = (rng.standard_normal((K, N), dtype=np.float32) * 0.02).astype(np.float16).astype(np.float32)
+    oracle.kahan_gemm(A[:8], B)  # warm the thread pool
+    t0 = time.perf_counter()
+    oracle.kahan_gemm(A, B)
+    dt = time.perf_counter() - t0
+    return {"value": 2.0 * rows * N * K / dt * 1e-12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": "oracle Kahan fp32 GEMM (port of test/kahan.cu:16-26) on the first %d of %d rows of the same "
+                      "M=N=K=4096 fp16 workload, %.1f s" % (rows, M, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="fp16_gemm_4096",
+                    help="fp16_gemm_4096 (headline) | fp8_gemm_fused_4096 | fp8_gemm_bf16_4096 | bf16_gemm_4096 | "
+                         "decode_<qkv|o|gate_up|down>_m<M>")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table")
+    ap.add_argument("--cpu-rows", type=int, default=2048)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every box has one GPU); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    import llmmm_amd  # noqa: F401  raises if libllmmm.so is missing
+
+    w = args.workload
+    M = N = K = 4096
+    if w in ("fp16_gemm_4096", "bf16_gemm_4096"):
+        dt = torch.float16 if w.startswith("fp16") else torch.bfloat16
+        r, _ = bench_fp16(M, N, K, args.steps, args.warmup, dt)
+        dtype, peak = ("f16" if dt == torch.float16 else "bf16"), PEAK_TFLOPS["f16"]
+        roof = {"bound": "mfma", "achieved": r["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": r["tflops"] / peak, "traffic": None,
+                "kernel": "fp16_gemm_kernel<%s,256,256,row-major B>" % dtype}
+        value, unit = r["tflops"], "TFLOP/s"
+        cfg = {"workload": "FP16 GEMM M=N=K=4096 (BASELINE configs[1]), A~N(0,1) B~N(0,0.02) seed 2, fp32 accumulate, %s out, "
+                           "single kernel, no split-K" % dtype, "M": M, "N": N, "K": K}
+    elif w in ("fp8_gemm_fused_4096", "fp8_gemm_bf16_4096"):
+        out = "fp8q" if "fused" in w else "bf16"
+        r = bench_fp8(M, N, K, out, args.steps, args.warmup)
+        dtype, peak = "fp8", PEAK_TFLOPS["fp8"]
+        roof = {"bound": "mfma", "achieved": r["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": r["tflops"] / peak, "traffic": None,
+                "kernel": "fp8_gemm_kernel<256,256,%s>" % out}
+        value, unit = r["tflops"], "TFLOP/s"
+        cfg = {"workload": "FP8 e4m3 blockwise GEMM M=N=K=4096 (A 1x128, B 128x128 scales), output %s" % out, "M": M, "N": N, "K": K}
+    elif w.startswith("decode_"):
+        import re
+        mo = re.fullmatch(r"decode_(qkv|o|gate_up|down)_m(\d+)", w)
+        if not mo:
+            print("unknown workload", w, file=sys.stderr)
+            sys.exit(2)
+        name, M = mo.group(1), int(mo.group(2))
+        N, K = QWEN3_4B[name]
+        r = bench_fp8(M, N, K, "fp8q", args.steps, args.warmup, rotate_bytes=768 << 20)
+        dtype = "fp8"
+        roof = {"bound": "hbm", "achieved": r["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": r["gbs"] / PEAK_HBM_GBS, "traffic": None,
+                "kernel": "fp8_skinny_kernel split_k=%d" % r["split_k"]}
+        value, unit = r["gbs"], "GB/s"
+        cfg = {"workload": "Qwen3-4B %s projection, FP8 blockwise GEMM + fused C quant, M=%d N=%d K=%d, weights rotated over %d "
+                           "copies" % (name, M, N, K, r["weight_copies"]), "M": M, "N": N, "K": K}
+    else:
+        print("unknown workload", w, file=sys.stderr)
+        sys.exit(2)
+
+    line = {
+        "metric": "TFLOPS (% of MI355X FP8/FP16 MFMA peak) at 4096^3; HBM GB/s at M<=16 decode",
+        "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms"],
+        "wall_ms_per_step": r["wall_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
+        "data": "synthetic", "config": cfg, "roofline": roof,
+    }
+
+    if not args.no_shapes:
+        shapes = []
+        s2, w2 = max(10, args.steps // 2), max(3, args.warmup // 2)
+        if w != "fp16_gemm_4096":
+            x, _ = bench_fp16(4096, 4096, 4096, s2, w2)
+            shapes.append({"name": "fp16_gemm_4096", "ms": x["ms"], "tflops": x["tflops"], "frac_of_fp16_peak": x["tflops"] / PEAK_TFLOPS["f16"]})
+        x, _ = bench_fp16(4096, 4096, 4096, s2, w2, torch.bfloat16)
+        shapes.append({"name": "bf16_gemm_4096", "ms": x["ms"], "tflops": x["tflops"], "frac_of_fp16_peak": x["tflops"] / PEAK_TFLOPS["f16"]})
+        x, _ = bench_fp16(1024, 1024, 1024, s2, w2)
+        shapes.append({"name": "fp16_gemm_1024", "ms": x["ms"], "tflops": x["tflops"], "frac_of_fp16_peak": x["tflops"] / PEAK_TFLOPS["f16"]})
+        x, _ = bench_fp16(1024, 1024, 1024, s2, w2, b_transposed=True)
+        shapes.append({"name": "fp16_gemm_1024_bt", "ms": x["ms"], "tflops": x["tflops"], "frac_of_fp16_peak": x["tflops"] / PEAK_TFLOPS["f16"]})
+        for out in ("bf16", "fp8q"):
+            x = bench_fp8(4096, 4096, 4096, out, s2, w2)
+            shapes.append({"name": "fp8_gemm_4096_" + out, "ms": x["ms"], "tflops": x["tflops"], "frac_of_fp8_peak": x["tflops"] / PEAK_TFLOPS["fp8"]})
+        for name, (n, k) in QWEN3_4B.items():
+            for m in (1, 16, 128, 2048):
+                x = bench_fp8(m, n, k, "fp8q", s2 * 2 if m <= 16 else s2, w2, rotate_bytes=(768 << 20) if m <= 128 else 0)
+                e = {"name": "qwen3_4b_%s_m%d" % (name, m), "M": m, "N": n, "K": k, "us": x["ms"] * 1e3, "tflops": x["tflops"],
+                     "frac_of_fp8_peak": x["tflops"] / PEAK_TFLOPS["fp8"], "tile": x["tile"], "split_k": x["split_k"]}
+                if m <= 128:
+                    e.update({"hbm_gbs": x["gbs"], "frac_of_hbm_peak": x["gbs"] / PEAK_HBM_GBS, "weight_copies": x["weight_copies"]})
+                shapes.append(e)
+                torch.cuda.empty_cache()
+        line["shapes"] = shapes
+
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline_fp16(4096, 4096, 4096, args.cpu_rows)
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

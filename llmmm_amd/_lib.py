@@ -6,6 +6,11 @@ this module raises, so nothing can silently run on another path.
 import ctypes
 import os
 
+# torch must be loaded first: it brings its own libamdhip64.so (soname libamdhip64.so.7) and
+# libllmmm.so then binds to that already-loaded runtime.  Loaded the other way round the process
+# ends up with two HIP runtimes, and launches on torch's streams from the second one fail.
+import torch  # noqa: F401
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libllmmm.so")
 

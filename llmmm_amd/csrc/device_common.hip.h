@@ -21,54 +21,53 @@ typedef int i32x8 __attribute__((ext_vector_type(8)));
 #define LLMMM_GLOBAL __attribute__((address_space(1)))
 
 // ---------------------------------------------------------------------------------------------
-// K-major operand tiles.  A tile is R rows, each row holding 128 bytes of the K extent (64 fp16
-// or 128 fp8 values) as eight 16-byte chunks.  Row r / chunk c lives at
-//     phys_row(r) * 128 + ((c ^ swz(r)) << 4).
+// K-major operand tiles in LDS.  A tile row holds ROW bytes of the K extent as 16-byte chunks;
+// row r / chunk c lives at  phys_row(r) * ROW + ((c ^ swz(r)) << 4).
 // ds_read_b128 serves a wavefront in four passes of 16 lanes -- {0-3,12-15,20-23,24-27},
 // {4-11,16-19,28-31} and the same two sets + 32 (measured on gfx950) -- and a pass is
 // conflict-free when its 16 lanes touch 16 different 16-byte slots of the 256-byte bank row.
-// Two placements are used, each matched to the lane -> (row, chunk) pattern of one MFMA shape:
-//   SWZ_ROWS32: lanes 0-31 read 32 consecutive rows at one chunk, lanes 32-63 another chunk
-//               (32x32x16 f16/bf16 operands).  Rows of a pair are swapped when bit 3 is set
-//               and the chunk is XOR-ed with row bits 1..3 and 4..6.
-//   SWZ_ROWS16: lanes 16g..16g+15 read 16 consecutive rows at chunk 2g (+1)
-//               (16x16x128 fp8 operands).  The chunk is XOR-ed with row bits 1..3 and, for
-//               rows 4..11 of every 16, with 2, which cancels the chunk difference between
-//               the two halves of a pass.
+// Each placement is matched to the lane -> (row, chunk) pattern of one MFMA operand shape:
+//   SWZ_ROW64:  64-byte rows (32 fp16).  Lanes 0-31 read 32 consecutive rows at one chunk,
+//               lanes 32-63 at another (32x32x16 f16/bf16 operands).  Four consecutive rows
+//               fill a bank row; the chunk is XOR-ed with row bits 2..3, inverted when bit 4
+//               is set, which separates the four row quads of a pass.
+//   SWZ_ROWS16: 128-byte rows (128 fp8).  Lanes 16g..16g+15 read 16 consecutive rows at chunk
+//               2g (+1) (16x16x128 fp8 operands).  The chunk is XOR-ed with row bits 1..3 and,
+//               for rows 4..11 of every 16, with 2, which cancels the chunk difference
+//               between the two halves of a pass.
 // ---------------------------------------------------------------------------------------------
-enum { SWZ_ROWS32 = 0, SWZ_ROWS16 = 1 };
+enum { SWZ_ROW64 = 0, SWZ_ROWS16 = 1 };
 
 template <int SWZ>
-__device__ __forceinline__ int kmajor_phys_row(int r)
-{
-  return SWZ == SWZ_ROWS32 ? (r ^ ((r >> 3) & 1)) : r;
-}
+struct KMajor {
+  static constexpr int ROW    = SWZ == SWZ_ROW64 ? 64 : 128;  // bytes per tile row
+  static constexpr int CHUNKS = ROW / 16;
+  static constexpr int ROWS_PER_KB = 1024 / ROW;              // tile rows covered by one 1 KB load
+};
+
 template <int SWZ>
 __device__ __forceinline__ int kmajor_swz(int r)
 {
-  return SWZ == SWZ_ROWS32 ? (((r >> 1) ^ (r >> 4)) & 7) : (((r >> 1) & 7) ^ ((((r >> 2) ^ (r >> 3)) & 1) << 1));
+  return SWZ == SWZ_ROW64 ? (((r >> 2) & 3) ^ (((r >> 4) & 1) * 3)) : (((r >> 1) & 7) ^ ((((r >> 2) ^ (r >> 3)) & 1) << 1));
 }
 template <int SWZ>
 __device__ __forceinline__ int kmajor_offset(int r, int c)
 {
-  return kmajor_phys_row<SWZ>(r) * 128 + ((c ^ kmajor_swz<SWZ>(r)) << 4);
+  return r * KMajor<SWZ>::ROW + ((c ^ kmajor_swz<SWZ>(r)) << 4);
 }
 
-// One wave copies eight tile rows (1024 bytes of LDS) with a single LDS-direct load: lane l
-// owns the 16 bytes at lds_group + 16*l, and fetches the logical (row, chunk) that the swizzle
-// places there.
+// One wave copies 1024 bytes of a tile with a single LDS-direct load: lane l owns the 16 bytes
+// at lds_group + 16*l, and fetches the logical (row, chunk) that the swizzle places there.
 struct KMajorLane {
   int row;    // logical tile row this lane fetches
-  int chunk;  // logical 16-byte chunk within the 128-byte row
+  int chunk;  // logical 16-byte chunk within the row
 };
 template <int SWZ>
 __device__ __forceinline__ KMajorLane kmajor_lane(int group, int lane)
 {
-  const int  prow = group * 8 + (lane >> 3);
-  const int  row  = kmajor_phys_row<SWZ>(prow);  // both placements are involutions on the row index
   KMajorLane p;
-  p.row   = row;
-  p.chunk = (lane & 7) ^ kmajor_swz<SWZ>(row);
+  p.row   = group * KMajor<SWZ>::ROWS_PER_KB + lane / KMajor<SWZ>::CHUNKS;
+  p.chunk = (lane % KMajor<SWZ>::CHUNKS) ^ kmajor_swz<SWZ>(p.row);
   return p;
 }
 
@@ -77,6 +76,33 @@ __device__ __forceinline__ KMajorLane kmajor_lane(int group, int lane)
 __device__ __forceinline__ void load_lds_16B(const void* gptr, void LLMMM_LDS* lds_base)
 {
   __builtin_amdgcn_global_load_lds((const void LLMMM_GLOBAL*)gptr, lds_base, 16, 0, 0);
+}
+
+// s_waitcnt vmcnt(N) lgkmcnt(0): at most N of this wave's vector-memory loads still in flight,
+// every LDS access done.  simm16 = vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+  static_assert(N >= 0 && N < 64, "vmcnt out of range");
+  __builtin_amdgcn_s_waitcnt((N & 15) | 0x70 | ((N >> 4) << 14));
+}
+
+// Logical tile id -> (tm, tn).  Hardware hands consecutive workgroup ids to the 8 XCDs in turn,
+// so ids congruent mod 8 share an L2: give each XCD a contiguous run of the grouped order
+// (GROUP_M tile rows swept along n), whose members reuse the same few A and B panels.
+__device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, int& tm, int& tn)
+{
+  const int tiles = tiles_m * tiles_n;
+  int       L     = wg;
+  if ((tiles & 7) == 0) L = (wg & 7) * (tiles >> 3) + (wg >> 3);
+  constexpr int GROUP_M = 4;
+  const int     per     = GROUP_M * tiles_n;
+  const int     group   = L / per;
+  const int     first   = group * GROUP_M;
+  const int     gm      = (tiles_m - first) < GROUP_M ? (tiles_m - first) : GROUP_M;
+  const int     in      = L - group * per;
+  tm                    = first + in % gm;
+  tn                    = in / gm;
 }
 
 __device__ __forceinline__ float wave_xor_max(float v, int mask)

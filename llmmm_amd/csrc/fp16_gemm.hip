@@ -8,11 +8,16 @@
 //  * one workgroup computes a BM x BN tile, one wavefront a 64(m) x 128(n) sub-tile built from
 //    v_mfma_f32_32x32x16_{f16,bf16}; the MFMA is issued with B as the row operand and A as the
 //    column operand so that each lane ends up with 4 consecutive n of one row m (packed stores);
-//  * K advances 64 elements (128 bytes per tile row) per stage; two LDS stages are filled by
-//    LDS-direct global loads (no staging registers, no ds_write) while the other one is consumed;
-//  * A (and Bt) tiles are K-major and read with ds_read_b128 through the XOR swizzle of
-//    device_common.hip.h; a row-major B tile is kept as [k][n] and read with the transposing
-//    ds_read_b64_tr_b16, its 64-byte column chunks XOR-ed with k&3;
+//  * K advances 32 elements per stage (64 bytes per tile row, (BM+BN)*64 bytes of LDS) and four
+//    stages form a ring that LDS-direct global loads fill three stages ahead of the MFMAs
+//    (no staging registers, no ds_write);
+//  * the single workgroup barrier of a stage sits between its two 16-wide k-steps: by then
+//    every wave has pulled the stage's operands into registers, so the barrier both frees the
+//    stage's buffer for the load of stage +4 and publishes stage +1, whose first fragments are
+//    fetched right behind it -- no wave ever waits on an LDS read it has just issued;
+//  * A (and Bt) tiles are K-major and read with ds_read_b128 through the SWZ_ROW64 placement;
+//    a row-major B tile is kept as [k][n] and read with the transposing ds_read_b64_tr_b16,
+//    its 64-byte column chunks XOR-ed with k&3;
 //  * workgroup ids are remapped so that the tiles resident on one XCD share A/B panels in its L2.
 #include "device_common.hip.h"
 #include "kernels.h"
@@ -32,87 +37,82 @@ struct Mfma16<__bf16> {
   static __device__ __forceinline__ f32x16 run(vec x, vec y, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(x, y, c, 0, 0, 0); }
 };
 
-// Logical tile id -> (tm, tn).  Hardware hands consecutive workgroup ids to the 8 XCDs in turn,
-// so ids congruent mod 8 share an L2: give each XCD a contiguous run of the grouped order
-// (GROUP_M tile rows swept along n), whose members reuse the same few A and B panels.
-__device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, int& tm, int& tn)
-{
-  const int tiles = tiles_m * tiles_n;
-  int       L     = wg;
-  if ((tiles & 7) == 0) L = (wg & 7) * (tiles >> 3) + (wg >> 3);
-  constexpr int GROUP_M = 4;
-  const int     per     = GROUP_M * tiles_n;
-  const int     group   = L / per;
-  const int     first   = group * GROUP_M;
-  const int     gm      = (tiles_m - first) < GROUP_M ? (tiles_m - first) : GROUP_M;
-  const int     in      = L - group * per;
-  tm                    = first + in % gm;
-  tn                    = in / gm;
-}
-
 template <typename T, int BM, int BN, bool B_NK>
 struct Fp16Tile {
   static constexpr int WAVES_M = BM / 64;
   static constexpr int WAVES_N = BN / 128;
   static constexpr int NW      = WAVES_M * WAVES_N;
   static constexpr int NT      = NW * 64;
-  static constexpr int BK      = 64;             // elements of K per stage
-  static constexpr int A_BYTES = BM * 128;       // K-major, 128 bytes per row
-  static constexpr int B_BYTES = BN * 128;       // either layout: 64 x BN x 2 bytes
-  static constexpr int B_ROW   = BN * 2;         // row pitch of the [k][n] layout
+  static constexpr int BK      = 32;              // elements of K per stage
+  static constexpr int A_BYTES = BM * 64;         // K-major, 64 bytes per row
+  static constexpr int B_BYTES = BN * 64;         // either layout: 32 x BN x 2 bytes
+  static constexpr int B_ROW   = BN * 2;          // row pitch of the [k][n] layout
   static constexpr int STAGE   = A_BYTES + B_BYTES;
-  static constexpr int A_LOADS = (BM / 8) / NW;  // 1024-byte groups per wave
-  static constexpr int B_LOADS = (B_BYTES / 1024) / NW;
+  static constexpr int A_LOADS = (BM / 16) / NW;  // 1024-byte groups per wave
+  static constexpr int B_LOADS = (BN / 16) / NW;
+  static constexpr int LOADS   = A_LOADS + B_LOADS;
+  // wave-uniform step between two loads of a wave
+  static constexpr int ROWS_PER_LOAD    = 16 * NW;        // K-major tiles: tile rows
+  static constexpr int B_KROWS_PER_GRP  = 1024 / B_ROW;   // [k][n] tile: k rows per 1 KB group
+  static constexpr int B_KROWS_PER_LOAD = B_KROWS_PER_GRP * NW;
 };
 
 // Issue the LDS-direct loads of one stage.  `kleft` = K - k0 (elements still to go); a stage
 // whose K range is cut short zero-fills the missing part so that the MFMAs need no masking.
-template <typename T, int BM, int BN, bool B_NK>
+// All loads of a wave share one per-lane offset: they differ by a wave-uniform row (or k) step
+// that the swizzles do not see.
+template <typename T, int BM, int BN, bool B_NK, bool KTAIL>
 __device__ __forceinline__ void fp16_issue_stage(char LLMMM_LDS* lds, const T* __restrict__ Ag, const T* __restrict__ Bg,
-                                                 const int (&a_off)[Fp16Tile<T, BM, BN, B_NK>::A_LOADS],
-                                                 const int (&a_chunk)[Fp16Tile<T, BM, BN, B_NK>::A_LOADS],
-                                                 const int (&b_off)[Fp16Tile<T, BM, BN, B_NK>::B_LOADS],
-                                                 const int (&b_kc)[Fp16Tile<T, BM, BN, B_NK>::B_LOADS], int wave, int lane,
-                                                 int kleft)
+                                                 unsigned a_off, int a_k, unsigned b_off, int b_k, int K, int N, int wave,
+                                                 int lane, int kleft)
 {
   typedef Fp16Tile<T, BM, BN, B_NK> TC;
-  const bool full = kleft >= TC::BK;
+  // without a K tail (K % 32 == 0) the loads are unconditional: straight-line code keeps the
+  // compiler's wait-count bookkeeping exact
+  const bool full = !KTAIL || kleft >= TC::BK;
 #pragma unroll
   for (int i = 0; i < TC::A_LOADS; ++i) {
-    const int         g   = wave + i * TC::NW;
-    char LLMMM_LDS*   dst = lds + g * 1024;
-    if (full || a_chunk[i] * 8 < kleft)
-      load_lds_16B(Ag + a_off[i], dst);
+    char LLMMM_LDS* dst = lds + (wave + i * TC::NW) * 1024;
+    if (full || a_k < kleft)
+      load_lds_16B(Ag + (size_t)(TC::ROWS_PER_LOAD * i) * K + a_off, dst);
     else
       *(i32x4 LLMMM_LDS*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
   }
   char LLMMM_LDS* ldsB = lds + TC::A_BYTES;
 #pragma unroll
   for (int i = 0; i < TC::B_LOADS; ++i) {
-    const int       g   = wave + i * TC::NW;
-    char LLMMM_LDS* dst = ldsB + g * 1024;
-    // b_kc: K-major layout -> first k of the lane's chunk; [k][n] layout -> the lane's k row
-    if (full || b_kc[i] < kleft)
-      load_lds_16B(Bg + b_off[i], dst);
-    else
-      *(i32x4 LLMMM_LDS*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
+    char LLMMM_LDS* dst = ldsB + (wave + i * TC::NW) * 1024;
+    if constexpr (B_NK) {
+      if (full || b_k < kleft)
+        load_lds_16B(Bg + (size_t)(TC::ROWS_PER_LOAD * i) * K + b_off, dst);
+      else
+        *(i32x4 LLMMM_LDS*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
+    }
+    else {
+      if (full || b_k + TC::B_KROWS_PER_LOAD * i < kleft)
+        load_lds_16B(Bg + (size_t)(TC::B_KROWS_PER_LOAD * i) * N + b_off, dst);
+      else
+        *(i32x4 LLMMM_LDS*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
+    }
   }
 }
 
-// Operand fragments of one 16-wide k-step: a[mf] = 32 rows of A, b[nf] = 32 rows of B^T.
+// Operand fragments of one 16-wide k-step (ks = 0 or 1 inside a stage): a[mf] = 32 rows of A,
+// b[nf] = 32 rows of B^T.
 template <typename T, int BM, int BN, bool B_NK>
-__device__ __forceinline__ void fp16_read_frags(const char LLMMM_LDS* ldsA, const char LLMMM_LDS* ldsB, const int (&a_rd)[2],
-                                                const int (&b_rd)[4], int ks, typename Mfma16<T>::vec (&a)[2],
-                                                typename Mfma16<T>::vec (&b)[4])
+__device__ __forceinline__ void fp16_read_frags(const char LLMMM_LDS* lds, int a_rd, const int (&b_rd)[4], int ks,
+                                                typename Mfma16<T>::vec (&a)[2], typename Mfma16<T>::vec (&b)[4])
 {
   typedef Fp16Tile<T, BM, BN, B_NK> TC;
   typedef typename Mfma16<T>::vec   vec;
+  const char LLMMM_LDS*             ldsA = lds;
+  const char LLMMM_LDS*             ldsB = lds + TC::A_BYTES;
 #pragma unroll
-  for (int mf = 0; mf < 2; ++mf) a[mf] = *(const vec LLMMM_LDS*)(ldsA + (a_rd[mf] ^ (ks << 5)));
+  for (int mf = 0; mf < 2; ++mf) a[mf] = *(const vec LLMMM_LDS*)(ldsA + (a_rd ^ (ks << 5)) + mf * 2048);
 #pragma unroll
   for (int nf = 0; nf < 4; ++nf) {
     if constexpr (B_NK) {
-      b[nf] = *(const vec LLMMM_LDS*)(ldsB + (b_rd[nf] ^ (ks << 5)));
+      b[nf] = *(const vec LLMMM_LDS*)(ldsB + (b_rd[0] ^ (ks << 5)) + nf * 2048);
     }
     else {
       union {
@@ -126,37 +126,29 @@ __device__ __forceinline__ void fp16_read_frags(const char LLMMM_LDS* ldsA, cons
   }
 }
 
-// One stage = four k-steps; the fragments of step ks+1 are fetched while step ks multiplies.
-template <typename T, int BM, int BN, bool B_NK>
-__device__ __forceinline__ void fp16_compute_stage(const char LLMMM_LDS* lds, const int (&a_rd)[2], const int (&b_rd)[4],
-                                                   f32x16 (&acc)[4][2])
+// Half of a k-step: the 4 MFMAs of fragments nf = 2h, 2h+1.
+template <typename T>
+__device__ __forceinline__ void fp16_mfma_half(int h, const typename Mfma16<T>::vec (&a)[2], const typename Mfma16<T>::vec (&b)[4],
+                                               f32x16 (&acc)[4][2])
 {
-  typedef Fp16Tile<T, BM, BN, B_NK> TC;
-  typedef typename Mfma16<T>::vec   vec;
-  const char LLMMM_LDS*             ldsA = lds;
-  const char LLMMM_LDS*             ldsB = lds + TC::A_BYTES;
-  vec                               a[2][2], b[2][4];
-  fp16_read_frags<T, BM, BN, B_NK>(ldsA, ldsB, a_rd, b_rd, 0, a[0], b[0]);
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    const int cur = ks & 1;
-    if (ks + 1 < 4) fp16_read_frags<T, BM, BN, B_NK>(ldsA, ldsB, a_rd, b_rd, ks + 1, a[cur ^ 1], b[cur ^ 1]);
-    __builtin_amdgcn_sched_barrier(0);  // all reads of step ks+1 are in flight before step ks multiplies
+  for (int nf = 2 * h; nf < 2 * h + 2; ++nf)
 #pragma unroll
-    for (int nf = 0; nf < 4; ++nf)
-#pragma unroll
-      for (int mf = 0; mf < 2; ++mf) acc[nf][mf] = Mfma16<T>::run(b[cur][nf], a[cur][mf], acc[nf][mf]);
-    __builtin_amdgcn_sched_barrier(0);
-  }
+    for (int mf = 0; mf < 2; ++mf) acc[nf][mf] = Mfma16<T>::run(b[nf], a[mf], acc[nf][mf]);
 }
 
-template <typename T, int BM, int BN, bool B_NK>
+template <typename T, int BM, int BN, bool B_NK, bool KTAIL>
 __global__ void __launch_bounds__((BM / 64) * (BN / 128) * 64)
 fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n)
 {
   typedef Fp16Tile<T, BM, BN, B_NK> TC;
+  typedef typename Mfma16<T>::vec   vec;
+  // four distinct arrays (not one indexed array) so that the compiler can tell which stage an
+  // access touches and does not serialise the LDS-direct loads against unrelated ds_reads
   __shared__ __attribute__((aligned(1024))) char lds0[TC::STAGE];
   __shared__ __attribute__((aligned(1024))) char lds1[TC::STAGE];
+  __shared__ __attribute__((aligned(1024))) char lds2[TC::STAGE];
+  __shared__ __attribute__((aligned(1024))) char lds3[TC::STAGE];
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -167,53 +159,39 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
   tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
-  // ---- loader setup: element offsets (relative to the tile's first row / column) per load
-  int a_off[TC::A_LOADS], a_chunk[TC::A_LOADS], b_off[TC::B_LOADS], b_kc[TC::B_LOADS];
-#pragma unroll
-  for (int i = 0; i < TC::A_LOADS; ++i) {
-    const KMajorLane p = kmajor_lane<SWZ_ROWS32>(wave + i * TC::NW, lane);
-    a_off[i]           = p.row * K + p.chunk * 8;
-    a_chunk[i]         = p.chunk;
+  // ---- loader setup
+  const KMajorLane lp    = kmajor_lane<SWZ_ROW64>(wave, lane);
+  const unsigned   a_off = (unsigned)(lp.row * K + lp.chunk * 8);
+  const int        a_k   = lp.chunk * 8;
+  unsigned         b_off;
+  int              b_k;
+  if constexpr (B_NK) {
+    b_off = a_off;
+    b_k   = a_k;
   }
-#pragma unroll
-  for (int i = 0; i < TC::B_LOADS; ++i) {
-    const int g = wave + i * TC::NW;
-    if constexpr (B_NK) {
-      const KMajorLane p = kmajor_lane<SWZ_ROWS32>(g, lane);
-      b_off[i]           = p.row * K + p.chunk * 8;
-      b_kc[i]            = p.chunk * 8;
-    }
-    else {
-      constexpr int ROWS_PER_GROUP = 1024 / TC::B_ROW;
-      const int     k              = g * ROWS_PER_GROUP + (lane * 16) / TC::B_ROW;
-      const int     pbyte          = (lane * 16) % TC::B_ROW;
-      const int     ch             = (pbyte >> 6) ^ (k & 3);
-      b_off[i]                     = k * N + ((ch << 6) + (pbyte & 63)) / 2;
-      b_kc[i]                      = k;
-    }
+  else {
+    const int k     = wave * TC::B_KROWS_PER_GRP + (lane * 16) / TC::B_ROW;
+    const int pbyte = (lane * 16) % TC::B_ROW;
+    const int ch    = (pbyte >> 6) ^ (k & 3);
+    b_off           = (unsigned)(k * N + ((ch << 6) + (pbyte & 63)) / 2);
+    b_k             = k;
   }
   const T* Ag = A + (size_t)m0 * K;
   const T* Bg = B_NK ? B + (size_t)n0 * K : B + n0;
 
   // ---- operand read setup (byte offsets inside a stage)
-  int a_rd[2], b_rd[4];
-  const int hi = lane >> 5;
-#pragma unroll
-  for (int mf = 0; mf < 2; ++mf) {
-    const int r = wm * 64 + mf * 32 + (lane & 31);
-    a_rd[mf]    = kmajor_phys_row<SWZ_ROWS32>(r) * 128 + ((hi ^ kmajor_swz<SWZ_ROWS32>(r)) << 4);
+  const int hi   = lane >> 5;
+  const int a_rd = kmajor_offset<SWZ_ROW64>(wm * 64 + (lane & 31), hi);
+  int       b_rd[4];
+  if constexpr (B_NK) {
+    b_rd[0] = kmajor_offset<SWZ_ROW64>(wn * 128 + (lane & 31), hi);
+    b_rd[1] = b_rd[2] = b_rd[3] = 0;
   }
+  else {
+    const int blk = lane >> 4, i = lane & 15;
 #pragma unroll
-  for (int nf = 0; nf < 4; ++nf) {
-    if constexpr (B_NK) {
-      const int r = wn * 128 + nf * 32 + (lane & 31);
-      b_rd[nf]    = kmajor_phys_row<SWZ_ROWS32>(r) * 128 + ((hi ^ kmajor_swz<SWZ_ROWS32>(r)) << 4);
-    }
-    else {
-      const int blk = lane >> 4, i = lane & 15;
-      const int ch  = wn * 4 + nf;
-      b_rd[nf] = (8 * (blk >> 1) + (i >> 2)) * TC::B_ROW + ((ch ^ (i >> 2)) << 6) + (blk & 1) * 32 + (i & 3) * 8;
-    }
+    for (int nf = 0; nf < 4; ++nf)
+      b_rd[nf] = (8 * (blk >> 1) + (i >> 2)) * TC::B_ROW + (((wn * 4 + nf) ^ (i >> 2)) << 6) + (blk & 1) * 32 + (i & 3) * 8;
   }
 
   f32x16 acc[4][2];
@@ -224,29 +202,74 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[nf][mf][r] = 0.0f;
 
-  const int    KT      = (K + TC::BK - 1) / TC::BK;
-  const size_t b_step  = B_NK ? (size_t)TC::BK : (size_t)TC::BK * N;
-  char LLMMM_LDS* const s0 = (char LLMMM_LDS*)lds0;
-  char LLMMM_LDS* const s1 = (char LLMMM_LDS*)lds1;
+  const int    KT          = (K + TC::BK - 1) / TC::BK;
+  const int    full_stages = K / TC::BK;
+  const size_t b_step      = B_NK ? (size_t)TC::BK : (size_t)TC::BK * N;
 
-  fp16_issue_stage<T, BM, BN, B_NK>(s0, Ag, Bg, a_off, a_chunk, b_off, b_kc, wave, lane, K);
-  for (int kt = 0; kt < KT; kt += 2) {
-    // even stage: data in lds0, prefetch into lds1
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): this wave's loads / zero-fills have landed
-    __syncthreads();
-    if (kt + 1 < KT)
-      fp16_issue_stage<T, BM, BN, B_NK>(s1, Ag + (size_t)(kt + 1) * TC::BK, Bg + (size_t)(kt + 1) * b_step, a_off, a_chunk, b_off,
-                                        b_kc, wave, lane, K - (kt + 1) * TC::BK);
-    fp16_compute_stage<T, BM, BN, B_NK>(s0, a_rd, b_rd, acc);
-    if (kt + 1 < KT) {
-      __builtin_amdgcn_s_waitcnt(0x0070);
-      __syncthreads();
-      if (kt + 2 < KT)
-        fp16_issue_stage<T, BM, BN, B_NK>(s0, Ag + (size_t)(kt + 2) * TC::BK, Bg + (size_t)(kt + 2) * b_step, a_off, a_chunk,
-                                          b_off, b_kc, wave, lane, K - (kt + 2) * TC::BK);
-      fp16_compute_stage<T, BM, BN, B_NK>(s1, a_rd, b_rd, acc);
-    }
+  char LLMMM_LDS* const ring[4] = {(char LLMMM_LDS*)lds0, (char LLMMM_LDS*)lds1, (char LLMMM_LDS*)lds2, (char LLMMM_LDS*)lds3};
+
+#define LLMMM_ISSUE(stage, buf)                                                                                              \
+  fp16_issue_stage<T, BM, BN, B_NK, KTAIL>(ring[buf], Ag + (size_t)(stage) * TC::BK, Bg + (size_t)(stage) * b_step, a_off, a_k, b_off, \
+                                    b_k, K, N, wave, lane, K - (stage) * TC::BK)
+
+  // prologue: stages 0..2 in flight, stage 0 landed and published, then stage 3 behind the barrier
+  LLMMM_ISSUE(0, 0);
+  if (1 < KT) LLMMM_ISSUE(1, 1);
+  if (2 < KT) LLMMM_ISSUE(2, 2);
+  wait_vmcnt<0>();
+  __builtin_amdgcn_s_barrier();
+  if (3 < KT) LLMMM_ISSUE(3, 3);
+
+  vec a0[2], b0[4], a1[2], b1[4];
+  fp16_read_frags<T, BM, BN, B_NK>(ring[0], a_rd, b_rd, 0, a0, b0);
+
+  // One stage s (in ring[u]).  STEADY = "stages s+1 .. s+4 exist and are full" (straight-line code).
+  // The LDS reads of the next k-step are issued between the two MFMA halves of the current one:
+  // by the time their data is needed four MFMAs (>= 128 cycles) have been issued behind them.
+  // (While LDS-direct loads are in flight the compiler only ever waits for *all* LDS reads, so a
+  // read must never be issued right before a wait.)
+#define LLMMM_STAGE(STEADY, s, u)                                                                                  \
+  {                                                                                                                \
+    fp16_mfma_half<T>(0, a0, b0, acc);                                                                             \
+    __builtin_amdgcn_sched_barrier(0);                                                                             \
+    fp16_read_frags<T, BM, BN, B_NK>(ring[u], a_rd, b_rd, 1, a1, b1);                                              \
+    __builtin_amdgcn_sched_barrier(0);                                                                             \
+    fp16_mfma_half<T>(1, a0, b0, acc);                                                                             \
+    __builtin_amdgcn_sched_barrier(0);                                                                             \
+    /* every LDS read of stage s has been issued; once they are back (lgkmcnt(0), part of each wait below) the */ \
+    /* barrier hands ring[u] to the loader and publishes stage s+1 */                                             \
+    if (STEADY || (s) + 3 < full_stages)                                                                           \
+      wait_vmcnt<2 * TC::LOADS>(); /* stages s+2 and s+3 may still be in flight */                                 \
+    else if ((s) + 2 < full_stages)                                                                                \
+      wait_vmcnt<TC::LOADS>();                                                                                     \
+    else                                                                                                           \
+      wait_vmcnt<0>();                                                                                             \
+    __builtin_amdgcn_s_barrier();                                                                                  \
+    if (STEADY || (s) + 4 < KT) LLMMM_ISSUE((s) + 4, u);                                                           \
+    fp16_mfma_half<T>(0, a1, b1, acc);                                                                             \
+    __builtin_amdgcn_sched_barrier(0);                                                                             \
+    /* unconditional: after the last stage this reads a stale buffer and the result is unused */                  \
+    fp16_read_frags<T, BM, BN, B_NK>(ring[((u) + 1) & 3], a_rd, b_rd, 0, a0, b0);                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                             \
+    fp16_mfma_half<T>(1, a1, b1, acc);                                                                             \
+    __builtin_amdgcn_sched_barrier(0);                                                                             \
   }
+
+  int kt = 0;
+  for (; kt + 8 <= full_stages; kt += 4) {
+    LLMMM_STAGE(true, kt + 0, 0)
+    LLMMM_STAGE(true, kt + 1, 1)
+    LLMMM_STAGE(true, kt + 2, 2)
+    LLMMM_STAGE(true, kt + 3, 3)
+  }
+  for (; kt < KT; kt += 4) {
+    if (kt + 0 < KT) LLMMM_STAGE(false, kt + 0, 0)
+    if (kt + 1 < KT) LLMMM_STAGE(false, kt + 1, 1)
+    if (kt + 2 < KT) LLMMM_STAGE(false, kt + 2, 2)
+    if (kt + 3 < KT) LLMMM_STAGE(false, kt + 3, 3)
+  }
+#undef LLMMM_STAGE
+#undef LLMMM_ISSUE
 
   // ---- epilogue: lane holds, for row m = ..+lane%32, the columns 8*(r/4) + 4*(lane/32) + r%4
   const int m = m0 + wm * 64 + (lane & 31);
@@ -257,9 +280,9 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
     for (int nf = 0; nf < 4; ++nf)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        typedef T       tx4 __attribute__((ext_vector_type(4)));
-        const f32x16&   v = acc[nf][mf];
-        tx4             o;
+        typedef T     tx4 __attribute__((ext_vector_type(4)));
+        const f32x16& v = acc[nf][mf];
+        tx4           o;
         o[0] = (T)v[4 * q + 0];
         o[1] = (T)v[4 * q + 1];
         o[2] = (T)v[4 * q + 2];
@@ -275,8 +298,12 @@ static hipError_t launch_fp16(const void* A, const void* B, void* C, int M, int 
 {
   typedef Fp16Tile<T, BM, BN, B_NK> TC;
   const int tiles_m = M / BM, tiles_n = N / BN;
-  hipLaunchKernelGGL((fp16_gemm_kernel<T, BM, BN, B_NK>), dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const T*)A,
-                     (const T*)B, (T*)C, M, N, K, tiles_m, tiles_n);
+  if (K % TC::BK)
+    hipLaunchKernelGGL((fp16_gemm_kernel<T, BM, BN, B_NK, true>), dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const T*)A,
+                       (const T*)B, (T*)C, M, N, K, tiles_m, tiles_n);
+  else
+    hipLaunchKernelGGL((fp16_gemm_kernel<T, BM, BN, B_NK, false>), dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const T*)A,
+                       (const T*)B, (T*)C, M, N, K, tiles_m, tiles_n);
   return hipGetLastError();
 }
 

@@ -37,21 +37,6 @@ __device__ __forceinline__ f32x4 mfma_fp8_k128(i32x8 x, i32x8 y)
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, z, 0, 0, 0, 0, 0, 0);
 }
 
-__device__ __forceinline__ void fp8_tile_coords(int wg, int tiles_m, int tiles_n, int& tm, int& tn)
-{
-  const int tiles = tiles_m * tiles_n;
-  int       L     = wg;
-  if ((tiles & 7) == 0) L = (wg & 7) * (tiles >> 3) + (wg >> 3);
-  constexpr int GROUP_M = 4;
-  const int     per     = GROUP_M * tiles_n;
-  const int     group   = L / per;
-  const int     first   = group * GROUP_M;
-  const int     gm      = (tiles_m - first) < GROUP_M ? (tiles_m - first) : GROUP_M;
-  const int     in      = L - group * per;
-  tm                    = first + in % gm;
-  tn                    = in / gm;
-}
-
 template <int BM, int BN>
 struct Fp8Tile {
   static constexpr int WAVES_M = BM / 64;
@@ -65,32 +50,38 @@ struct Fp8Tile {
   static constexpr int B_LOADS = (BN / 8) / NW;
 };
 
+// All loads of a wave share one per-lane offset: load i of the wave covers tile rows
+// 8*(wave + i*NW) .. +7, and the SWZ_ROWS16 placement only looks at row bits 0..3, so moving by
+// 8*NW (>= 16) rows changes nothing but the (wave-uniform) row base.
 template <int BM, int BN>
 __device__ __forceinline__ void fp8_issue_stage(char LLMMM_LDS* lds, const uint8_t* __restrict__ Ag,
-                                                const uint8_t* __restrict__ Bg, const int (&a_off)[Fp8Tile<BM, BN>::A_LOADS],
-                                                const int (&b_off)[Fp8Tile<BM, BN>::B_LOADS], int wave)
+                                                const uint8_t* __restrict__ Bg, int lane_off, int K, int wave)
 {
   typedef Fp8Tile<BM, BN> TC;
 #pragma unroll
-  for (int i = 0; i < TC::A_LOADS; ++i) load_lds_16B(Ag + a_off[i], lds + (wave + i * TC::NW) * 1024);
+  for (int i = 0; i < TC::A_LOADS; ++i)
+    load_lds_16B(Ag + (size_t)(8 * TC::NW * i) * K + lane_off, lds + (wave + i * TC::NW) * 1024);
 #pragma unroll
-  for (int i = 0; i < TC::B_LOADS; ++i) load_lds_16B(Bg + b_off[i], lds + TC::A_BYTES + (wave + i * TC::NW) * 1024);
+  for (int i = 0; i < TC::B_LOADS; ++i)
+    load_lds_16B(Bg + (size_t)(8 * TC::NW * i) * K + lane_off, lds + TC::A_BYTES + (wave + i * TC::NW) * 1024);
 }
 
-__device__ __forceinline__ i32x8 fp8_read_frag(const char LLMMM_LDS* tile, int rd)
+// 32 bytes of one row: chunk 2g at rd0 and chunk 2g+1 at rd1 (= rd0 ^ 16); `imm` selects the
+// 16-row fragment (a multiple of 2048 bytes, which the swizzle does not see).
+__device__ __forceinline__ i32x8 fp8_read_frag(const char LLMMM_LDS* tile, int rd0, int rd1, int imm)
 {
   union {
     i32x4 h[2];
     i32x8 v;
   } u;
-  u.h[0] = *(const i32x4 LLMMM_LDS*)(tile + rd);
-  u.h[1] = *(const i32x4 LLMMM_LDS*)(tile + (rd ^ 16));
+  u.h[0] = *(const i32x4 LLMMM_LDS*)(tile + rd0 + imm);
+  u.h[1] = *(const i32x4 LLMMM_LDS*)(tile + rd1 + imm);
   return u.v;
 }
 
 // One 128-K slice of the wave's 64 x 128 sub-tile.  s[mf] = As[kb, row] * Bs[nb, kb].
 template <int BM, int BN>
-__device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, const int (&a_rd)[4], const int (&b_rd)[8],
+__device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int a_rd0, int a_rd1, int b_rd0, int b_rd1,
                                                   const float (&s)[4], f32x4 (&acc)[8][4])
 {
   typedef Fp8Tile<BM, BN> TC;
@@ -99,12 +90,12 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, con
   i32x8                   a[4], b[2];
   f32x4                   p[2][4];
 #pragma unroll
-  for (int mf = 0; mf < 4; ++mf) a[mf] = fp8_read_frag(ldsA, a_rd[mf]);
-  b[0] = fp8_read_frag(ldsB, b_rd[0]);
+  for (int mf = 0; mf < 4; ++mf) a[mf] = fp8_read_frag(ldsA, a_rd0, a_rd1, mf * 2048);
+  b[0] = fp8_read_frag(ldsB, b_rd0, b_rd1, 0);
 #pragma unroll
   for (int nf = 0; nf < 8; ++nf) {
     const int cur = nf & 1;
-    if (nf + 1 < 8) b[cur ^ 1] = fp8_read_frag(ldsB, b_rd[nf + 1]);
+    if (nf + 1 < 8) b[cur ^ 1] = fp8_read_frag(ldsB, b_rd0, b_rd1, (nf + 1) * 2048);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int mf = 0; mf < 4; ++mf) p[cur][mf] = mfma_fp8_k128(b[cur], a[mf]);
@@ -113,6 +104,15 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, con
       for (int mf = 0; mf < 4; ++mf)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[nf - 1][mf][r] = __builtin_fmaf(p[cur ^ 1][mf][r], s[mf], acc[nf - 1][mf][r]);
+      // Pin the promotion here (an empty asm the optimiser cannot move or sink), then ask for
+      // MFMA, 4 FMA, MFMA, 4 FMA ...: the FMAs of fragment nf-1 run under the MFMAs of fragment nf.
+#pragma unroll
+      for (int mf = 0; mf < 4; ++mf) asm volatile("" : "+v"(acc[nf - 1][mf]));
+#pragma unroll
+      for (int mf = 0; mf < 4; ++mf) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -120,6 +120,8 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, con
   for (int mf = 0; mf < 4; ++mf)
 #pragma unroll
     for (int r = 0; r < 4; ++r) acc[7][mf][r] = __builtin_fmaf(p[1][mf][r], s[mf], acc[7][mf][r]);
+#pragma unroll
+  for (int mf = 0; mf < 4; ++mf) asm volatile("" : "+v"(acc[7][mf]));
 }
 
 __device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float d)
@@ -151,32 +153,20 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const int wm   = wave % TC::WAVES_M;
   const int wn   = wave / TC::WAVES_M;
   int       tm, tn;
-  fp8_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
   const int KB = K >> 7;
 
-  int a_off[TC::A_LOADS], b_off[TC::B_LOADS];
-#pragma unroll
-  for (int i = 0; i < TC::A_LOADS; ++i) {
-    const KMajorLane p = kmajor_lane<SWZ_ROWS16>(wave + i * TC::NW, lane);
-    a_off[i]           = p.row * K + p.chunk * 16;
-  }
-#pragma unroll
-  for (int i = 0; i < TC::B_LOADS; ++i) {
-    const KMajorLane p = kmajor_lane<SWZ_ROWS16>(wave + i * TC::NW, lane);
-    b_off[i]           = p.row * K + p.chunk * 16;
-  }
-  const uint8_t* Ag = A + (size_t)m0 * K;
-  const uint8_t* Bg = Bt + (size_t)n0 * K;
+  const KMajorLane lp       = kmajor_lane<SWZ_ROWS16>(wave, lane);
+  const int        lane_off = lp.row * K + lp.chunk * 16;
+  const uint8_t*   Ag       = A + (size_t)m0 * K;
+  const uint8_t*   Bg       = Bt + (size_t)n0 * K;
 
   // operand reads: lane = (g = lane/16, i = lane%16) takes row i of a 16-row fragment and the
-  // 32 bytes k = 32g .. 32g+31 (chunks 2g and 2g+1; the second one sits at offset ^ 16)
-  int       a_rd[4], b_rd[8];
-  const int g = lane >> 4;
-#pragma unroll
-  for (int mf = 0; mf < 4; ++mf) a_rd[mf] = kmajor_offset<SWZ_ROWS16>(wm * 64 + mf * 16 + (lane & 15), 2 * g);
-#pragma unroll
-  for (int nf = 0; nf < 8; ++nf) b_rd[nf] = kmajor_offset<SWZ_ROWS16>(wn * 128 + nf * 16 + (lane & 15), 2 * g);
+  // 32 bytes k = 32g .. 32g+31 (chunks 2g and 2g+1)
+  const int g     = lane >> 4;
+  const int a_rd0 = kmajor_offset<SWZ_ROWS16>(wm * 64 + (lane & 15), 2 * g), a_rd1 = a_rd0 ^ 16;
+  const int b_rd0 = kmajor_offset<SWZ_ROWS16>(wn * 128 + (lane & 15), 2 * g), b_rd1 = b_rd0 ^ 16;
 
   f32x4 acc[8][4];
 #pragma unroll
@@ -188,7 +178,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const int    mrow = m0 + wm * 64 + (lane & 15);
   const float* Asp  = As + mrow;
   const float* Bsp  = Bs + (size_t)((n0 >> 7) + wn) * KB;
-  float        sa[4], sa_next[4], sb, sb_next;
+  float        sa_next[4], sb_next;
 #pragma unroll
   for (int mf = 0; mf < 4; ++mf) sa_next[mf] = Asp[mf * 16];
   sb_next = Bsp[0];
@@ -196,7 +186,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   char LLMMM_LDS* const s0 = (char LLMMM_LDS*)lds0;
   char LLMMM_LDS* const s1 = (char LLMMM_LDS*)lds1;
 
-  fp8_issue_stage<BM, BN>(s0, Ag, Bg, a_off, b_off, wave);
+  fp8_issue_stage<BM, BN>(s0, Ag, Bg, lane_off, K, wave);
   for (int kb = 0; kb < KB; kb += 2) {
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
@@ -208,17 +198,15 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
 #pragma unroll
         for (int mf = 0; mf < 4; ++mf) s[mf] = sa_next[mf] * sb_next;
         if (kc + 1 < KB) {
-          fp8_issue_stage<BM, BN>(half ? s0 : s1, Ag + (size_t)(kc + 1) * 128, Bg + (size_t)(kc + 1) * 128, a_off, b_off, wave);
+          fp8_issue_stage<BM, BN>(half ? s0 : s1, Ag + (size_t)(kc + 1) * 128, Bg + (size_t)(kc + 1) * 128, lane_off, K, wave);
 #pragma unroll
           for (int mf = 0; mf < 4; ++mf) sa_next[mf] = Asp[(size_t)(kc + 1) * M + mf * 16];
           sb_next = Bsp[kc + 1];
         }
-        fp8_compute_stage<BM, BN>(half ? s1 : s0, a_rd, b_rd, s, acc);
+        fp8_compute_stage<BM, BN>(half ? s1 : s0, a_rd0, a_rd1, b_rd0, b_rd1, s, acc);
       }
     }
   }
-  (void)sa;
-  (void)sb;
 
   // ---- epilogue.  lane (g, i): row m = .. + mf*16 + i, columns n = nf*16 + 4g + r
   const int ncol = n0 + wn * 128 + 4 * g;

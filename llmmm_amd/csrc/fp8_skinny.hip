@@ -50,8 +50,8 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   const int ng   = blockIdx.x;
   const int sp   = blockIdx.y;
   const int KB   = K >> 7;
-  const int kb0  = (int)((long)sp * KB / S);
-  const int kb1  = (int)((long)(sp + 1) * KB / S);
+  const int kb0  = sp * KB / S;  // KB * S is small: 32-bit arithmetic (a 64-bit divide costs hundreds of scalar ops)
+  const int kb1  = (sp + 1) * KB / S;
 
   const int      nrow = ng * 128 + wave * 16 + i;
   const uint8_t* wp   = Bt + (size_t)nrow * K + 16 * g;
@@ -111,12 +111,20 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   const int ncol = ng * 128 + wave * 16 + 4 * g;
 
   if (S > 1) {
+    // Partials travel through device-coherent (agent-scope, relaxed) stores and loads, which
+    // write through / read past the per-XCD L2.  That makes full release/acquire fences
+    // unnecessary: a fence at agent scope writes back and invalidates the whole L2 of the XCD,
+    // which costs far more than this kernel's entire run.
 #pragma unroll
     for (int mb = 0; mb < MBLK; ++mb) {
       const int m = mb * 16 + i;
-      if (m < M) *(f32x4*)(partial + ((size_t)sp * M + m) * N + ncol) = acc[mb];
+      if (m < M) {
+        float* dst = partial + ((size_t)sp * M + m) * N + ncol;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) __hip_atomic_store(dst + r, acc[mb][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
-    __threadfence();
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): this wave's partial stores are acknowledged
     __syncthreads();
     if (tid == 0) {
       const unsigned old = __hip_atomic_fetch_add(counters + ng, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -124,23 +132,20 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
     }
     __syncthreads();
     if (!is_last) return;
-    __threadfence();
 #pragma unroll
     for (int mb = 0; mb < MBLK; ++mb) {
       const int m = mb * 16 + i;
       f32x4     t = {0.f, 0.f, 0.f, 0.f};
       if (m < M) {
-        for (int s = 0; s < S; ++s) {
-          const f32x4 v = *(const f32x4*)(partial + ((size_t)s * M + m) * N + ncol);
-          t[0] += v[0];
-          t[1] += v[1];
-          t[2] += v[2];
-          t[3] += v[3];
+        for (int s = 0; s < S; ++s) {  // fixed order 0..S-1, whoever arrived last
+          const float* src = partial + ((size_t)s * M + m) * N + ncol;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) t[r] += __hip_atomic_load(src + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
       acc[mb] = t;
     }
-    if (tid == 0) counters[ng] = 0;  // ready for the next launch
+    if (tid == 0) __hip_atomic_store(counters + ng, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
   }
 
   if constexpr (OUT == SK_OUT_F32) {
