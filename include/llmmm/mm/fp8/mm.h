@@ -1,0 +1,77 @@
+// The reference's FP8 launchers, promoted from examples/005.fp8.mm*.cu into the library with
+// their signatures unchanged (device pointers, stream last, std::runtime_error on misuse):
+//
+//   fp8_blockwise_symmetric_quantization<QUANT_M, QUANT_N, SCALE_TRANSPOSE>(x, q, scale, M, N, stream)
+//                                                                   examples/005.fp8.mm.cu:547-549
+//   fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(A, A_scale_transposed, B_transposed,
+//        B_scale_transposed, C, M, N, K, stream)                    examples/005.fp8.mm.cu:217-225
+//   fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(A, A_scale_transposed, B_transposed,
+//        B_scale_transposed, C, C_scale_transposed, M, N, K, stream)
+//                                   examples/005.fp8.mm.cu:2467-2476, examples/005.fp8.mm.opt.cu:468-508
+//   ...__output_bf16: the fp32 variant's result rounded to bf16 (no reference kernel).
+//
+// fp8_t stands for the reference's __nv_fp8_e4m3: one byte of OCP E4M3.  The launchers follow the
+// reference's rule M % 128 == 0, N % 128 == 0, K % 128 == 0 (examples/005.fp8.mm.cu:2490-2492) and
+// additionally accept 1 <= M <= 64 (decode), which the reference does not cover; small-M calls run
+// without split-K here because the reference signature has no workspace -- use llmmm_fp8_gemm()
+// with a workspace for the split-K path.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdexcept>
+#include <string>
+
+#include "../../../llmmm.h"
+
+namespace LLMMM {
+
+struct fp8_t {
+  unsigned char bits;  // OCP FP8 E4M3 code
+};
+static_assert(sizeof(fp8_t) == 1, "fp8_t must be one byte");
+
+namespace detail8 {
+inline void throw_on_error(int code)
+{
+  if (code == LLMMM_OK) return;
+  if (code == LLMMM_ERR_NOT_ALIGNED || code == LLMMM_ERR_UNSUPPORTED_TYPE) throw std::runtime_error(llmmm_error_string(code));
+  throw std::runtime_error(std::string(llmmm_error_string(code)) + ": " + llmmm_last_error());
+}
+}  // namespace detail8
+
+template <int QUANT_M, int QUANT_N, bool SCALE_TRANSPOSE>
+void fp8_blockwise_symmetric_quantization(const float* x, fp8_t* q, float* scale, int M, int N, hipStream_t stream)
+{
+  static_assert(QUANT_M == 1 || QUANT_M == 128, "QUANT_M must be 1 or 128");  // examples/005.fp8.mm.cu:551-552
+  static_assert(QUANT_N == 128, "QUANT_N must be 128");
+  constexpr int kind = QUANT_M == 1 ? (SCALE_TRANSPOSE ? LLMMM_QUANT_1x128_T : LLMMM_QUANT_1x128)
+                                    : (SCALE_TRANSPOSE ? LLMMM_QUANT_128x128_T : LLMMM_QUANT_128x128);
+  detail8::throw_on_error(llmmm_quant_fp8(kind, x, q, scale, M, N, (void*)stream));
+}
+
+inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(const fp8_t* A, const float* A_scale_transposed,
+                                                                     const fp8_t* B_transposed, const float* B_scale_transposed,
+                                                                     float* C, int M, int N, int K, hipStream_t stream)
+{
+  detail8::throw_on_error(
+    llmmm_fp8_gemm(LLMMM_OUT_F32, A, A_scale_transposed, B_transposed, B_scale_transposed, C, nullptr, M, N, K, nullptr, 0, (void*)stream));
+}
+
+inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(const fp8_t* A, const float* A_scale_transposed,
+                                                                     const fp8_t* B_transposed, const float* B_scale_transposed,
+                                                                     void* C, int M, int N, int K, hipStream_t stream)
+{
+  detail8::throw_on_error(
+    llmmm_fp8_gemm(LLMMM_OUT_BF16, A, A_scale_transposed, B_transposed, B_scale_transposed, C, nullptr, M, N, K, nullptr, 0, (void*)stream));
+}
+
+inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(const fp8_t* A, const float* A_scale_transposed,
+                                                                             const fp8_t* B_transposed,
+                                                                             const float* B_scale_transposed, fp8_t* C,
+                                                                             float* C_scale_transposed, int M, int N, int K,
+                                                                             hipStream_t stream)
+{
+  detail8::throw_on_error(llmmm_fp8_gemm(LLMMM_OUT_FP8Q, A, A_scale_transposed, B_transposed, B_scale_transposed, C, C_scale_transposed, M,
+                                         N, K, nullptr, 0, (void*)stream));
+}
+
+}  // namespace LLMMM

@@ -58,5 +58,19 @@ def build(verbose=False):
     return LIB
 
 
+def build_dropin_test():
+    """Compile tests/cpp/dropin_test.cpp (the C++ drop-in shims of include/llmmm/mm) against the library."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "cpp", "dropin_test.cpp")
+    out = os.path.join(root, "tests", "cpp", "dropin_test")
+    cmd = ["hipcc", "-std=c++17", "-O1", "-Wno-unused-command-line-argument", "-I", os.path.join(root, "include"), "-o", out, src,
+           "-L", HERE, "-lllmmm", "-Wl,-rpath,$ORIGIN/../../llmmm_amd"]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed for dropin_test.cpp:\n" + res.stdout)
+    return out
+
+
 if __name__ == "__main__":
     print(build(verbose="-v" in sys.argv))
+    print(build_dropin_test())

@@ -1,0 +1,100 @@
+// Drop-in check of the C++ entry points: same namespace, names, argument order and exceptions as
+// the reference (src/mm/fp16/mm.h:9-10, examples/005.fp8.mm.cu:217-225, :547-549, :2467-2476),
+// driven the way test/fp16_mm_test.cc drives them: raw device pointers, nullptr stream, sync outside.
+// Checks the reference's closed-form known answers (A = I corner; B = I) and the exception texts.
+#include "llmmm/mm/fp16/mm.h"
+#include "llmmm/mm/fp8/mm.h"
+
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#define CHECK(x)                                                                  \
+  do {                                                                            \
+    hipError_t e = (x);                                                           \
+    if (e != hipSuccess) {                                                        \
+      fprintf(stderr, "%s:%d %s\n", __FILE__, __LINE__, hipGetErrorString(e));    \
+      return 2;                                                                   \
+    }                                                                             \
+  } while (0)
+
+template <typename F>
+static bool throws_with(F f, const char* text)
+{
+  try {
+    f();
+  }
+  catch (const std::runtime_error& e) {
+    return std::string(e.what()) == text;
+  }
+  return false;
+}
+
+int main()
+{
+  int fails = 0;
+  const int M = 256, N = 256, K = 256, limit = 16;
+  // ---- fp16_mm<half>: A = I on a corner, B = row*limit + col  =>  C corner == B
+  std::vector<_Float16> hA(M * K, (_Float16)0.f), hB(K * N, (_Float16)0.f), hC(M * N);
+  for (int i = 0; i < limit; ++i) hA[i * K + i] = (_Float16)1.f;
+  for (int r = 0; r < limit; ++r)
+    for (int c = 0; c < limit; ++c) hB[r * N + c] = (_Float16)(float)(r * limit + c);
+  _Float16 *dA, *dB, *dC;
+  CHECK(hipMalloc(&dA, hA.size() * 2));
+  CHECK(hipMalloc(&dB, hB.size() * 2));
+  CHECK(hipMalloc(&dC, hC.size() * 2));
+  CHECK(hipMemcpy(dA, hA.data(), hA.size() * 2, hipMemcpyHostToDevice));
+  CHECK(hipMemcpy(dB, hB.data(), hB.size() * 2, hipMemcpyHostToDevice));
+  LLMMM::fp16_mm(dA, dB, dC, M, N, K, nullptr);
+  CHECK(hipDeviceSynchronize());
+  CHECK(hipMemcpy(hC.data(), dC, hC.size() * 2, hipMemcpyDeviceToHost));
+  for (int r = 0; r < M; ++r)
+    for (int c = 0; c < N; ++c) {
+      const float want = (r < limit && c < limit) ? (float)(r * limit + c) : 0.f;
+      if ((float)hC[r * N + c] != want) ++fails;
+    }
+  printf("fp16_mm<half> identity-corner KAT: %s\n", fails ? "FAIL" : "ok");
+  // ---- exceptions, texts of src/mm/fp16/mm.cu:15-21
+  if (!throws_with([&] { LLMMM::fp16_mm(dA, dB, dC, 128, N, K, nullptr); }, "M or N or K are not aligned.")) { ++fails; printf("misaligned M: FAIL\n"); }
+  if (!throws_with([&] { LLMMM::fp16_mm(dA, dB, dC, M, N, 8, nullptr); }, "M or N or K are not aligned.")) { ++fails; printf("misaligned K: FAIL\n"); }
+  if (!throws_with([&] { LLMMM::fp16_mm((const float*)dA, (const float*)dB, (float*)dC, M, N, K, nullptr); }, "T is not supported.")) { ++fails; printf("unsupported T: FAIL\n"); }
+  // ---- FP8: quantise A (1x128, transposed scales) and B^T = I (128x128), GEMM with fused C quant  =>  Cq == Aq
+  std::vector<float> fA(M * K), fI(N * K, 0.f);
+  unsigned s = 12345;
+  for (auto& v : fA) { s = s * 1664525u + 1013904223u; v = ((s >> 8) / 16777216.0f) * 10.f - 5.f; }
+  for (int i = 0; i < N; ++i) fI[i * K + i] = 1.f;
+  float *dfA, *dfI, *dAs, *dBs, *dCs, *dC32;
+  LLMMM::fp8_t *dAq, *dBq, *dCq;
+  CHECK(hipMalloc(&dfA, fA.size() * 4)); CHECK(hipMalloc(&dfI, fI.size() * 4));
+  CHECK(hipMalloc(&dAq, M * K)); CHECK(hipMalloc(&dBq, N * K)); CHECK(hipMalloc(&dCq, M * N));
+  CHECK(hipMalloc(&dAs, (K / 128) * M * 4)); CHECK(hipMalloc(&dBs, (N / 128) * (K / 128) * 4)); CHECK(hipMalloc(&dCs, (N / 128) * M * 4));
+  CHECK(hipMalloc(&dC32, M * N * 4));
+  CHECK(hipMemcpy(dfA, fA.data(), fA.size() * 4, hipMemcpyHostToDevice));
+  CHECK(hipMemcpy(dfI, fI.data(), fI.size() * 4, hipMemcpyHostToDevice));
+  LLMMM::fp8_blockwise_symmetric_quantization<1, 128, true>(dfA, dAq, dAs, M, K, nullptr);
+  LLMMM::fp8_blockwise_symmetric_quantization<128, 128, false>(dfI, dBq, dBs, N, K, nullptr);
+  LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(dAq, dAs, dBq, dBs, dCq, dCs, M, N, K, nullptr);
+  LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dAq, dAs, dBq, dBs, dC32, M, N, K, nullptr);
+  CHECK(hipDeviceSynchronize());
+  std::vector<unsigned char> hAq(M * K), hCq(M * N);
+  std::vector<float> hAs((K / 128) * M), hCs((N / 128) * M);
+  CHECK(hipMemcpy(hAq.data(), dAq, hAq.size(), hipMemcpyDeviceToHost));
+  CHECK(hipMemcpy(hCq.data(), dCq, hCq.size(), hipMemcpyDeviceToHost));
+  CHECK(hipMemcpy(hAs.data(), dAs, hAs.size() * 4, hipMemcpyDeviceToHost));
+  CHECK(hipMemcpy(hCs.data(), dCs, hCs.size() * 4, hipMemcpyDeviceToHost));
+  int f8 = 0;
+  if (memcmp(hAq.data(), hCq.data(), hAq.size()) != 0) ++f8;
+  for (size_t i = 0; i < hAs.size(); ++i)
+    if (!(hCs[i] >= hAs[i] * (1 - 1e-6f) && hCs[i] <= hAs[i] * (1 + 1e-6f))) ++f8;
+  printf("fp8 B = I KAT (Cq == Aq, Cs == As): %s\n", f8 ? "FAIL" : "ok");
+  fails += f8;
+  if (!throws_with([&] { LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dAq, dAs, dBq, dBs, dC32, M, 100, K, nullptr); },
+                   "M or N or K are not aligned.")) { ++fails; printf("fp8 misaligned N: FAIL\n"); }
+  if (!throws_with([&] { LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(dAq, dAs, dBq, dBs, dCq, dCs, 100, N, K, nullptr); },
+                   "M or N or K are not aligned.")) { ++fails; printf("fp8 misaligned M: FAIL\n"); }
+  printf(fails ? "DROPIN FAIL (%d)\n" : "DROPIN OK\n", fails);
+  return fails ? 1 : 0;
+}

@@ -1,0 +1,57 @@
+#!/usr/bin/env python3
+"""Writes the golden fixtures of the test-suite (inputs + expected outputs of the CPU oracle).
+
+    python tests/golden/make_golden.py
+
+The reference stores no golden vectors of its own (its tests print error statistics and assert
+nothing, test/fp16_mm_test.cc:63-82), so these fixtures are produced by this repository's
+oracle, which tests/test_oracle_*.py pin against closed forms and exact arithmetic.  They guard
+against drift of the oracle and give the GPU tests inputs with byte-stable expected outputs.
+"""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+import oracle  # noqa: E402
+
+
+def main():
+    rng = np.random.default_rng(20240601)
+    # FP16 GEMM 128 x 128 x 80 (K not a multiple of 32: exercises the K tail), fp16 and bf16 inputs
+    A = rng.uniform(-1, 1, (128, 80)).astype(np.float32)
+    B = rng.uniform(-1, 1, (80, 128)).astype(np.float32)
+    a16, b16 = oracle.f32_to_f16_bits(A), oracle.f32_to_f16_bits(B)
+    abf, bbf = oracle.f32_to_bf16_bits(A), oracle.f32_to_bf16_bits(B)
+    np.savez_compressed(os.path.join(HERE, "fp16_gemm_128x128x80.npz"),
+                        a_f16=a16, b_f16=b16, c_f16_kahan=oracle.kahan_gemm(oracle.f16_bits_to_f32(a16), oracle.f16_bits_to_f32(b16)),
+                        a_bf16=abf, b_bf16=bbf, c_bf16_kahan=oracle.kahan_gemm(oracle.bf16_bits_to_f32(abf), oracle.bf16_bits_to_f32(bbf)))
+    # quantiser: ragged rows, an outlier column, a zero block
+    x = rng.normal(0, 1, (130, 256)).astype(np.float32)
+    x[:, 77] *= 20
+    x[3, 128:] = 0
+    q1, s1 = oracle.quant_fp8(x, 1, True)
+    q128, s128 = oracle.quant_fp8(x, 128, False)
+    np.savez_compressed(os.path.join(HERE, "quant_130x256.npz"), x=x, q_1x128=q1, s_1x128_t=s1, q_128x128=q128, s_128x128=s128)
+    # FP8 blockwise GEMM 128 x 256 x 256 and a skinny M = 5 case on the same weights
+    X = rng.normal(0, 1, (128, 256)).astype(np.float32)
+    X[:, [9, 200]] *= 20
+    W = rng.normal(0, 0.02, (256, 256)).astype(np.float32)
+    Aq, As = oracle.quant_fp8(X, 1, True)
+    Bq, Bs = oracle.quant_fp8(W, 128, False)
+    C = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    Cq, Cs = oracle.requant_c_1x128(C)
+    A5q, A5s = oracle.quant_fp8(X[:5], 1, True)
+    C5 = oracle.fp8_gemm(A5q, A5s, Bq, Bs, promote=128)
+    C5q, C5s = oracle.requant_c_1x128(C5)
+    np.savez_compressed(os.path.join(HERE, "fp8_gemm_128x256x256.npz"), aq=Aq, a_scale_t=As, bq_t=Bq, b_scale=Bs, c_f32=C,
+                        c_bf16=oracle.f32_to_bf16_bits(C), cq=Cq, c_scale_t=Cs, a5q=A5q, a5_scale_t=A5s, c5_f32=C5, c5q=C5q, c5_scale_t=C5s)
+    for f in sorted(os.listdir(HERE)):
+        if f.endswith(".npz"):
+            print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,139 @@
+"""The C-ABI library without a GPU: it loads, exports every symbol that include/llmmm.h declares,
+and rejects bad arguments before any device work -- with the reference's exception texts
+(src/mm/fp16/mm.cu:15-21, examples/005.fp8.mm.cu:2490-2492).  No compute call is made here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "llmmm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"LLMMM_API\s+[\w\s\*]+?\b(llmmm_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from llmmm_amd import _lib
+    names = _declared_symbols()
+    assert len(names) >= 11
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), "libllmmm.so does not export " + n
+    assert sorted(_lib.SIGNATURES) == names, "llmmm_amd._lib.SIGNATURES and include/llmmm.h disagree"
+
+
+def test_error_strings_are_the_reference_texts():
+    from llmmm_amd._lib import lib
+    assert lib.llmmm_error_string(1) == b"M or N or K are not aligned."
+    assert lib.llmmm_error_string(2) == b"T is not supported."
+    assert lib.llmmm_error_string(0) == b"ok"
+    assert lib.llmmm_version() >= 100
+
+
+FAKE = ctypes.c_void_p(0x1000)  # 16-byte aligned, never dereferenced: validation fails first
+
+
+def test_fp16_validation_without_device():
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    f = lib.llmmm_fp16_gemm
+    assert f(0, FAKE, FAKE, FAKE, 100, 256, 256, 0, None) == _lib.ERR_NOT_ALIGNED
+    assert f(0, FAKE, FAKE, FAKE, 256, 200, 256, 0, None) == _lib.ERR_NOT_ALIGNED
+    assert f(0, FAKE, FAKE, FAKE, 256, 256, 24, 0, None) == _lib.ERR_NOT_ALIGNED
+    assert f(7, FAKE, FAKE, FAKE, 256, 256, 256, 0, None) == _lib.ERR_UNSUPPORTED_TYPE
+    assert f(0, FAKE, FAKE, FAKE, 256, 256, 256, 5, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(0, None, FAKE, FAKE, 256, 256, 256, 0, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(0, ctypes.c_void_p(0x1004), FAKE, FAKE, 256, 256, 256, 0, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(0, FAKE, FAKE, FAKE, 0, 256, 256, 0, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(0, FAKE, FAKE, FAKE, -256, 256, 256, 0, None) == _lib.ERR_INVALID_ARGUMENT
+    cfg = _lib.GemmCfg(_lib.TILE_256x256, 0)
+    assert lib.llmmm_fp16_gemm_ex(0, FAKE, FAKE, FAKE, 128, 256, 256, 0, ctypes.byref(cfg), None) == _lib.ERR_NOT_ALIGNED
+    cfg = _lib.GemmCfg(99, 0)
+    assert lib.llmmm_fp16_gemm_ex(0, FAKE, FAKE, FAKE, 256, 256, 256, 0, ctypes.byref(cfg), None) == _lib.ERR_INVALID_ARGUMENT
+
+
+def test_fp8_validation_without_device():
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    f = lib.llmmm_fp8_gemm
+    args = (FAKE, FAKE, FAKE, FAKE, FAKE, FAKE)
+    assert f(2, *args, 128, 100, 256, None, 0, None) == _lib.ERR_NOT_ALIGNED
+    assert f(2, *args, 128, 128, 200, None, 0, None) == _lib.ERR_NOT_ALIGNED
+    assert f(2, *args, 100, 128, 256, None, 0, None) == _lib.ERR_NOT_ALIGNED  # 64 < M, M % 128 != 0
+    assert f(9, *args, 128, 128, 256, None, 0, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(2, FAKE, FAKE, FAKE, FAKE, FAKE, None, 128, 128, 256, None, 0, None) == _lib.ERR_INVALID_ARGUMENT  # Cs missing
+    assert f(0, None, FAKE, FAKE, FAKE, FAKE, None, 128, 128, 256, None, 0, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(2, *args, 0, 128, 256, None, 0, None) == _lib.ERR_INVALID_ARGUMENT
+    # explicit split-K with a workspace that is too small
+    cfg = _lib.GemmCfg(_lib.TILE_SKINNY, 4)
+    assert lib.llmmm_fp8_gemm_ex(2, *args, 16, 256, 1024, FAKE, 4096, ctypes.byref(cfg), None) == _lib.ERR_WORKSPACE
+    assert b"workspace" in lib.llmmm_last_error()
+    cfg = _lib.GemmCfg(_lib.TILE_SKINNY, 1)
+    assert lib.llmmm_fp8_gemm_ex(2, *args, 128, 256, 1024, None, 0, ctypes.byref(cfg), None) == _lib.ERR_INVALID_ARGUMENT
+
+
+def test_quant_and_workspace_validation_without_device():
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    assert lib.llmmm_quant_fp8(0, FAKE, FAKE, FAKE, 16, 130, None) == _lib.ERR_NOT_ALIGNED
+    assert lib.llmmm_quant_fp8(9, FAKE, FAKE, FAKE, 16, 128, None) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.llmmm_quant_fp8(0, None, FAKE, FAKE, 16, 128, None) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.llmmm_quant_fp8(0, FAKE, FAKE, FAKE, 0, 128, None) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.llmmm_workspace_init(None, 0, None) == _lib.ERR_WORKSPACE
+    assert lib.llmmm_workspace_init(FAKE, 100, None) == _lib.ERR_WORKSPACE
+
+
+def test_workspace_sizes_and_config_queries():
+    import llmmm_amd
+    from llmmm_amd import _lib
+    # the tile kernels never need a workspace; the skinny kernel needs counters + S partial tiles
+    assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, 4096, 4096, 4096) == 0
+    assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, 128, 6144, 2560) == 0
+    for (n, k) in [(6144, 2560), (2560, 4096), (19456, 2560), (2560, 9728)]:
+        for m in (1, 16):
+            tile, split = llmmm_amd.query_config(_lib.OUT_FP8Q, m, n, k)
+            assert tile == _lib.TILE_SKINNY and 1 <= split <= min(32, k // 128)
+            assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, m, n, k) >= 4096 + split * m * n * 4
+        for m in (128, 2048):
+            tile, split = llmmm_amd.query_config(_lib.OUT_FP8Q, m, n, k)
+            assert tile in (_lib.TILE_256x256, _lib.TILE_128x256, _lib.TILE_256x128, _lib.TILE_128x128) and split == 1
+    assert llmmm_amd.query_config(_lib.OUT_FP8Q, 4096, 4096, 4096) == (_lib.TILE_256x256, 1)
+    with pytest.raises(RuntimeError, match="M or N or K are not aligned."):
+        llmmm_amd.query_config(_lib.OUT_FP8Q, 100, 4096, 4096)
+
+
+def test_python_mirror_raises_like_the_reference():
+    import torch
+    import llmmm_amd
+    a = torch.zeros((256, 256), dtype=torch.float32)
+    with pytest.raises(RuntimeError, match="T is not supported."):
+        llmmm_amd.fp16_mm(a, a, a, 256, 256, 256)
+    h = torch.zeros((256, 256), dtype=torch.float16)
+    for (m, n, k) in [(128, 256, 256), (256, 128, 256), (256, 256, 8)]:
+        with pytest.raises(RuntimeError, match="M or N or K are not aligned."):
+            llmmm_amd.fp16_mm(h, h, h, m, n, k)  # the reference's rule: M, N % 256, K % 16
+    with pytest.raises(TypeError):
+        llmmm_amd.fp16_mm(h, h, h, 256, 256, 256)  # host tensors are not device pointers
+    with pytest.raises(ValueError):
+        llmmm_amd.fp8_blockwise_symmetric_quantization(a, a, a, 256, 256, 64)  # QUANT_M must be 1 or 128
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    # the product has no fallback: without libllmmm.so the binding refuses to load
+    from llmmm_amd import _lib
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libllmmm.so"))
+    with pytest.raises(ImportError, match="no fallback"):
+        _lib.load()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "llmmm_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text and "liboracle" not in text, f

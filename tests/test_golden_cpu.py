@@ -1,0 +1,39 @@
+"""The committed golden fixtures are what the oracle produces today (guards against drift)."""
+import os
+
+import numpy as np
+
+G = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def test_fp16_fixture(oracle):
+    d = np.load(os.path.join(G, "fp16_gemm_128x128x80.npz"))
+    assert (oracle.kahan_gemm(oracle.f16_bits_to_f32(d["a_f16"]), oracle.f16_bits_to_f32(d["b_f16"])) == d["c_f16_kahan"]).all()
+    assert (oracle.kahan_gemm(oracle.bf16_bits_to_f32(d["a_bf16"]), oracle.bf16_bits_to_f32(d["b_bf16"])) == d["c_bf16_kahan"]).all()
+    # closed-form cross-check of the stored result: float64 matmul of the same fp16 values
+    ref = oracle.f16_bits_to_f32(d["a_f16"]).astype(np.float64) @ oracle.f16_bits_to_f32(d["b_f16"]).astype(np.float64)
+    assert np.abs(d["c_f16_kahan"] - ref).max() <= 2e-6
+
+
+def test_quant_fixture(oracle):
+    d = np.load(os.path.join(G, "quant_130x256.npz"))
+    q, s = oracle.quant_fp8(d["x"], 1, True)
+    assert (q == d["q_1x128"]).all() and (s == d["s_1x128_t"]).all()
+    q, s = oracle.quant_fp8(d["x"], 128, False)
+    assert (q == d["q_128x128"]).all() and (s == d["s_128x128"]).all()
+    assert (d["q_1x128"][3, 128:] == 0).all() and d["s_1x128_t"][1, 3] == 0
+
+
+def test_fp8_fixture(oracle):
+    d = np.load(os.path.join(G, "fp8_gemm_128x256x256.npz"))
+    C = oracle.fp8_gemm(d["aq"], d["a_scale_t"], d["bq_t"], d["b_scale"], promote=128)
+    assert (C == d["c_f32"]).all()
+    Cq, Cs = oracle.requant_c_1x128(C)
+    assert (Cq == d["cq"]).all() and (Cs == d["c_scale_t"]).all()
+    assert (oracle.f32_to_bf16_bits(C) == d["c_bf16"]).all()
+    C5 = oracle.fp8_gemm(d["a5q"], d["a5_scale_t"], d["bq_t"], d["b_scale"], promote=128)
+    assert (C5 == d["c5_f32"]).all() and (C5 == C[:5]).all()  # rows are independent
+    # closed-form cross-check: dequantise and multiply in float64
+    A = oracle.dequant_fp8(d["aq"], d["a_scale_t"], 1, True).astype(np.float64)
+    W = oracle.dequant_fp8(d["bq_t"], d["b_scale"], 128, False).astype(np.float64)
+    assert np.abs(C - A @ W.T).max() <= 1e-5 * np.abs(C).max()

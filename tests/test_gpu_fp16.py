@@ -1,0 +1,112 @@
+"""GPU parity tests of the FP16/BF16 GEMM (through the C ABI) against the Kahan oracle.
+Bar: |d| <= 1e-3 + 1e-2 * |ref| element-wise (fp32-accumulate Kahan reference on the rounded inputs)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_fp16_close, fp16_inputs_normal, fp16_inputs_uniform
+
+pytestmark = pytest.mark.gpu
+G = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+TILES = {"auto": -1, "256x256": 0, "128x256": 1, "256x128": 2, "128x128": 3}
+
+
+def _gpu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def test_cfg1_1024_both_layouts_bit_identical(lib, oracle):
+    # BASELINE configs[0]: M=N=K=1024, U(-1,1) seed 1, B row-major and transposed
+    A, B = fp16_inputs_uniform(1024, 1024, 1024, seed=1)
+    ref = oracle.kahan_gemm(A.astype(np.float32), B.astype(np.float32))
+    tA, tB = _gpu(A), _gpu(B)
+    C = torch.empty((1024, 1024), dtype=torch.float16, device="cuda")
+    lib.fp16_mm(tA, tB, C, 1024, 1024, 1024)  # the reference entry point
+    torch.cuda.synchronize()
+    c_rm = C.cpu().numpy()
+    assert_fp16_close(c_rm, ref, "fp16_mm 1024^3")
+    c_bt = lib.fp16_gemm(tA, _gpu(B.T), b_transposed=True).cpu().numpy()
+    assert_fp16_close(c_bt, ref, "fp16 gemm 1024^3 transposed B")
+    assert (c_rm.view(np.uint16) == c_bt.view(np.uint16)).all(), "the two B layouts must give identical bits"
+
+
+@pytest.mark.parametrize("tile", ["256x256", "128x256", "256x128", "128x128"])
+@pytest.mark.parametrize("bt", [False, True])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_every_tile_and_dtype(lib, oracle, tile, bt, dtype):
+    M, N, K = 512, 768, 544  # K = 17 stages: exercises the ring wrap-around and the pipeline tail
+    rng = np.random.default_rng(5)
+    A32 = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    B32 = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    tA, tB = torch.from_numpy(A32).cuda().to(tdt), torch.from_numpy(B32).cuda().to(tdt)
+    ref = oracle.kahan_gemm(tA.float().cpu().numpy(), tB.float().cpu().numpy())
+    C = lib.fp16_gemm(tA, tB.t().contiguous() if bt else tB, b_transposed=bt, tile=TILES[tile])
+    assert_fp16_close(C.float().cpu().numpy(), ref, "%s %s bt=%s" % (dtype, tile, bt))
+
+
+@pytest.mark.parametrize("K", [16, 32, 48, 80, 96, 112, 128, 144, 272])
+def test_k_tails_and_short_k(lib, oracle, K):
+    # the reference accepts any K % 16 == 0 (src/mm/fp16/mm.cu:18-21); stages are 32 wide here
+    rng = np.random.default_rng(K)
+    A = rng.uniform(-1, 1, (128, K)).astype(np.float16)
+    B = rng.uniform(-1, 1, (K, 256)).astype(np.float16)
+    ref = oracle.kahan_gemm(A.astype(np.float32), B.astype(np.float32))
+    for bt in (False, True):
+        C = lib.fp16_gemm(_gpu(A), _gpu(B.T if bt else B), b_transposed=bt)
+        assert_fp16_close(C.cpu().numpy(), ref, "K=%d bt=%s" % (K, bt))
+
+
+def test_golden_fixture(lib, oracle):
+    d = np.load(os.path.join(G, "fp16_gemm_128x128x80.npz"))
+    a = torch.from_numpy(d["a_f16"].view(np.int16)).cuda().view(torch.float16)
+    b = torch.from_numpy(d["b_f16"].view(np.int16)).cuda().view(torch.float16)
+    assert_fp16_close(lib.fp16_gemm(a, b).cpu().numpy(), d["c_f16_kahan"], "golden f16")
+    a = torch.from_numpy(d["a_bf16"].view(np.int16)).cuda().view(torch.bfloat16)
+    b = torch.from_numpy(d["b_bf16"].view(np.int16)).cuda().view(torch.bfloat16)
+    assert_fp16_close(lib.fp16_gemm(a, b).float().cpu().numpy(), d["c_bf16_kahan"], "golden bf16")
+
+
+def test_identity_corner_and_all_ones_known_answers(lib):
+    # reference KATs: A = I on a 16x16 corner, B = row*16 + col there (examples/004.fp16.mm.ldmatrix.cu:6750-6775)
+    M = N = K = 256
+    A = np.zeros((M, K), np.float16)
+    B = np.zeros((K, N), np.float16)
+    A[:16, :16] = np.eye(16)
+    B[:16, :16] = np.arange(256).reshape(16, 16)
+    C = lib.fp16_gemm(_gpu(A), _gpu(B)).cpu().numpy()
+    assert (C[:16, :16] == B[:16, :16]).all() and not C[16:].any() and not C[:, 16:].any()
+    ones = torch.ones((256, 2048), dtype=torch.float16, device="cuda")
+    C = lib.fp16_gemm(ones, ones, b_transposed=True)
+    assert (C == 2048).all()  # exact in fp16
+
+
+def test_output_is_fully_overwritten_and_deterministic(lib):
+    A, B = fp16_inputs_uniform(256, 256, 256, seed=9)
+    tA, tB = _gpu(A), _gpu(B)
+    C1 = torch.full((256, 256), float("nan"), dtype=torch.float16, device="cuda")
+    C2 = torch.full((256, 256), 7.0, dtype=torch.float16, device="cuda")
+    lib.fp16_mm(tA, tB, C1, 256, 256, 256)
+    lib.fp16_mm(tA, tB, C2, 256, 256, 256)
+    torch.cuda.synchronize()
+    assert not torch.isnan(C1).any() and torch.equal(C1, C2)
+
+
+def test_cfg2_4096_slab_against_kahan_and_linearity(lib, oracle):
+    # BASELINE configs[1] at full size: A ~ N(0,1), B ~ N(0,0.02), seed 2.  The Kahan oracle checks a
+    # 256-row slab of the full product; a size-independent property covers the rest:
+    # the rows of C only depend on the matching rows of A (row independence) -> compare with the GEMM of a
+    # permuted A.
+    M = N = K = 4096
+    A, B = fp16_inputs_normal(M, N, K, seed=2)
+    tA, tB = _gpu(A), _gpu(B)
+    C = lib.fp16_gemm(tA, tB)
+    torch.cuda.synchronize()
+    rows = np.r_[0:64, 1000:1064, 2047:2111, 4032:4096]
+    ref = oracle.kahan_gemm(A[rows].astype(np.float32), B.astype(np.float32))
+    assert_fp16_close(C[torch.from_numpy(rows).cuda()].cpu().numpy(), ref, "4096^3 slab")
+    perm = torch.randperm(M, device="cuda", generator=torch.Generator(device="cuda").manual_seed(0))
+    Cp = lib.fp16_gemm(tA[perm].contiguous(), tB)
+    assert torch.equal(Cp, C[perm]), "row permutation of A must permute the rows of C bit-exactly"

@@ -1,0 +1,188 @@
+"""GPU parity tests of the FP8 blockwise GEMM (fp32 / bf16 output and fused C re-quantisation),
+MFMA tile kernels and the small-M split-K kernel, through the C ABI, against the oracle.
+
+Bars: fp32/bf16 output within 2e-2 relative (floored at row-block amax * 2^-7); fused output:
+codes within one e4m3 step on >= 99.9 % of the elements, scales within 1e-3 relative."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_fp8_gemm_close, assert_fused_close, fp8_inputs
+
+pytestmark = pytest.mark.gpu
+G = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+TILES = {"auto": -1, "256x256": 0, "128x256": 1, "256x128": 2, "128x128": 3}
+
+
+def _gpu(*arrs):
+    return [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in arrs]
+
+
+def _run_all(lib, Aq, As, Bq, Bs, tile=-1, split_k=0, use_ws=True):
+    M, K = Aq.shape
+    N = Bq.shape[0]
+    t = _gpu(Aq, As, Bq, Bs)
+    ws = lib.make_workspace(2, M, N, K) if use_ws else None
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
+    Cb = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    Cq = torch.full((M, N), 0x55, dtype=torch.uint8, device="cuda")
+    Cs = torch.full((N // 128, M), -1.0, dtype=torch.float32, device="cuda")
+    kw = dict(workspace=ws, tile=tile, split_k=split_k)
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(*t, C, M, N, K, **kw)
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(*t, Cb, M, N, K, **kw)
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(*t, Cq, Cs, M, N, K, **kw)
+    torch.cuda.synchronize()
+    return C.cpu().numpy(), Cb.view(torch.int16).cpu().numpy().view(np.uint16), Cq.cpu().numpy(), Cs.cpu().numpy()
+
+
+def _check_all(oracle, out, ref, what):
+    C, Cb, Cq, Cs = out
+    assert_fp8_gemm_close(C, ref, what + " fp32")
+    # bf16 output is defined as the round-to-nearest-even cast of the fp32 result
+    assert (Cb == oracle.f32_to_bf16_bits(C)).all(), what + " bf16 is not RNE(fp32 output)"
+    assert_fp8_gemm_close(oracle.bf16_bits_to_f32(Cb), ref, what + " bf16")
+    rq, rs = oracle.requant_c_1x128(ref)
+    assert_fused_close(oracle, Cq, Cs, rq, rs, what + " fused")
+    # the fused epilogue is exactly the oracle's re-quantisation applied to the kernel's own fp32 result
+    oq, os_ = oracle.requant_c_1x128(C)
+    assert (Cq == oq).all() and (Cs.view(np.uint32) == os_.view(np.uint32)).all(), what + " fused != requant(own fp32)"
+
+
+@pytest.mark.parametrize("tile", ["256x256", "128x256", "256x128", "128x128"])
+def test_tile_kernels_against_oracle(lib, oracle, tile):
+    M, N, K = 512, 768, 1152  # 9 slices: odd count exercises both LDS stages' tails
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=3)
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, tile=TILES[tile]), ref, "tile " + tile)
+
+
+def test_single_slice(lib, oracle):
+    Aq, As, Bq, Bs = fp8_inputs(oracle, 128, 128, 128, seed=11)
+    _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs), oracle.fp8_gemm(Aq, As, Bq, Bs), "K=128")
+
+
+def test_golden_fixture(lib, oracle):
+    d = np.load(os.path.join(G, "fp8_gemm_128x256x256.npz"))
+    out = _run_all(lib, d["aq"], d["a_scale_t"], d["bq_t"], d["b_scale"])
+    _check_all(oracle, out, d["c_f32"], "golden 128x256x256")
+    assert_fused_close(oracle, out[2], out[3], d["cq"], d["c_scale_t"], "golden fused")
+    out5 = _run_all(lib, d["a5q"], d["a5_scale_t"], d["bq_t"], d["b_scale"])
+    _check_all(oracle, out5, d["c5_f32"], "golden skinny M=5")
+    assert_fused_close(oracle, out5[2], out5[3], d["c5q"], d["c5_scale_t"], "golden skinny fused")
+
+
+def test_b_identity_known_answer(lib, oracle):
+    # reference KAT (examples/005.fp8.mm.cu:2620-2634): B = I  =>  C == dequant(A), Cq == Aq, Cs == As
+    M = N = K = 256
+    rng = np.random.default_rng(21)
+    A = rng.uniform(-5, 5, (M, K)).astype(np.float32)
+    Aq, As = oracle.quant_fp8(A, 1, True)
+    Bq, Bs = oracle.quant_fp8(np.eye(N, K, dtype=np.float32), 128, False)
+    C, Cb, Cq, Cs = _run_all(lib, Aq, As, Bq, Bs)
+    deq = oracle.dequant_fp8(Aq, As, 1, True)
+    assert np.abs(C - deq).max() <= 4 * np.spacing(np.abs(deq).max())
+    assert (Cq == Aq).all()
+    assert np.abs(Cs - As).max() <= 1e-6 * As.max()
+
+
+def test_zero_blocks_give_zero_codes_and_scales(lib, oracle):
+    # a 1x128 group of zeros: the reference's unguarded 0 * (448/0) yields NaN codes (0x7F); this
+    # library emits code 0 and scale 0 (documented deviation)
+    Aq, As, Bq, Bs = fp8_inputs(oracle, 128, 256, 256, seed=5)
+    Aq[7] = 0
+    As[:, 7] = 0
+    Bq[128:] = 0
+    Bs[1] = 0
+    C, Cb, Cq, Cs = _run_all(lib, Aq, As, Bq, Bs)
+    assert not C[7].any() and not C[:, 128:].any()
+    assert not Cq[7].any() and not Cq[:, 128:].any() and not Cs[:, 7].any() and not Cs[1].any()
+    assert np.isfinite(oracle.e4m3_decode(Cq)).all()
+
+
+@pytest.mark.parametrize("M", [1, 2, 15, 16, 17, 33, 64])
+@pytest.mark.parametrize("split", [1, 3, 8])
+def test_skinny_kernel_against_oracle(lib, oracle, M, split):
+    N, K = 384, 1024
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=M)
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, tile=8, split_k=split), ref, "skinny M=%d S=%d" % (M, split))
+
+
+def test_skinny_without_workspace_does_not_split(lib, oracle):
+    Aq, As, Bq, Bs = fp8_inputs(oracle, 4, 256, 2560, seed=8)
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, use_ws=False), ref, "skinny no workspace")
+
+
+def test_split_k_is_deterministic_and_reusable(lib, oracle):
+    # fixed-order reduction: bit-identical results run after run on the same workspace; the counters
+    # return to zero, so the workspace needs no re-initialisation between calls
+    M, N, K = 16, 2560, 4096
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=4)
+    t = _gpu(Aq, As, Bq, Bs)
+    ws = lib.make_workspace(2, M, N, K)
+    outs = []
+    for _ in range(5):
+        Cq = torch.empty((M, N), dtype=torch.uint8, device="cuda")
+        Cs = torch.empty((N // 128, M), dtype=torch.float32, device="cuda")
+        C = torch.empty((M, N), dtype=torch.float32, device="cuda")
+        lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(*t, Cq, Cs, M, N, K, workspace=ws)
+        lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(*t, C, M, N, K, workspace=ws)
+        outs.append((Cq.clone(), Cs.clone(), C.clone()))
+    torch.cuda.synchronize()
+    for o in outs[1:]:
+        assert all(torch.equal(a, b) for a, b in zip(o, outs[0]))
+    assert_fp8_gemm_close(outs[0][2].cpu().numpy(), oracle.fp8_gemm(Aq, As, Bq, Bs), "split-K auto")
+    assert int(ws[:4096].view(torch.int32).abs().sum()) == 0, "arrival counters must be back at zero"
+
+
+@pytest.mark.parametrize("name,N,K", [("qkv", 6144, 2560), ("o", 2560, 4096), ("gate_up", 19456, 2560), ("down", 2560, 9728)])
+@pytest.mark.parametrize("M", [1, 16])
+def test_cfg5_decode_shapes(lib, oracle, name, N, K, M):
+    # BASELINE configs[4] at M in {1, 16}: full shapes, oracle on the whole (small-M) product
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=hash(name) % 1000)
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs), ref, "%s M=%d" % (name, M))
+
+
+def _slab_check(lib, oracle, M, N, K, rows, seed):
+    """Full-size run on GPU-quantised inputs; the oracle checks a row slab, properties the rest."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    X = torch.randn((M, K), generator=g, device="cuda")
+    X[:, torch.randperm(K, generator=g, device="cuda")[:max(1, -(-K // 100))]] *= 20
+    W = torch.randn((N, K), generator=g, device="cuda") * 0.02
+    Aq, As = lib.quantize_activation(X)
+    Bq, Bs = lib.quantize_weight(W)
+    C = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    Cq = torch.empty((M, N), dtype=torch.uint8, device="cuda")
+    Cs = torch.empty((N // 128, M), dtype=torch.float32, device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(Aq, As, Bq, Bs, C, M, N, K)
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(Aq, As, Bq, Bs, Cq, Cs, M, N, K)
+    torch.cuda.synchronize()
+    r = torch.from_numpy(rows).cuda()
+    ref = oracle.fp8_gemm(Aq[r].cpu().numpy(), As[:, r].contiguous().cpu().numpy(), Bq.cpu().numpy(), Bs.cpu().numpy(), promote=128)
+    assert_fp8_gemm_close(C[r].cpu().numpy(), ref, "slab fp32")
+    rq, rs = oracle.requant_c_1x128(ref)
+    assert_fused_close(oracle, Cq[r].cpu().numpy(), Cs[:, r].contiguous().cpu().numpy(), rq, rs, "slab fused")
+    # properties over the whole output: every 1x128 group has a code of magnitude 448 (its amax element),
+    # scales equal amax/448 of the fp32 result, and re-quantising the dequantised output is the identity
+    dec = Cq.view(torch.float8_e4m3fn).float()
+    assert (dec.abs().reshape(M, N // 128, 128).amax(-1) == 448).all()
+    amax = C.abs().reshape(M, N // 128, 128).amax(-1)
+    assert ((Cs.t() - amax / 448.0).abs() <= 1e-6 * amax / 448.0).all()  # torch's own division may differ in the last bit
+    deq = dec * Cs.t().repeat_interleave(128, dim=1)
+    assert (deq - C).abs().max() <= amax.max() / 448 * 16.5
+    q2, s2 = lib.quantize_activation(deq)
+    assert (q2.view(torch.float8_e4m3fn).float() - dec).abs().max() == 0 or torch.equal(q2, Cq)
+
+
+def test_cfg3_cfg4_4096_full_size(lib, oracle):
+    _slab_check(lib, oracle, 4096, 4096, 4096, np.r_[0:48, 2040:2088, 4048:4096], seed=3)
+
+
+@pytest.mark.parametrize("name,N,K", [("qkv", 6144, 2560), ("down", 2560, 9728)])
+@pytest.mark.parametrize("M", [128, 2048])
+def test_cfg5_prefill_shapes(lib, oracle, name, N, K, M):
+    _slab_check(lib, oracle, M, N, K, np.r_[0:32, M - 32:M], seed=17)

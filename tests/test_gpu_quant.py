@@ -1,0 +1,77 @@
+"""GPU quantiser (through the C ABI) against the oracle: bit-exact codes and scales."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+G = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _run(lib, x, quant_m, transpose, sshape):
+    M, N = x.shape
+    q = torch.full((M, N), 0x55, dtype=torch.uint8, device="cuda")
+    s = torch.full(sshape, -1.0, dtype=torch.float32, device="cuda")
+    lib.fp8_blockwise_symmetric_quantization(torch.from_numpy(x).cuda(), q, s, M, N, quant_m, 128, transpose)
+    torch.cuda.synchronize()
+    return q.cpu().numpy(), s.cpu().numpy()
+
+
+@pytest.mark.parametrize("M,N", [(512, 1024), (77, 384), (1, 2560), (16, 128), (130, 260), (300, 132), (1, 4)])
+@pytest.mark.parametrize("quant_m,transpose", [(1, True), (1, False), (128, False), (128, True)])
+def test_bit_exact_against_oracle(lib, oracle, M, N, quant_m, transpose):
+    rng = np.random.default_rng(M * 1000 + N)
+    x = rng.normal(0, 1, (M, N)).astype(np.float32)
+    x[:, ::37] *= 20
+    if M > 3:
+        x[3, :] = 0
+    rq, rs = oracle.quant_fp8(x, quant_m, transpose)
+    q, s = _run(lib, x, quant_m, transpose, rs.shape)
+    assert (q == rq).all()
+    if quant_m == 128 and transpose:
+        # row stride M with only ceil(M/128) entries used per row (the reference's layout)
+        mb = -(-M // 128)
+        assert (s[:, :mb].view(np.uint32) == rs[:, :mb].view(np.uint32)).all()
+    else:
+        assert (s.view(np.uint32) == rs.view(np.uint32)).all()
+
+
+def test_golden_fixture(lib):
+    d = np.load(os.path.join(G, "quant_130x256.npz"))
+    q, s = _run(lib, d["x"], 1, True, d["s_1x128_t"].shape)
+    assert (q == d["q_1x128"]).all() and (s == d["s_1x128_t"]).all()
+    q, s = _run(lib, d["x"], 128, False, d["s_128x128"].shape)
+    assert (q == d["q_128x128"]).all() and (s == d["s_128x128"]).all()
+
+
+def test_special_values(lib, oracle):
+    x = np.zeros((4, 128), np.float32)
+    x[1, :] = 448.0
+    x[1, 5] = -448.0
+    x[2, 0] = 1e30
+    x[2, 1] = -3e29
+    x[2, 2] = 1e-30
+    x[3, :] = np.float32(1e-40)  # denormal amax: scale underflows, codes stay finite
+    rq, rs = oracle.quant_fp8(x, 1, True)
+    q, s = _run(lib, x, 1, True, rs.shape)
+    assert (q == rq).all() and (s.view(np.uint32) == rs.view(np.uint32)).all()
+    assert (q[0] == 0).all() and s[0, 0] == 0
+
+
+def test_full_size_activation_and_weight(lib, oracle):
+    # cfg3 shapes: activations 4096x4096 (1x128, transposed scales), weights 4096x4096 (128x128)
+    g = torch.Generator(device="cuda").manual_seed(3)
+    x = torch.randn((4096, 4096), generator=g, device="cuda")
+    x[:, torch.randperm(4096, generator=g, device="cuda")[:41]] *= 20
+    q, s = lib.quantize_activation(x)
+    wq, ws = lib.quantize_weight(x * 0.02)
+    torch.cuda.synchronize()
+    xs = x[:256].cpu().numpy()
+    rq, rs = oracle.quant_fp8(xs, 1, True)
+    assert (q[:256].cpu().numpy() == rq).all() and (s[:, :256].cpu().numpy() == rs).all()
+    rq, rs = oracle.quant_fp8((x * 0.02)[:256].cpu().numpy(), 128, False)
+    assert (wq[:256].cpu().numpy() == rq).all() and (ws[:2].cpu().numpy() == rs).all()
+    # size-independent invariant over the whole matrix: |q| <= 448 and every 1x128 block reaches +-448
+    dec = q.view(torch.float8_e4m3fn).float().abs().reshape(4096, 32, 128).amax(-1)
+    assert (dec == 448).all()
