@@ -32,12 +32,15 @@ constexpr int    NUM_CUS         = 256;   // MI355X
 
 int max_split_for(int K) { return (K / 128) < MAX_SPLIT_K ? (K / 128) : MAX_SPLIT_K; }
 
-// Split count for the weight-streaming kernel: enough workgroups (one per 128 columns x split)
-// to cover the chip about twice, every split at least two 128-K slices long.
-int heuristic_split(int N, int K)
+// Split count for the weight-streaming kernel when the tune table has no entry: about one
+// workgroup (one 128-column group x one split) per CU -- what the measured Qwen3-4B shapes
+// settle on -- every split at least two 128-K slices long, fewer splits when there are many
+// rows (the fp32 partial tiles grow with M).
+int heuristic_split(int M, int N, int K)
 {
   const int groups = N / 128, kb = K / 128;
-  int       s      = (2 * NUM_CUS + groups - 1) / groups;
+  int       s      = (240 + groups / 2) / groups;
+  if (M > 16) s = (s + 1) / 2;
   if (s > kb / 2) s = kb / 2;
   if (s > MAX_SPLIT_K) s = MAX_SPLIT_K;
   if (s < 1) s = 1;
@@ -94,7 +97,7 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
         cfg->split_k = e.split_k;
         break;
       }
-    if (cfg->split_k == 0) cfg->split_k = heuristic_split(N, K);
+    if (cfg->split_k == 0) cfg->split_k = heuristic_split(M, N, K);
     return LLMMM_OK;
   }
   if (M % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");

@@ -78,6 +78,24 @@ __device__ __forceinline__ void load_lds_16B(const void* gptr, void LLMMM_LDS* l
   __builtin_amdgcn_global_load_lds((const void LLMMM_GLOBAL*)gptr, lds_base, 16, 0, 0);
 }
 
+// The same load written as inline assembly, invisible to the compiler's wait-count bookkeeping.
+// While an LDS-direct load that the compiler knows about is in flight, every wait it inserts on
+// its own becomes "all loads done", which defeats a deep software pipeline; kernels that keep
+// many slices in flight issue all their vector-memory loads through these helpers and place the
+// s_waitcnt themselves.  lds_addr is the wave-uniform LDS byte address (goes to M0).
+__device__ __forceinline__ void asm_load_lds_16B(const void* gptr, unsigned lds_addr)
+{
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_addr) : "memory");
+}
+__device__ __forceinline__ void asm_load_16B(i32x4& dst, const void* gptr)
+{
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(gptr) : "memory");
+}
+__device__ __forceinline__ void asm_load_f32(float& dst, const void* gptr)
+{
+  asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(gptr) : "memory");
+}
+
 // s_waitcnt vmcnt(N) lgkmcnt(0): at most N of this wave's vector-memory loads still in flight,
 // every LDS access done.  simm16 = vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14.
 template <int N>

@@ -5,11 +5,11 @@
 // does not cover (its launchers require M % 128 == 0, examples/005.fp8.mm.opt.cu:492; split-K
 // is listed as unfinished in README.md:22).
 //
-//  * HBM-bound: every byte of Bt[N,K] is read exactly once, straight from global memory into
-//    the MFMA operand registers (no LDS).  One wavefront owns 16 weight rows; per 128-K slice
-//    lane (g = lane/16, i = lane%16) loads bytes [16g,16g+16) and [64+16g,64+16g+16) of row i,
-//    so each of the two load instructions touches 64 contiguous bytes per row.  The activation
-//    operand uses the same k -> register mapping, which is all the MFMA needs.
+//  * HBM-bound: every byte of Bt[N,K] is read exactly once.  One wavefront owns 16 weight rows;
+//    per 128-K slice it moves their 16 x 128 bytes global -> LDS with two LDS-direct loads that
+//    each cover 8 whole rows (full 128-byte lines per instruction), into a wave-private ring of
+//    D slots, and reads the MFMA operand back with two conflict-free ds_read_b128.  The
+//    activation rows go straight from global memory (L2) into the other operand's registers.
 //  * A workgroup = 8 waves = one 128-column quantisation group; grid.y = number of K splits.
 //  * split-K: each split writes its fp32 partial tile to the workspace; the workgroup that
 //    arrives last at the group's counter adds the partials in split order 0..S-1 (fixed order,
@@ -32,13 +32,102 @@ __device__ __forceinline__ uint32_t sk_pack_e4m3x4(float a, float b, float c, fl
   return (uint32_t)v;
 }
 
-template <int MBLK, int OUT>
+// What one 128-K slice needs besides the weights: the activation rows (straight into the MFMA
+// operand registers) and both scales.  Rows beyond M are clamped to M-1 (a valid address, no
+// divergence); their products are computed and never stored.
+template <int MBLK>
+struct SkinnySlot {
+  i32x4 a[MBLK][2];
+  float sa[MBLK];
+  float sb;
+};
+
+// Weights: the wave's 16 rows x 128 bytes of a slice travel global -> LDS with two LDS-direct
+// loads of 1 KB each.  A load covers 8 whole rows, so every 128-byte line is fetched by one
+// instruction in full; the SWZ_ROWS16 placement makes the operand read-back conflict-free.
+// One wave-private ring slot = 2 KB; no workgroup barrier is involved.
+constexpr int SKINNY_LOADS_PER_SLOT_BASE = 2;  // LDS-direct loads; + 3 per 16 activation rows
+
+// All vector-memory loads of a slot, in a fixed order, as inline assembly (see device_common.hip.h):
+// the kernel counts them itself.
+template <int MBLK>
+__device__ __forceinline__ void skinny_fetch(SkinnySlot<MBLK>& t, unsigned ring_slot, const uint8_t* wrow, unsigned w_off0,
+                                             unsigned w_off1, const uint8_t* const (&ap)[MBLK], const float* const (&asp)[MBLK],
+                                             const float* bsp, int kb, int M)
+{
+  asm_load_lds_16B(wrow + (size_t)kb * 128 + w_off0, ring_slot);
+  asm_load_lds_16B(wrow + (size_t)kb * 128 + w_off1, ring_slot + 1024);
+#pragma unroll
+  for (int mb = 0; mb < MBLK; ++mb) {
+    asm_load_16B(t.a[mb][0], ap[mb] + (size_t)kb * 128);
+    asm_load_16B(t.a[mb][1], ap[mb] + (size_t)kb * 128 + 16);
+    asm_load_f32(t.sa[mb], asp[mb] + (size_t)kb * M);
+  }
+  t.sb = bsp[kb];
+}
+
+// s_waitcnt vmcnt(N) that also "touches" the slot's registers, so that nothing reading them can
+// be moved in front of it.
+template <int N, int MBLK>
+__device__ __forceinline__ void skinny_wait(SkinnySlot<MBLK>& t)
+{
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  if constexpr (MBLK == 1)
+    asm volatile("s_waitcnt vmcnt(%3)" : "+v"(t.a[0][0]), "+v"(t.a[0][1]), "+v"(t.sa[0]) : "n"(N) : "memory");
+  else if constexpr (MBLK == 2)
+    asm volatile("s_waitcnt vmcnt(%6)"
+                 : "+v"(t.a[0][0]), "+v"(t.a[0][1]), "+v"(t.sa[0]), "+v"(t.a[1][0]), "+v"(t.a[1][1]), "+v"(t.sa[1])
+                 : "n"(N)
+                 : "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(%12)"
+                 : "+v"(t.a[0][0]), "+v"(t.a[0][1]), "+v"(t.sa[0]), "+v"(t.a[1][0]), "+v"(t.a[1][1]), "+v"(t.sa[1]), "+v"(t.a[2][0]),
+                   "+v"(t.a[2][1]), "+v"(t.sa[2]), "+v"(t.a[3][0]), "+v"(t.a[3][1]), "+v"(t.sa[3])
+                 : "n"(N)
+                 : "memory");
+}
+
+template <int MBLK>
+__device__ __forceinline__ void skinny_consume(const SkinnySlot<MBLK>& t, const char LLMMM_LDS* ring_slot, int w_rd, bool valid,
+                                               f32x4 (&acc)[MBLK])
+{
+  union {
+    i32x4 h[2];
+    i32x8 v;
+  } wf, af;
+  wf.h[0] = *(const i32x4 LLMMM_LDS*)(ring_slot + w_rd);
+  wf.h[1] = *(const i32x4 LLMMM_LDS*)(ring_slot + (w_rd ^ 16));
+#pragma unroll
+  for (int mb = 0; mb < MBLK; ++mb) {
+    af.h[0]       = t.a[mb][0];
+    af.h[1]       = t.a[mb][1];
+    const float s = valid ? t.sa[mb] * t.sb : 0.f;
+    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+    const f32x4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf.v, af.v, z, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[mb][r] = __builtin_fmaf(p[r], s, acc[mb][r]);
+  }
+}
+
+// D = ring depth = slices in flight per wave.  The host picks the largest D that does not exceed
+// the number of slices of the shortest split.
+template <int MBLK, int OUT, int D>
 __global__ void __launch_bounds__(512)
 fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
                   const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int S,
                   float* __restrict__ partial, unsigned* __restrict__ counters)
 {
-  constexpr int UNROLL = 4;
+  constexpr int LOADS = SKINNY_LOADS_PER_SLOT_BASE + 3 * MBLK;  // vector-memory loads per slot, issued in slot order
+  static_assert((D - 1) * LOADS < 64, "vmcnt is a 6-bit counter");
+  // one array per ring slot, so that the compiler can tell the slots apart
+  __shared__ __attribute__((aligned(1024))) char ring0[8 * 2048];
+  __shared__ __attribute__((aligned(1024))) char ring1[8 * 2048];
+  __shared__ __attribute__((aligned(1024))) char ring2[D > 2 ? 8 * 2048 : 16];
+  __shared__ __attribute__((aligned(1024))) char ring3[D > 2 ? 8 * 2048 : 16];
+  __shared__ __attribute__((aligned(1024))) char ring4[D > 4 ? 8 * 2048 : 16];
+  __shared__ __attribute__((aligned(1024))) char ring5[D > 4 ? 8 * 2048 : 16];
+  __shared__ __attribute__((aligned(1024))) char ring6[D > 4 ? 8 * 2048 : 16];
+  __shared__ __attribute__((aligned(1024))) char ring7[D > 4 ? 8 * 2048 : 16];
   __shared__ float    wave_amax[8][MBLK][16];
   __shared__ unsigned is_last;
 
@@ -53,59 +142,63 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   const int kb0  = sp * KB / S;  // KB * S is small: 32-bit arithmetic (a 64-bit divide costs hundreds of scalar ops)
   const int kb1  = (sp + 1) * KB / S;
 
-  const int      nrow = ng * 128 + wave * 16 + i;
-  const uint8_t* wp   = Bt + (size_t)nrow * K + 16 * g;
-  const float*   bsp  = Bs + (size_t)ng * KB;
+  char LLMMM_LDS* const ring[8] = {(char LLMMM_LDS*)ring0 + wave * 2048, (char LLMMM_LDS*)ring1 + wave * 2048,
+                                   (char LLMMM_LDS*)ring2 + wave * 2048, (char LLMMM_LDS*)ring3 + wave * 2048,
+                                   (char LLMMM_LDS*)ring4 + wave * 2048, (char LLMMM_LDS*)ring5 + wave * 2048,
+                                   (char LLMMM_LDS*)ring6 + wave * 2048, (char LLMMM_LDS*)ring7 + wave * 2048};
+  unsigned ring_addr[8];  // the same slots as wave-uniform LDS byte addresses, for the loader
+#pragma unroll
+  for (int u = 0; u < 8; ++u) ring_addr[u] = __builtin_amdgcn_readfirstlane((unsigned)(size_t)ring[u]);
+
+  // weights: loader lane -> (row, chunk) of the 1 KB group it fills; reader lane (g, i) -> row i, chunks 2g, 2g+1
+  const uint8_t*   wrow = Bt + (size_t)(ng * 128 + wave * 16) * K;
+  const KMajorLane l0   = kmajor_lane<SWZ_ROWS16>(0, lane);
+  const KMajorLane l1   = kmajor_lane<SWZ_ROWS16>(1, lane);
+  const unsigned   w_off0 = (unsigned)(l0.row * K + l0.chunk * 16), w_off1 = (unsigned)(l1.row * K + l1.chunk * 16);
+  const int        w_rd   = kmajor_offset<SWZ_ROWS16>(i, 2 * g);
+  const float*     bsp    = Bs + (size_t)ng * KB;
+  const uint8_t*   ap[MBLK];
+  const float*     asp[MBLK];
+#pragma unroll
+  for (int mb = 0; mb < MBLK; ++mb) {
+    const int m = min(mb * 16 + i, M - 1);
+    ap[mb]      = A + (size_t)m * K + 32 * g;  // same k -> register mapping as the weights: bytes 32g .. 32g+31
+    asp[mb]     = As + m;
+  }
 
   f32x4 acc[MBLK];
 #pragma unroll
   for (int mb = 0; mb < MBLK; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int kb = kb0; kb < kb1; kb += UNROLL) {
-    i32x4 w0[UNROLL], w1[UNROLL];
+  // Software pipeline, D slices in flight per wave, all vector-memory loads issued strictly in
+  // slot order so that "at most n loads outstanding" pins down which slots have landed.
+  // Slice indices beyond the split are clamped to its last slice (a repeated, cached load) and
+  // consumed with a zero scale; the last pass issues nothing and counts its waits down.
+  SkinnySlot<MBLK> slot[D];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      if (kb + u < kb1) {
-        w0[u] = __builtin_nontemporal_load((const i32x4*)(wp + (size_t)(kb + u) * 128));
-        w1[u] = __builtin_nontemporal_load((const i32x4*)(wp + (size_t)(kb + u) * 128 + 64));
-      }
-    }
+  for (int u = 0; u < D; ++u) {
+    skinny_fetch<MBLK>(slot[u], ring_addr[u], wrow, w_off0, w_off1, ap, asp, bsp, min(kb0 + u, kb1 - 1), M);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  int kb = kb0;
+  for (; kb + D < kb1; kb += D) {  // passes followed by another pass: consume a slot, refill it
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      if (kb + u < kb1) {
-        const float sb = bsp[kb + u];
-        union {
-          i32x4 h[2];
-          i32x8 v;
-        } wf;
-        wf.h[0] = w0[u];
-        wf.h[1] = w1[u];
-#pragma unroll
-        for (int mb = 0; mb < MBLK; ++mb) {
-          const int m = mb * 16 + i;
-          union {
-            i32x4 h[2];
-            i32x8 v;
-          } af;
-          float s = 0.f;
-          if (m < M) {
-            const uint8_t* ap = A + (size_t)m * K + (size_t)(kb + u) * 128 + 16 * g;
-            af.h[0]           = *(const i32x4*)ap;
-            af.h[1]           = *(const i32x4*)(ap + 64);
-            s                 = As[(size_t)(kb + u) * M + m] * sb;
-          }
-          else {
-            af.h[0] = i32x4{0, 0, 0, 0};
-            af.h[1] = i32x4{0, 0, 0, 0};
-          }
-          const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-          const f32x4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf.v, af.v, z, 0, 0, 0, 0, 0, 0);
-#pragma unroll
-          for (int r = 0; r < 4; ++r) acc[mb][r] = __builtin_fmaf(p[r], s, acc[mb][r]);
-        }
-      }
+    for (int u = 0; u < D; ++u) {
+      skinny_wait<(D - 1) * LOADS, MBLK>(slot[u]);
+      skinny_consume<MBLK>(slot[u], ring[u], w_rd, true, acc);
+      __builtin_amdgcn_sched_barrier(0);
+      skinny_fetch<MBLK>(slot[u], ring_addr[u], wrow, w_off0, w_off1, ap, asp, bsp, min(kb + u + D, kb1 - 1), M);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
+#define LLMMM_LAST(u)                                                              \
+  if constexpr ((u) < D) {                                                         \
+    skinny_wait<(D - 1 - (u)) * LOADS, MBLK>(slot[u]);                             \
+    skinny_consume<MBLK>(slot[u], ring[u], w_rd, kb + (u) < kb1, acc);             \
+    __builtin_amdgcn_sched_barrier(0);                                             \
+  }
+  LLMMM_LAST(0) LLMMM_LAST(1) LLMMM_LAST(2) LLMMM_LAST(3) LLMMM_LAST(4) LLMMM_LAST(5) LLMMM_LAST(6) LLMMM_LAST(7)
+#undef LLMMM_LAST
 
   // lane (g, i): row m = mb*16 + i, columns ncol .. ncol+3
   const int ncol = ng * 128 + wave * 16 + 4 * g;
@@ -137,10 +230,23 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
       const int m = mb * 16 + i;
       f32x4     t = {0.f, 0.f, 0.f, 0.f};
       if (m < M) {
-        for (int s = 0; s < S; ++s) {  // fixed order 0..S-1, whoever arrived last
-          const float* src = partial + ((size_t)s * M + m) * N + ncol;
+        // fixed order 0..S-1, whoever arrived last; the loads of eight splits are put in flight
+        // together (one round trip per batch instead of one per split), the sums stay sequential
+        for (int s0 = 0; s0 < S; s0 += 8) {
+          f32x4 v[8];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) t[r] += __hip_atomic_load(src + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int u = 0; u < 8; ++u) {
+            const int    sc  = (s0 + u < S) ? s0 + u : S - 1;  // clamped duplicate: loaded, not added
+            const float* src = partial + ((size_t)sc * M + m) * N + ncol;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[u][r] = __hip_atomic_load(src + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            if (s0 + u < S) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) t[r] += v[u][r];
+            }
         }
       }
       acc[mb] = t;
@@ -196,11 +302,11 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   }
 }
 
-template <int MBLK, int OUT>
+template <int MBLK, int OUT, int D>
 static hipError_t launch_skinny(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
                                 int N, int K, int S, float* partial, unsigned* counters, hipStream_t stream)
 {
-  hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT>), dim3(N / 128, S), dim3(512), 0, stream, (const uint8_t*)A, As,
+  hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D>), dim3(N / 128, S), dim3(512), 0, stream, (const uint8_t*)A, As,
                      (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial, counters);
   return hipGetLastError();
 }
@@ -209,9 +315,22 @@ template <int OUT>
 static hipError_t dispatch_skinny(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
                                   int N, int K, int S, float* partial, unsigned* counters, hipStream_t stream)
 {
-  if (M <= 16) return launch_skinny<1, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, counters, stream);
-  if (M <= 32) return launch_skinny<2, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, counters, stream);
-  if (M <= 64) return launch_skinny<4, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, counters, stream);
+  const int slices = (K / 128) / S;  // of the shortest split
+#define LLMMM_GO(MBLK, D) return launch_skinny<MBLK, OUT, D>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, counters, stream)
+  if (M <= 16) {
+    if (slices >= 8) LLMMM_GO(1, 8);
+    if (slices >= 4) LLMMM_GO(1, 4);
+    LLMMM_GO(1, 2);
+  }
+  if (M <= 32) {
+    if (slices >= 4) LLMMM_GO(2, 4);
+    LLMMM_GO(2, 2);
+  }
+  if (M <= 64) {
+    if (slices >= 4) LLMMM_GO(4, 4);
+    LLMMM_GO(4, 2);
+  }
+#undef LLMMM_GO
   return hipErrorInvalidValue;
 }
 

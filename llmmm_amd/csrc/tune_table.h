@@ -1,4 +1,4 @@
-// Offline auto-tune results, compiled in.  Regenerate with `python -m llmmm_amd.tune` on an
+// Offline auto-tune results, compiled in.  Regenerate with `python -m llmmm_amd.tune --write` on an
 // MI355X; shapes that are not listed fall back to the heuristics in capi.cpp.
 // (The reference only sketches this interface: `tune(N, K)` in src/mm/fp32/impl.h:20-23.)
 #pragma once
@@ -7,7 +7,7 @@
 namespace llmmm {
 
 struct SkinnyTune {
-  int m_max;  // entry applies to M <= m_max
+  int m_max;  // entry applies to M <= m_max (entries are ordered by m_max per shape)
   int N, K;
   int split_k;
 };
@@ -16,23 +16,31 @@ struct TileTune {
   int tile;
 };
 
-// FP8 weight-streaming kernel (M <= 64): Qwen3-4B projections.
+// FP8 weight-streaming kernel (M <= 64).
 static const SkinnyTune kSkinnyTune[] = {
-  {64, 6144, 2560, 10},   // QKV
-  {64, 2560, 4096, 16},   // O
-  {64, 19456, 2560, 4},   // gate_up
-  {64, 2560, 9728, 19},   // down
+  {1, 2560, 4096, 8},
+  {16, 2560, 4096, 8},
+  {64, 2560, 4096, 8},
+  {1, 2560, 9728, 10},
+  {16, 2560, 9728, 5},
+  {64, 2560, 9728, 8},
+  {1, 6144, 2560, 5},
+  {16, 6144, 2560, 5},
+  {64, 6144, 2560, 1},
+  {1, 19456, 2560, 3},
+  {16, 19456, 2560, 1},
+  {64, 19456, 2560, 1},
 };
 
 // FP8 MFMA tile kernels (M % 128 == 0).
 static const TileTune kTileTune[] = {
-  {4096, 4096, 4096, LLMMM_TILE_256x256},
+  {4096, 4096, 4096, 0},
 };
 
 // FP16/BF16 MFMA tile kernels.
 static const TileTune kFp16TileTune[] = {
-  {4096, 4096, 4096, LLMMM_TILE_256x256},
-  {1024, 1024, 1024, LLMMM_TILE_128x128},
+  {4096, 4096, 4096, 0},
+  {1024, 1024, 1024, 3},
 };
 
 }  // namespace llmmm

@@ -1,0 +1,136 @@
+"""Offline auto-tune driver: measures every candidate configuration of the FP8 GEMM for a list
+of shapes on the GPU at hand and writes ``csrc/tune_table.h`` (compiled into ``libllmmm.so``).
+
+    python -m llmmm_amd.tune [--write] [--shapes qwen3-4b] [--m 1,16,128,2048]
+
+The reference only hints at such an interface (``tune(N, K)`` in src/mm/fp32/impl.h:20-23, a
+stub that throws).  Candidates: for M <= 64 the split-K factor of the weight-streaming kernel;
+for M % 128 == 0 the MFMA tile.  Timing: HIP events around a HIP graph of back-to-back launches
+that rotate over enough weight copies to defeat the caches (decode shapes) -- the same method
+``bench.py`` uses.  Without ``--write`` the table is only printed.
+"""
+import argparse
+import os
+import sys
+
+import torch
+
+from . import _lib, mm
+
+QWEN3_4B = {"qkv": (6144, 2560), "o": (2560, 4096), "gate_up": (19456, 2560), "down": (2560, 9728)}
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _time_ms(fn, iters, graph):
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    if graph:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(iters):
+                fn()
+        g.replay()
+        torch.cuda.synchronize()
+        e0.record()
+        g.replay()
+        e1.record()
+    else:
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def _inputs(M, N, K, copies):
+    g = torch.Generator(device="cuda").manual_seed(1)
+    X = torch.randn((M, K), generator=g, device="cuda")
+    Aq, As = mm.quantize_activation(X)
+    weights = []
+    for _ in range(copies):
+        W = torch.randn((N, K), generator=g, device="cuda") * 0.02
+        weights.append(mm.quantize_weight(W))
+        del W
+    return Aq, As, weights
+
+
+def tune_shape(M, N, K, iters=40, rotate_bytes=768 << 20, verbose=True):
+    """Returns (best_tile, best_split, {candidate: ms})."""
+    skinny = M <= 64
+    copies = max(2, -(-rotate_bytes // (N * K))) if M <= 128 else 1
+    Aq, As, weights = _inputs(M, N, K, copies)
+    Cq = torch.empty((M, N), dtype=torch.uint8, device="cuda")
+    Cs = torch.empty((N // 128, M), dtype=torch.float32, device="cuda")
+    ws = mm.make_workspace(_lib.OUT_FP8Q, M, N, K)
+    if skinny:
+        kb = K // 128
+        cands = [(_lib.TILE_SKINNY, s) for s in sorted({1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 19, 20, 24, 32, kb, kb // 2}) if 1 <= s <= min(32, kb)]
+    else:
+        cands = [(t, 1) for t, (bm, bn) in {_lib.TILE_256x256: (256, 256), _lib.TILE_128x256: (128, 256), _lib.TILE_256x128: (256, 128),
+                                             _lib.TILE_128x128: (128, 128)}.items() if M % bm == 0 and N % bn == 0]
+    results = {}
+    for tile, split in cands:
+        state = {"i": 0}
+
+        def step():
+            Bq, Bs = weights[state["i"] % copies]
+            state["i"] += 1
+            mm.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(Aq, As, Bq, Bs, Cq, Cs, M, N, K, workspace=ws, tile=tile,
+                                                                                split_k=split)
+        results[(tile, split)] = _time_ms(step, iters, graph=M <= 128)
+    best = min(results, key=results.get)
+    if verbose:
+        print("M=%d N=%d K=%d:" % (M, N, K), " ".join("%s/%d:%.1fus" % (t, s, v * 1e3) for (t, s), v in sorted(results.items())),
+              "-> best", best, flush=True)
+    return best[0], best[1], results
+
+
+def render_table(skinny_rows, tile_rows, fp16_rows):
+    out = ["// Offline auto-tune results, compiled in.  Regenerate with `python -m llmmm_amd.tune --write` on an",
+           "// MI355X; shapes that are not listed fall back to the heuristics in capi.cpp.",
+           "// (The reference only sketches this interface: `tune(N, K)` in src/mm/fp32/impl.h:20-23.)",
+           "#pragma once", '#include "kernels.h"', "", "namespace llmmm {", "",
+           "struct SkinnyTune {", "  int m_max;  // entry applies to M <= m_max (entries are ordered by m_max per shape)", "  int N, K;", "  int split_k;", "};",
+           "struct TileTune {", "  int M, N, K;", "  int tile;", "};", "",
+           "// FP8 weight-streaming kernel (M <= 64).", "static const SkinnyTune kSkinnyTune[] = {"]
+    out += ["  {%d, %d, %d, %d}," % r for r in skinny_rows]
+    out += ["};", "", "// FP8 MFMA tile kernels (M % 128 == 0).", "static const TileTune kTileTune[] = {"]
+    out += ["  {%d, %d, %d, %d}," % r for r in tile_rows]
+    out += ["};", "", "// FP16/BF16 MFMA tile kernels.", "static const TileTune kFp16TileTune[] = {"]
+    out += ["  {%d, %d, %d, %d}," % r for r in fp16_rows]
+    out += ["};", "", "}  // namespace llmmm", ""]
+    return "\n".join(out)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--write", action="store_true", help="rewrite csrc/tune_table.h with the results")
+    ap.add_argument("--m", default="1,16,64,128,2048")
+    ap.add_argument("--iters", type=int, default=40)
+    args = ap.parse_args()
+    torch.cuda.set_device(0)
+    ms = [int(x) for x in args.m.split(",")]
+    skinny_rows, tile_rows = [], [(4096, 4096, 4096, _lib.TILE_256x256)]
+    for name, (N, K) in QWEN3_4B.items():
+        for M in ms:
+            tile, split, _ = tune_shape(M, N, K, iters=args.iters)
+            if M <= 64:
+                skinny_rows.append((M, N, K, split))
+            else:
+                tile_rows.append((M, N, K, tile))
+            torch.cuda.empty_cache()
+    skinny_rows.sort(key=lambda r: (r[1], r[2], r[0]))
+    fp16_rows = [(4096, 4096, 4096, _lib.TILE_256x256), (1024, 1024, 1024, _lib.TILE_128x128)]
+    text = render_table(skinny_rows, tile_rows, fp16_rows)
+    print(text)
+    if args.write:
+        with open(os.path.join(HERE, "csrc", "tune_table.h"), "w") as f:
+            f.write(text)
+        print("wrote csrc/tune_table.h -- rebuild with `python -m llmmm_amd.build`", file=sys.stderr)
+
+
+if __name__ == "__main__":
+    main()
