@@ -26,6 +26,12 @@ import torch
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "fp8": 5000.0}  # MI355X dense MFMA, published
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE counter runs of
+# these same workloads, each scaled by the counter's reading for a 1 GiB device copy (FETCH_SIZE x 2.0 KiB,
+# WRITE_SIZE x 1.0 KiB per count).  Counters cannot be read from inside this process, so the figures are
+# carried here; the summaries they come from are kept under profiles/.
+MEASURED_TRAFFIC_BYTES = {"fp16_gemm_4096": 235.0e6, "fp8_gemm_fused_4096": 119.2e6, "decode_gate_up_m1": 51.2e6}
+
 QWEN3_4B = {"qkv": (6144, 2560), "o": (2560, 4096), "gate_up": (19456, 2560), "down": (2560, 9728)}
 
 
@@ -165,7 +171,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="fp16_gemm_4096",
                     help="fp16_gemm_4096 (headline) | fp8_gemm_fused_4096 | fp8_gemm_bf16_4096 | bf16_gemm_4096 | "
-                         "decode_<qkv|o|gate_up|down>_m<M>")
+                         "decode_<qkv|o|gate_up|down>_m<M> | copy_1g (counter calibration only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table")
     ap.add_argument("--cpu-rows", type=int, default=2048)
@@ -182,6 +188,15 @@ def main():
 
     w = args.workload
     M = N = K = 4096
+    if w == "copy_1g":
+        # Calibration aid for hardware-counter runs: a plain device copy that reads 1 GiB and writes
+        # 1 GiB per step, so a counter's reading can be scaled to bytes.
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        ms, _ = _events_ms(lambda: dst.copy_(src), args.steps, args.warmup)
+        print(json.dumps({"workload": "copy_1g", "read_bytes": 1 << 30, "write_bytes": 1 << 30, "ms_per_step": ms,
+                          "gbs": 2.0 * (1 << 30) / ms * 1e-6}))
+        return
     if w in ("fp16_gemm_4096", "bf16_gemm_4096"):
         dt = torch.float16 if w.startswith("fp16") else torch.bfloat16
         r, _ = bench_fp16(M, N, K, args.steps, args.warmup, dt)
@@ -218,8 +233,10 @@ def main():
         print("unknown workload", w, file=sys.stderr)
         sys.exit(2)
 
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(w)
+    roof["algorithmic_bytes"] = r["bytes"]
     line = {
-        "metric": "TFLOPS (% of MI355X FP8/FP16 MFMA peak) at 4096^3; HBM GB/s at M<=16 decode",
+        "metric": "TFLOPS (% of MI355X FP8/FP16 MFMA peak) at 4096\u00b3; HBM GB/s at M\u226416 decode",
         "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms"],
         "wall_ms_per_step": r["wall_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
         "data": "synthetic", "config": cfg, "roofline": roof,
