@@ -50,20 +50,49 @@ struct Fp8Tile {
   static constexpr int B_LOADS = (BN / 8) / NW;
 };
 
-// All loads of a wave share one per-lane offset: load i of the wave covers tile rows
-// 8*(wave + i*NW) .. +7, and the SWZ_ROWS16 placement only looks at row bits 0..3, so moving by
-// 8*NW (>= 16) rows changes nothing but the (wave-uniform) row base.
-template <int BM, int BN>
-__device__ __forceinline__ void fp8_issue_stage(char LLMMM_LDS* lds, const uint8_t* __restrict__ Ag,
-                                                const uint8_t* __restrict__ Bg, int lane_off, int K, int wave)
+// Operand and scale loads of the main loop are written as inline assembly, with a wave-uniform
+// base in SGPRs and one constant per-lane byte offset, and the kernel places its own s_waitcnt:
+// the compiler then never sees an LDS-direct load in flight (it would turn every wait it
+// inserts into "all loads done"), and no vector ALU work goes into addresses.
+__device__ __forceinline__ void fp8_load_lds_16B(const void* sbase, unsigned voff, unsigned lds_addr)
+{
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory");
+}
+template <int IMM>
+__device__ __forceinline__ void fp8_load_f32(float& dst, const void* sbase, unsigned voff)
+{
+  asm volatile("global_load_dword %0, %1, %2 offset:%3" : "=v"(dst) : "v"(voff), "s"(sbase), "n"(IMM) : "memory");
+}
+
+// Load i (0 .. A_LOADS + B_LOADS - 1) of a wave for one stage.  All loads of a wave share one
+// per-lane offset: load i covers tile rows 8*(wave + i*NW) .. +7, and the SWZ_ROWS16 placement
+// only looks at row bits 0..3, so moving by 8*NW (>= 16) rows changes nothing but the
+// wave-uniform row base.
+template <int BM, int BN, int I>
+__device__ __forceinline__ void fp8_issue_load(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned lane_off, int K, int wave)
 {
   typedef Fp8Tile<BM, BN> TC;
-#pragma unroll
-  for (int i = 0; i < TC::A_LOADS; ++i)
-    load_lds_16B(Ag + (size_t)(8 * TC::NW * i) * K + lane_off, lds + (wave + i * TC::NW) * 1024);
-#pragma unroll
-  for (int i = 0; i < TC::B_LOADS; ++i)
-    load_lds_16B(Bg + (size_t)(8 * TC::NW * i) * K + lane_off, lds + TC::A_BYTES + (wave + i * TC::NW) * 1024);
+  if constexpr (I < TC::A_LOADS)
+    fp8_load_lds_16B(Ag + (size_t)(8 * TC::NW * I) * K, lane_off, lds_stage + (wave + I * TC::NW) * 1024);
+  else if constexpr (I < TC::A_LOADS + TC::B_LOADS)
+    fp8_load_lds_16B(Bg + (size_t)(8 * TC::NW * (I - TC::A_LOADS)) * K, lane_off, lds_stage + TC::A_BYTES + (wave + (I - TC::A_LOADS) * TC::NW) * 1024);
+}
+template <int BM, int BN, int FIRST, int COUNT>
+__device__ __forceinline__ void fp8_issue_loads(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned lane_off, int K, int wave)
+{
+  if constexpr (COUNT > 0) {
+    fp8_issue_load<BM, BN, FIRST>(lds_stage, Ag, Bg, lane_off, K, wave);
+    fp8_issue_loads<BM, BN, FIRST + 1, COUNT - 1>(lds_stage, Ag, Bg, lane_off, K, wave);
+  }
+}
+// The slice scales of the lane's four 16-row fragments and of the wave's column group.
+__device__ __forceinline__ void fp8_issue_scales(float (&sa)[4], float& sb, const float* As_slice, unsigned row_off, const float* Bs_elem, unsigned zero)
+{
+  fp8_load_f32<0>(sa[0], As_slice, row_off);
+  fp8_load_f32<64>(sa[1], As_slice, row_off);
+  fp8_load_f32<128>(sa[2], As_slice, row_off);
+  fp8_load_f32<192>(sa[3], As_slice, row_off);
+  fp8_load_f32<0>(sb, Bs_elem, zero);
 }
 
 // 32 bytes of one row: chunk 2g at rd0 and chunk 2g+1 at rd1 (= rd0 ^ 16); `imm` selects the
@@ -79,23 +108,45 @@ __device__ __forceinline__ i32x8 fp8_read_frag(const char LLMMM_LDS* tile, int r
   return u.v;
 }
 
+// What a slice issues for its successor while it computes.
+struct Fp8Next {
+  unsigned       lds_stage;  // LDS byte address of the stage buffer to fill
+  const uint8_t* Ag;         // tile's A rows / Bt rows at the next slice's k offset
+  const uint8_t* Bg;
+  const float*   As_slice;   // As + kb_next * M
+  const float*   Bs_elem;    // &Bs[nb, kb_next]
+};
+
 // One 128-K slice of the wave's 64 x 128 sub-tile.  s[mf] = As[kb, row] * Bs[nb, kb].
-template <int BM, int BN>
+// With LOAD, the next stage's loads go out two or more per fragment step during the first four
+// steps (spread, so that no wave sits in the memory pipeline's issue queue while its matrix
+// work waits, and early enough to land within the slice), its scales during the fifth.
+template <int BM, int BN, bool LOAD>
 __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int a_rd0, int a_rd1, int b_rd0, int b_rd1,
-                                                  const float (&s)[4], f32x4 (&acc)[8][4])
+                                                  const float (&s)[4], f32x4 (&acc)[8][4], const Fp8Next& nx, unsigned lane_off,
+                                                  unsigned row_off, unsigned zero, int K, int wave, float (&sa_next)[4], float& sb_next)
 {
   typedef Fp8Tile<BM, BN> TC;
+  constexpr int           NL   = TC::A_LOADS + TC::B_LOADS;
+  constexpr int           LPG  = (NL + 3) / 4;
   const char LLMMM_LDS*   ldsA = lds;
   const char LLMMM_LDS*   ldsB = lds + TC::A_BYTES;
   i32x8                   a[4], b[2];
   f32x4                   p[2][4];
+  b[0] = fp8_read_frag(ldsB, b_rd0, b_rd1, 0);
 #pragma unroll
   for (int mf = 0; mf < 4; ++mf) a[mf] = fp8_read_frag(ldsA, a_rd0, a_rd1, mf * 2048);
-  b[0] = fp8_read_frag(ldsB, b_rd0, b_rd1, 0);
 #pragma unroll
   for (int nf = 0; nf < 8; ++nf) {
     const int cur = nf & 1;
     if (nf + 1 < 8) b[cur ^ 1] = fp8_read_frag(ldsB, b_rd0, b_rd1, (nf + 1) * 2048);
+    if constexpr (LOAD) {
+      if (nf == 0) fp8_issue_loads<BM, BN, 0, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
+      if (nf == 1) fp8_issue_loads<BM, BN, LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
+      if (nf == 2) fp8_issue_loads<BM, BN, 2 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
+      if (nf == 3) fp8_issue_loads<BM, BN, 3 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
+      if (nf == 4) fp8_issue_scales(sa_next, sb_next, nx.As_slice, row_off, nx.Bs_elem, zero);
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int mf = 0; mf < 4; ++mf) p[cur][mf] = mfma_fp8_k128(b[cur], a[mf]);
@@ -144,8 +195,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
                 int tiles_n)
 {
   typedef Fp8Tile<BM, BN> TC;
-  __shared__ __attribute__((aligned(1024))) char lds0[TC::STAGE];
-  __shared__ __attribute__((aligned(1024))) char lds1[TC::STAGE];
+  __shared__ __attribute__((aligned(1024))) char lds[2 * TC::STAGE];
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -158,7 +208,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const int KB = K >> 7;
 
   const KMajorLane lp       = kmajor_lane<SWZ_ROWS16>(wave, lane);
-  const int        lane_off = lp.row * K + lp.chunk * 16;
+  const unsigned   lane_off = (unsigned)(lp.row * K + lp.chunk * 16);
   const uint8_t*   Ag       = A + (size_t)m0 * K;
   const uint8_t*   Bg       = Bt + (size_t)n0 * K;
 
@@ -175,60 +225,95 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
     for (int mf = 0; mf < 4; ++mf) acc[nf][mf] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // scales: As[kb*M + m] for the lane's 4 rows, Bs[(n/128)*KB + kb] for the wave's column group
-  const int    mrow = m0 + wm * 64 + (lane & 15);
-  const float* Asp  = As + mrow;
-  const float* Bsp  = Bs + (size_t)((n0 >> 7) + wn) * KB;
-  float        sa_next[4], sb_next;
-#pragma unroll
-  for (int mf = 0; mf < 4; ++mf) sa_next[mf] = Asp[mf * 16];
-  sb_next = Bsp[0];
+  const int      mrow    = m0 + wm * 64 + (lane & 15);
+  const unsigned row_off = (unsigned)mrow * 4u;
+  const float*   Bsp     = Bs + (size_t)((n0 >> 7) + wn) * KB;
+  unsigned       zero    = 0;
+  asm volatile("" : "+v"(zero));  // a VGPR holding 0: the per-lane offset of the wave-uniform Bs load
+  float sa_next[4], sb_next;
 
-  char LLMMM_LDS* const s0 = (char LLMMM_LDS*)lds0;
-  char LLMMM_LDS* const s1 = (char LLMMM_LDS*)lds1;
+  const unsigned lds0 = (unsigned)(size_t)(char LLMMM_LDS*)lds;
+  char LLMMM_LDS* const s0 = (char LLMMM_LDS*)lds;
 
-  fp8_issue_stage<BM, BN>(s0, Ag, Bg, lane_off, K, wave);
-  for (int kb = 0; kb < KB; kb += 2) {
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      const int kc = kb + half;
-      if (kc < KB) {
-        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): this wave's LDS-direct loads have landed
-        __syncthreads();
-        float s[4];
-#pragma unroll
-        for (int mf = 0; mf < 4; ++mf) s[mf] = sa_next[mf] * sb_next;
-        if (kc + 1 < KB) {
-          fp8_issue_stage<BM, BN>(half ? s0 : s1, Ag + (size_t)(kc + 1) * 128, Bg + (size_t)(kc + 1) * 128, lane_off, K, wave);
-#pragma unroll
-          for (int mf = 0; mf < 4; ++mf) sa_next[mf] = Asp[(size_t)(kc + 1) * M + mf * 16];
-          sb_next = Bsp[kc + 1];
-        }
-        fp8_compute_stage<BM, BN>(half ? s1 : s0, a_rd0, a_rd1, b_rd0, b_rd1, s, acc);
-      }
-    }
+  fp8_issue_loads<BM, BN, 0, TC::A_LOADS + TC::B_LOADS>(lds0, Ag, Bg, lane_off, K, wave);
+  fp8_issue_scales(sa_next, sb_next, As, row_off, Bsp, zero);
+
+  // One slice: wait for this wave's loads of the slice (all of them were issued at least half a
+  // slice ago), meet the other waves, then compute it while the loads of the next one go out.
+#define LLMMM_FP8_SLICE(LOAD, CUR, NXT_LDS, KC)                                                                                   \
+  {                                                                                                                               \
+    wait_vmcnt<0>();                                                                                                              \
+    asm volatile("" : "+v"(sa_next[0]), "+v"(sa_next[1]), "+v"(sa_next[2]), "+v"(sa_next[3]), "+v"(sb_next));                     \
+    __syncthreads();                                                                                                              \
+    float s[4];                                                                                                                   \
+    _Pragma("unroll") for (int mf = 0; mf < 4; ++mf) s[mf] = sa_next[mf] * sb_next;                                               \
+    Fp8Next nx;                                                                                                                   \
+    nx.lds_stage = NXT_LDS;                                                                                                       \
+    nx.Ag        = Ag + (size_t)((KC) + 1) * 128;                                                                                 \
+    nx.Bg        = Bg + (size_t)((KC) + 1) * 128;                                                                                 \
+    nx.As_slice  = As + (size_t)((KC) + 1) * M;                                                                                   \
+    nx.Bs_elem   = Bsp + (KC) + 1;                                                                                                \
+    fp8_compute_stage<BM, BN, LOAD>(CUR, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, row_off, zero, K, wave, sa_next,       \
+                                    sb_next);                                                                                     \
   }
 
-  // ---- epilogue.  lane (g, i): row m = .. + mf*16 + i, columns n = nf*16 + 4g + r
-  const int ncol = n0 + wn * 128 + 4 * g;
+  unsigned cur = 0;  // byte offset of the stage being computed: 0 or STAGE
+  for (int kc = 0; kc < KB - 1; ++kc) {
+    LLMMM_FP8_SLICE(true, s0 + cur, lds0 + (TC::STAGE - cur), kc)
+    cur = TC::STAGE - cur;
+  }
+  LLMMM_FP8_SLICE(false, s0 + cur, 0u, KB - 1)
+#undef LLMMM_FP8_SLICE
+
+  // ---- epilogue.  lane (g, i): row m = .. + mf*16 + i, columns n = nf*16 + 4g + r.
+  // Written straight from this layout, one store instruction would touch 16 rows with 16..64
+  // bytes each; the memory pipeline pays per row segment, not per byte.  So every wave first
+  // lays its 64 x 128 result out row-major in a private 16 KB piece of the (now idle) operand
+  // buffers -- 16-byte chunks XOR-ed with row bits so that neither the writes nor the
+  // ds_read_b128 reads conflict -- and stores it back out 16 bytes per lane, whole rows at a time.
+  __syncthreads();  // every wave is done reading the last operand stage
+  char LLMMM_LDS* const stg  = s0 + wave * 16384;
+  const int             row0 = m0 + wm * 64;
+  const int             col0 = n0 + wn * 128;
+  const int             li   = lane & 15;
   if constexpr (OUT == OUT_F32) {
     float* C = (float*)Cv;
 #pragma unroll
-    for (int mf = 0; mf < 4; ++mf)
+    for (int h = 0; h < 2; ++h) {  // 32 rows x 512 B per round
 #pragma unroll
-      for (int nf = 0; nf < 8; ++nf) *(f32x4*)(C + (size_t)(mrow + mf * 16) * N + ncol + nf * 16) = acc[nf][mf];
+      for (int mfl = 0; mfl < 2; ++mfl) {
+        const int r = mfl * 16 + li;
+#pragma unroll
+        for (int nf = 0; nf < 8; ++nf) *(f32x4 LLMMM_LDS*)(stg + r * 512 + (((nf * 4 + g) ^ ((r & 7) << 1)) << 4)) = acc[nf][2 * h + mfl];
+      }
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int   r = 2 * j + (lane >> 5), c = lane & 31;
+        const f32x4 v = *(const f32x4 LLMMM_LDS*)(stg + r * 512 + ((c ^ ((r & 7) << 1)) << 4));
+        *(f32x4*)(C + (size_t)(row0 + 32 * h + r) * N + col0 + c * 4) = v;
+      }
+    }
   }
   else if constexpr (OUT == OUT_BF16) {
     __bf16* C = (__bf16*)Cv;
     typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int mf = 0; mf < 4; ++mf)
+    for (int mf = 0; mf < 4; ++mf) {
+      const int r = mf * 16 + li;
 #pragma unroll
       for (int nf = 0; nf < 8; ++nf) {
         bf16x4 o;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[nf][mf][r];
-        *(bf16x4*)(C + (size_t)(mrow + mf * 16) * N + ncol + nf * 16) = o;
+        for (int q = 0; q < 4; ++q) o[q] = (__bf16)acc[nf][mf][q];
+        *(bf16x4 LLMMM_LDS*)(stg + r * 256 + (((nf * 2 + (g >> 1)) ^ (r & 15)) << 4) + 8 * (g & 1)) = o;
       }
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int   r = 4 * j + (lane >> 4), c = lane & 15;
+      const i32x4 v = *(const i32x4 LLMMM_LDS*)(stg + r * 256 + ((c ^ (r & 15)) << 4));
+      *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 8) = v;
+    }
   }
   else {
     uint8_t* C = (uint8_t*)Cv;
@@ -238,18 +323,24 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
 #pragma unroll
       for (int nf = 0; nf < 8; ++nf)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) amax = fmaxf(amax, __builtin_fabsf(acc[nf][mf][r]));
+        for (int q = 0; q < 4; ++q) amax = fmaxf(amax, __builtin_fabsf(acc[nf][mf][q]));
       amax              = wave_xor_max(amax, 16);
       amax              = wave_xor_max(amax, 32);
       const float scale = amax / 448.f;
       const float inv   = amax > 0.f ? 448.f / amax : 0.f;
-      uint8_t*    crow  = C + (size_t)(mrow + mf * 16) * N + ncol;
+      const int   r     = mf * 16 + li;
 #pragma unroll
       for (int nf = 0; nf < 8; ++nf) {
-        const f32x4 v                   = acc[nf][mf];
-        *(uint32_t*)(crow + nf * 16) = pack_e4m3x4(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+        const f32x4 v = acc[nf][mf];
+        *(uint32_t LLMMM_LDS*)(stg + r * 128 + ((nf ^ ((r >> 1) & 7)) << 4) + 4 * g) = pack_e4m3x4(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
       }
-      if (g == 0) Cs[(size_t)((n0 >> 7) + wn) * M + mrow + mf * 16] = scale;
+      if (g == 0) Cs[(size_t)((n0 >> 7) + wn) * M + row0 + r] = scale;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int   r = 8 * j + (lane >> 3), c = lane & 7;
+      const i32x4 v = *(const i32x4 LLMMM_LDS*)(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
+      *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 16) = v;
     }
   }
 }
