@@ -25,6 +25,7 @@ import torch
 
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "fp8": 5000.0}  # MI355X dense MFMA, published
 PEAK_HBM_GBS = 8000.0
+PREHEAT_S = 0.25  # seconds of untimed launches before the warm-up steps of every measurement
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE counter runs of
 # these same workloads, each scaled by the counter's reading for a 1 GiB device copy (FETCH_SIZE x 2.0 KiB,
@@ -40,6 +41,13 @@ def _events_ms(fn, steps, warmup, graph=False):
     every launch below is enqueued on).  With graph=True the `steps` launches are captured into
     one HIP graph and replayed, so that microsecond kernels are timed back-to-back on the GPU
     instead of at the pace of the Python launch loop."""
+    # Untimed pre-heat: the GPU's clocks take tens of milliseconds of sustained load to settle, far
+    # longer than a handful of warm-up launches of a ~100 us kernel; time the settled state.
+    t_heat = time.perf_counter()
+    while time.perf_counter() - t_heat < PREHEAT_S:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()

@@ -60,9 +60,16 @@ struct Fp16Tile {
 // Issue the LDS-direct loads of one stage.  `kleft` = K - k0 (elements still to go); a stage
 // whose K range is cut short zero-fills the missing part so that the MFMAs need no masking.
 // All loads of a wave share one per-lane offset: they differ by a wave-uniform row (or k) step
-// that the swizzles do not see.
+// that the swizzles do not see.  The loads are inline assembly with the wave-uniform part of the
+// address in SGPRs: no vector ALU work goes into addresses, and the compiler -- which would
+// turn every wait it inserts into "all loads done" while it knows of an LDS-direct load in
+// flight -- never sees them; the kernel places the s_waitcnt vmcnt itself.
+__device__ __forceinline__ void sload_lds_16B(const void* sbase, unsigned voff, unsigned lds_addr)
+{
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory");
+}
 template <typename T, int BM, int BN, bool B_NK, bool KTAIL>
-__device__ __forceinline__ void fp16_issue_stage(char LLMMM_LDS* lds, const T* __restrict__ Ag, const T* __restrict__ Bg,
+__device__ __forceinline__ void fp16_issue_stage(char LLMMM_LDS* lds, unsigned lds_addr, const T* __restrict__ Ag, const T* __restrict__ Bg,
                                                  unsigned a_off, int a_k, unsigned b_off, int b_k, int K, int N, int wave,
                                                  int lane, int kleft)
 {
@@ -74,7 +81,7 @@ __device__ __forceinline__ void fp16_issue_stage(char LLMMM_LDS* lds, const T* _
   for (int i = 0; i < TC::A_LOADS; ++i) {
     char LLMMM_LDS* dst = lds + (wave + i * TC::NW) * 1024;
     if (full || a_k < kleft)
-      load_lds_16B(Ag + (size_t)(TC::ROWS_PER_LOAD * i) * K + a_off, dst);
+      sload_lds_16B(Ag + (size_t)(TC::ROWS_PER_LOAD * i) * K, a_off * 2u, lds_addr + (wave + i * TC::NW) * 1024);
     else
       *(i32x4 LLMMM_LDS*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
   }
@@ -84,13 +91,13 @@ __device__ __forceinline__ void fp16_issue_stage(char LLMMM_LDS* lds, const T* _
     char LLMMM_LDS* dst = ldsB + (wave + i * TC::NW) * 1024;
     if constexpr (B_NK) {
       if (full || b_k < kleft)
-        load_lds_16B(Bg + (size_t)(TC::ROWS_PER_LOAD * i) * K + b_off, dst);
+        sload_lds_16B(Bg + (size_t)(TC::ROWS_PER_LOAD * i) * K, b_off * 2u, lds_addr + TC::A_BYTES + (wave + i * TC::NW) * 1024);
       else
         *(i32x4 LLMMM_LDS*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
     }
     else {
       if (full || b_k + TC::B_KROWS_PER_LOAD * i < kleft)
-        load_lds_16B(Bg + (size_t)(TC::B_KROWS_PER_LOAD * i) * N + b_off, dst);
+        sload_lds_16B(Bg + (size_t)(TC::B_KROWS_PER_LOAD * i) * N, b_off * 2u, lds_addr + TC::A_BYTES + (wave + i * TC::NW) * 1024);
       else
         *(i32x4 LLMMM_LDS*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
     }
@@ -143,12 +150,7 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
 {
   typedef Fp16Tile<T, BM, BN, B_NK> TC;
   typedef typename Mfma16<T>::vec   vec;
-  // four distinct arrays (not one indexed array) so that the compiler can tell which stage an
-  // access touches and does not serialise the LDS-direct loads against unrelated ds_reads
-  __shared__ __attribute__((aligned(1024))) char lds0[TC::STAGE];
-  __shared__ __attribute__((aligned(1024))) char lds1[TC::STAGE];
-  __shared__ __attribute__((aligned(1024))) char lds2[TC::STAGE];
-  __shared__ __attribute__((aligned(1024))) char lds3[TC::STAGE];
+  __shared__ __attribute__((aligned(1024))) char lds_raw[4 * TC::STAGE];  // the ring of four stages
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -206,10 +208,13 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
   const int    full_stages = K / TC::BK;
   const size_t b_step      = B_NK ? (size_t)TC::BK : (size_t)TC::BK * N;
 
-  char LLMMM_LDS* const ring[4] = {(char LLMMM_LDS*)lds0, (char LLMMM_LDS*)lds1, (char LLMMM_LDS*)lds2, (char LLMMM_LDS*)lds3};
+  char LLMMM_LDS* const lds      = (char LLMMM_LDS*)lds_raw;
+  char LLMMM_LDS* const ring[4]  = {lds, lds + TC::STAGE, lds + 2 * TC::STAGE, lds + 3 * TC::STAGE};
+  const unsigned        lds_base = (unsigned)(size_t)lds;  // the same buffers as LDS byte addresses, for the loader
+  const unsigned ring_addr[4]    = {lds_base, lds_base + TC::STAGE, lds_base + 2 * TC::STAGE, lds_base + 3 * TC::STAGE};
 
 #define LLMMM_ISSUE(stage, buf)                                                                                              \
-  fp16_issue_stage<T, BM, BN, B_NK, KTAIL>(ring[buf], Ag + (size_t)(stage) * TC::BK, Bg + (size_t)(stage) * b_step, a_off, a_k, b_off, \
+  fp16_issue_stage<T, BM, BN, B_NK, KTAIL>(ring[buf], ring_addr[buf], Ag + (size_t)(stage) * TC::BK, Bg + (size_t)(stage) * b_step, a_off, a_k, b_off, \
                                     b_k, K, N, wave, lane, K - (stage) * TC::BK)
 
   // prologue: stages 0..2 in flight, stage 0 landed and published, then stage 3 behind the barrier
@@ -271,24 +276,39 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
 #undef LLMMM_STAGE
 #undef LLMMM_ISSUE
 
-  // ---- epilogue: lane holds, for row m = ..+lane%32, the columns 8*(r/4) + 4*(lane/32) + r%4
-  const int m = m0 + wm * 64 + (lane & 31);
+  // ---- epilogue: lane holds, for row m = ..+lane%32, the columns 8*(r/4) + 4*(lane/32) + r%4.
+  // Stored straight from this layout, one instruction would write 16 bytes to each of 32 rows,
+  // and the memory pipeline pays per row segment.  Instead every wave lays its 64 x 128 result
+  // out row-major (256-byte rows, 16-byte chunks XOR-ed with the row so that the ds_read_b128
+  // below is conflict-free) in a private 16 KB piece of the ring and stores whole rows, 16
+  // bytes per lane.  Behind the last stage's barrier no wave reads operands any more and every
+  // load has landed, so the ring is free.
+  {
+    typedef T             tx4 __attribute__((ext_vector_type(4)));
+    char LLMMM_LDS* const stg = lds + wave * 16384;
 #pragma unroll
-  for (int mf = 0; mf < 2; ++mf) {
-    T* crow = C + (size_t)(m + mf * 32) * N + n0 + wn * 128 + 4 * hi;
+    for (int mf = 0; mf < 2; ++mf) {
+      const int r = mf * 32 + (lane & 31);
 #pragma unroll
-    for (int nf = 0; nf < 4; ++nf)
+      for (int nf = 0; nf < 4; ++nf)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        typedef T     tx4 __attribute__((ext_vector_type(4)));
-        const f32x16& v = acc[nf][mf];
-        tx4           o;
-        o[0] = (T)v[4 * q + 0];
-        o[1] = (T)v[4 * q + 1];
-        o[2] = (T)v[4 * q + 2];
-        o[3] = (T)v[4 * q + 3];
-        *(tx4*)(crow + nf * 32 + q * 8) = o;
-      }
+        for (int q = 0; q < 4; ++q) {
+          const f32x16& v = acc[nf][mf];
+          tx4           o;
+          o[0] = (T)v[4 * q + 0];
+          o[1] = (T)v[4 * q + 1];
+          o[2] = (T)v[4 * q + 2];
+          o[3] = (T)v[4 * q + 3];
+          *(tx4 LLMMM_LDS*)(stg + r * 256 + (((nf * 4 + q) ^ (r & 15)) << 4) + 8 * hi) = o;
+        }
+    }
+    T* cbase = C + (size_t)(m0 + wm * 64) * N + n0 + wn * 128;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int   r = 4 * j + (lane >> 4), ch = lane & 15;
+      const i32x4 v = *(const i32x4 LLMMM_LDS*)(stg + r * 256 + ((ch ^ (r & 15)) << 4));
+      *(i32x4*)(cbase + (size_t)r * N + ch * 8) = v;
+    }
   }
 }
 

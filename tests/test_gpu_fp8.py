@@ -58,6 +58,15 @@ def test_tile_kernels_against_oracle(lib, oracle, tile):
     _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, tile=TILES[tile]), ref, "tile " + tile)
 
 
+@pytest.mark.parametrize("K", [128, 256, 384, 512, 640])
+def test_short_k(lib, oracle, K):
+    """1 to 5 slices through the 256x256 tile kernel: prologue-only, odd and even slice counts."""
+    M, N = 256, 512
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=40 + K)
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, tile=TILES["256x256"]), ref, "K=%d" % K)
+
+
 def test_single_slice(lib, oracle):
     Aq, As, Bq, Bs = fp8_inputs(oracle, 128, 128, 128, seed=11)
     _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs), oracle.fp8_gemm(Aq, As, Bq, Bs), "K=128")
