@@ -60,7 +60,7 @@ extern "C" {
 #define LLMMM_TILE_128x256 1
 #define LLMMM_TILE_256x128 2
 #define LLMMM_TILE_128x128 3
-#define LLMMM_TILE_SKINNY 8 /* M <= 64 weight-streaming kernel */
+#define LLMMM_TILE_SKINNY 8 /* M <= 128 weight-streaming kernel */
 
 typedef struct llmmm_gemm_cfg {
   int tile;
@@ -85,8 +85,8 @@ LLMMM_API int llmmm_fp16_gemm_ex(int dtype, const void* A, const void* B, void* 
  *                                                                     examples/005.fp8.mm.opt.cu:468-508.
  * C is float* (OUT_F32), bf16* (OUT_BF16) or e4m3 uint8_t* (OUT_FP8Q); Cs is only used (and
  * required) for OUT_FP8Q.  N % 128 == 0 and K % 128 == 0 are required.  M % 128 == 0 runs the
- * MFMA tile kernels (the reference's domain); 1 <= M <= 64 runs the weight-streaming kernel,
- * which may split K: then `workspace` must hold llmmm_fp8_gemm_workspace() bytes, prepared once
+ * MFMA tile kernels (the reference's domain); 1 <= M <= 128 runs the weight-streaming kernel
+ * (M = 128: unless a tile is requested through llmmm_fp8_gemm_ex), which may split K: then `workspace` must hold llmmm_fp8_gemm_workspace() bytes, prepared once
  * with llmmm_workspace_init().  With workspace == NULL no split is used.  Other M are rejected
  * as not aligned.  Calls that share a workspace must be ordered on one stream. */
 LLMMM_API int llmmm_fp8_gemm(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,

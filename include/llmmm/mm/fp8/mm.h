@@ -12,7 +12,7 @@
 //
 // fp8_t stands for the reference's __nv_fp8_e4m3: one byte of OCP E4M3.  The launchers follow the
 // reference's rule M % 128 == 0, N % 128 == 0, K % 128 == 0 (examples/005.fp8.mm.cu:2490-2492) and
-// additionally accept 1 <= M <= 64 (decode), which the reference does not cover; small-M calls run
+// additionally accept 1 <= M <= 128 (decode), which the reference does not cover; small-M calls run
 // without split-K here because the reference signature has no workspace -- use llmmm_fp8_gemm()
 // with a workspace for the split-K path.
 #pragma once

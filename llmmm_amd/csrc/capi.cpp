@@ -30,6 +30,8 @@ constexpr size_t WS_HEADER_BYTES = 4096;  // arrival counters: one uint32 per 12
 constexpr int    MAX_SPLIT_K     = 32;
 constexpr int    NUM_CUS         = 256;   // MI355X
 
+constexpr int SKINNY_MAX_M = 128;  // rows the weight-streaming kernel takes (two groups of 64)
+
 int max_split_for(int K) { return (K / 128) < MAX_SPLIT_K ? (K / 128) : MAX_SPLIT_K; }
 
 // Split count for the weight-streaming kernel when the tune table has no entry: about one
@@ -38,9 +40,9 @@ int max_split_for(int K) { return (K / 128) < MAX_SPLIT_K ? (K / 128) : MAX_SPLI
 // rows (the fp32 partial tiles grow with M).
 int heuristic_split(int M, int N, int K)
 {
-  const int groups = N / 128, kb = K / 128;
+  const int groups = (N / 128) * ((M + 63) / 64), kb = K / 128;
   int       s      = (240 + groups / 2) / groups;
-  if (M > 16) s = (s + 1) / 2;
+  if (M > 16 && M <= 64) s = (s + 1) / 2;
   if (s > kb / 2) s = kb / 2;
   if (s > MAX_SPLIT_K) s = MAX_SPLIT_K;
   if (s < 1) s = 1;
@@ -74,6 +76,23 @@ int heuristic_tile(int M, int N)
   return best;
 }
 
+constexpr int MAX_TILE_SPLIT = 8;
+
+bool tile_dims(int tile, int& bm, int& bn);
+
+// Split-K factor for the MFMA tile kernels: only when the tiles alone leave most of the chip
+// idle; about one workgroup per CU, every split at least two slices long.
+int heuristic_tile_split(int tile, int M, int N, int K)
+{
+  int bm, bn;
+  if (!tile_dims(tile, bm, bn)) return 1;
+  const int tiles = (M / bm) * (N / bn), kb = K / 128;
+  int       s     = NUM_CUS / tiles;
+  if (s > kb / 2) s = kb / 2;
+  if (s > MAX_TILE_SPLIT) s = MAX_TILE_SPLIT;
+  return s < 2 ? 1 : s;
+}
+
 bool tile_dims(int tile, int& bm, int& bn)
 {
   switch (tile) {
@@ -89,7 +108,7 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
 {
   if (M <= 0 || N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "M, N and K must be positive (got %d, %d, %d)", M, N, K);
   if (N % 128 || K % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
-  if (M <= 64) {
+  if (M <= SKINNY_MAX_M && M % 128) {  // M = 128 is better served by a split tile kernel
     cfg->tile    = LLMMM_TILE_SKINNY;
     cfg->split_k = 0;
     for (const auto& e : llmmm::kSkinnyTune)
@@ -102,13 +121,19 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
   }
   if (M % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
   cfg->tile    = -1;
-  cfg->split_k = 1;
+  cfg->split_k = 0;
   for (const auto& e : llmmm::kTileTune)
     if (e.M == M && e.N == N && e.K == K) {
-      cfg->tile = e.tile;
+      cfg->tile    = e.tile;
+      cfg->split_k = e.split_k;
       break;
     }
   if (cfg->tile < 0) cfg->tile = heuristic_tile(M, N);
+  if (cfg->tile == LLMMM_TILE_SKINNY) {
+    if (cfg->split_k <= 0) cfg->split_k = heuristic_split(M, N, K);
+  }
+  else if (cfg->split_k <= 0)
+    cfg->split_k = heuristic_tile_split(cfg->tile, M, N, K);
   return LLMMM_OK;
 }
 
@@ -177,8 +202,13 @@ int llmmm_fp8_gemm_query(int out_kind, int M, int N, int K, llmmm_gemm_cfg* cfg)
 size_t llmmm_fp8_gemm_workspace(int out_kind, int M, int N, int K)
 {
   (void)out_kind;
-  if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128 || M > 64) return 0;
-  return WS_HEADER_BYTES + (size_t)max_split_for(K) * M * N * sizeof(float);
+  if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
+  llmmm_gemm_cfg cfg;
+  if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
+  // the weight-streaming kernel: room for any split the tuner may try; tile kernels: the split chosen
+  const int s = cfg.tile == LLMMM_TILE_SKINNY ? max_split_for(K) : cfg.split_k;
+  if (s <= 1) return 0;
+  return WS_HEADER_BYTES + (size_t)s * M * N * sizeof(float);
 }
 
 int llmmm_workspace_init(void* workspace, size_t workspace_bytes, void* stream)
@@ -202,14 +232,14 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
   if (!aligned16(A) || !aligned16(Bt) || !aligned16(C)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
   if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
-  if (N / 128 > (int)(WS_HEADER_BYTES / 4)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "N too large");
+  if ((N / 128) * 2 > (int)(WS_HEADER_BYTES / 4)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "N too large");
   if (user) {
     if (user->tile != LLMMM_TILE_AUTO) cfg.tile = user->tile;
     if (user->split_k > 0) cfg.split_k = user->split_k;
   }
   hipError_t e;
   if (cfg.tile == LLMMM_TILE_SKINNY) {
-    if (M > 64) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the skinny kernel handles M <= 64");
+    if (M > SKINNY_MAX_M) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the weight-streaming kernel handles M <= %d", SKINNY_MAX_M);
     int split = cfg.split_k;
     if (split > max_split_for(K)) split = max_split_for(K);
     if (split < 1) split = 1;
@@ -229,7 +259,25 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
     int bm, bn;
     if (!tile_dims(cfg.tile, bm, bn)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown tile id %d", cfg.tile);
     if (M % bm || N % bn) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
-    e = llmmm::fp8_gemm_launch(out_kind, cfg.tile, A, As, Bt, Bs, C, Cs, M, N, K, (hipStream_t)stream);
+    if (user && user->tile != LLMMM_TILE_AUTO && user->split_k <= 0) cfg.split_k = heuristic_tile_split(cfg.tile, M, N, K);
+    int split = cfg.split_k;
+    if (split > K / 128) split = K / 128;
+    if (split > MAX_SPLIT_K) split = MAX_SPLIT_K;
+    if (split < 1 || !workspace) split = 1;  // documented: no workspace, no split
+    float* planes = nullptr;
+    if (split > 1 && !(user && user->split_k > 0)) {
+      // a split the library chose itself shrinks to what the caller's workspace holds
+      const size_t plane = (size_t)M * N * sizeof(float);
+      const size_t room  = workspace_bytes > WS_HEADER_BYTES ? (workspace_bytes - WS_HEADER_BYTES) / plane : 0;
+      if ((size_t)split > room) split = room < 2 ? 1 : (int)room;
+    }
+    if (split > 1) {
+      const size_t need = WS_HEADER_BYTES + (size_t)split * M * N * sizeof(float);
+      if (workspace_bytes < need) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace_bytes, split, need);
+      if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+      planes = (float*)((char*)workspace + WS_HEADER_BYTES);
+    }
+    e = llmmm::fp8_gemm_launch(out_kind, cfg.tile, A, As, Bt, Bs, C, Cs, M, N, K, split, planes, (hipStream_t)stream);
   }
   if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "fp8 gemm launch: %s", hipGetErrorString(e));
   return LLMMM_OK;

@@ -206,11 +206,18 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
   const int KB = K >> 7;
+  // split-K: gridDim.y workgroups share a tile, each taking a contiguous run of slices and (the
+  // host only splits the fp32 instantiation) writing its partial sums to its own [M, N] plane
+  // of C; a second kernel adds the planes in order.  gridDim.y == 1: the whole K range.
+  const int S   = gridDim.y;
+  const int sp  = blockIdx.y;
+  const int kb0 = sp * KB / S;
+  const int KBL = (sp + 1) * KB / S - kb0;  // slices of this workgroup (>= 1: the host keeps S <= KB)
 
   const KMajorLane lp       = kmajor_lane<SWZ_ROWS16>(wave, lane);
   const unsigned   lane_off = (unsigned)(lp.row * K + lp.chunk * 16);
-  const uint8_t*   Ag       = A + (size_t)m0 * K;
-  const uint8_t*   Bg       = Bt + (size_t)n0 * K;
+  const uint8_t*   Ag       = A + (size_t)m0 * K + (size_t)kb0 * 128;
+  const uint8_t*   Bg       = Bt + (size_t)n0 * K + (size_t)kb0 * 128;
 
   // operand reads: lane = (g = lane/16, i = lane%16) takes row i of a 16-row fragment and the
   // 32 bytes k = 32g .. 32g+31 (chunks 2g and 2g+1)
@@ -227,7 +234,8 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   // scales: As[kb*M + m] for the lane's 4 rows, Bs[(n/128)*KB + kb] for the wave's column group
   const int      mrow    = m0 + wm * 64 + (lane & 15);
   const unsigned row_off = (unsigned)mrow * 4u;
-  const float*   Bsp     = Bs + (size_t)((n0 >> 7) + wn) * KB;
+  const float*   Bsp     = Bs + (size_t)((n0 >> 7) + wn) * KB + kb0;
+  const float*   Asl     = As + (size_t)kb0 * M;
   unsigned       zero    = 0;
   asm volatile("" : "+v"(zero));  // a VGPR holding 0: the per-lane offset of the wave-uniform Bs load
   float sa_next[4], sb_next;
@@ -236,7 +244,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   char LLMMM_LDS* const s0 = (char LLMMM_LDS*)lds;
 
   fp8_issue_loads<BM, BN, 0, TC::A_LOADS + TC::B_LOADS>(lds0, Ag, Bg, lane_off, K, wave);
-  fp8_issue_scales(sa_next, sb_next, As, row_off, Bsp, zero);
+  fp8_issue_scales(sa_next, sb_next, Asl, row_off, Bsp, zero);
 
   // One slice: wait for this wave's loads of the slice (all of them were issued at least half a
   // slice ago), meet the other waves, then compute it while the loads of the next one go out.
@@ -251,18 +259,18 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
     nx.lds_stage = NXT_LDS;                                                                                                       \
     nx.Ag        = Ag + (size_t)((KC) + 1) * 128;                                                                                 \
     nx.Bg        = Bg + (size_t)((KC) + 1) * 128;                                                                                 \
-    nx.As_slice  = As + (size_t)((KC) + 1) * M;                                                                                   \
+    nx.As_slice  = Asl + (size_t)((KC) + 1) * M;                                                                                  \
     nx.Bs_elem   = Bsp + (KC) + 1;                                                                                                \
     fp8_compute_stage<BM, BN, LOAD>(CUR, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, row_off, zero, K, wave, sa_next,       \
                                     sb_next);                                                                                     \
   }
 
   unsigned cur = 0;  // byte offset of the stage being computed: 0 or STAGE
-  for (int kc = 0; kc < KB - 1; ++kc) {
+  for (int kc = 0; kc < KBL - 1; ++kc) {
     LLMMM_FP8_SLICE(true, s0 + cur, lds0 + (TC::STAGE - cur), kc)
     cur = TC::STAGE - cur;
   }
-  LLMMM_FP8_SLICE(false, s0 + cur, 0u, KB - 1)
+  LLMMM_FP8_SLICE(false, s0 + cur, 0u, KBL - 1)
 #undef LLMMM_FP8_SLICE
 
   // ---- epilogue.  lane (g, i): row m = .. + mf*16 + i, columns n = nf*16 + 4g + r.
@@ -277,7 +285,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const int             col0 = n0 + wn * 128;
   const int             li   = lane & 15;
   if constexpr (OUT == OUT_F32) {
-    float* C = (float*)Cv;
+    float* C = (float*)Cv + (size_t)sp * M * N;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {  // 32 rows x 512 B per round
 #pragma unroll
@@ -345,38 +353,104 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   }
 }
 
+// Second kernel of a split-K run: C = epilogue(sum over s = 0..S-1, in that order, of plane s).
+// Half a wavefront (32 lanes x 4 columns) owns one row of one 128-column group, which is also
+// one quantisation group of the fused output; a workgroup of 256 threads covers 8 rows per step.
+// The arithmetic of each epilogue is that of fp8_gemm_kernel, so a split run only differs from an
+// unsplit one by the (fixed) order of the fp32 additions.
+template <int OUT>
+__global__ void __launch_bounds__(256)
+fp8_splitk_reduce_kernel(const float* __restrict__ planes, int S, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N,
+                         int rows_per_wg)
+{
+  const int    tid   = threadIdx.x;
+  const int    sub   = tid >> 5;
+  const int    l32   = tid & 31;
+  const int    nb    = blockIdx.x;
+  const int    n     = nb * 128 + l32 * 4;
+  const int    mbeg  = blockIdx.y * rows_per_wg;
+  const int    mend  = min(M, mbeg + rows_per_wg);
+  const size_t plane = (size_t)M * N;
+  for (int m = mbeg + sub; m < mend; m += 8) {
+    const float* src = planes + (size_t)m * N + n;
+    f32x4        v   = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < S; s0 += 4) {  // four planes in flight, added in order
+      f32x4 t[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) t[u] = __builtin_nontemporal_load((const f32x4*)(src + (size_t)min(s0 + u, S - 1) * plane));
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (s0 + u < S) v += t[u];
+    }
+    if constexpr (OUT == OUT_F32) {
+      *(f32x4*)((float*)Cv + (size_t)m * N + n) = v;
+    }
+    else if constexpr (OUT == OUT_BF16) {
+      typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+      bf16x4         o;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) o[q] = (__bf16)v[q];
+      *(bf16x4*)((__bf16*)Cv + (size_t)m * N + n) = o;
+    }
+    else {
+      float a = fmaxf(fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1])), fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
+      a       = wave_xor_max(a, 1);
+      a       = wave_xor_max(a, 2);
+      a       = wave_xor_max(a, 4);
+      a       = wave_xor_max(a, 8);
+      a       = wave_xor_max(a, 16);
+      const float scale = a / 448.f;
+      const float inv   = a > 0.f ? 448.f / a : 0.f;
+      *(uint32_t*)((uint8_t*)Cv + (size_t)m * N + n) = pack_e4m3x4(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+      if (l32 == 0) Cs[(size_t)nb * M + m] = scale;
+    }
+  }
+}
+
 // --------------------------------------------------------------------------------------------- host
 template <int BM, int BN, int OUT>
 static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N,
-                             int K, hipStream_t stream)
+                             int K, int S, float* planes, hipStream_t stream)
 {
   typedef Fp8Tile<BM, BN> TC;
   const int tiles_m = M / BM, tiles_n = N / BN;
-  hipLaunchKernelGGL((fp8_gemm_kernel<BM, BN, OUT>), dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As,
-                     (const uint8_t*)Bt, Bs, C, Cs, M, N, K, tiles_m, tiles_n);
+  if (S <= 1) {
+    hipLaunchKernelGGL((fp8_gemm_kernel<BM, BN, OUT>), dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As,
+                       (const uint8_t*)Bt, Bs, C, Cs, M, N, K, tiles_m, tiles_n);
+    return hipGetLastError();
+  }
+  // split-K: S partial planes from the fp32 instantiation, then the ordered sum + epilogue
+  hipLaunchKernelGGL((fp8_gemm_kernel<BM, BN, OUT_F32>), dim3(tiles_m * tiles_n, S), dim3(TC::NT), 0, stream, (const uint8_t*)A, As,
+                     (const uint8_t*)Bt, Bs, (void*)planes, (float*)nullptr, M, N, K, tiles_m, tiles_n);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  int rows_per_wg = 8;
+  while (rows_per_wg < 64 && (long)(N / 128) * ((M + 2 * rows_per_wg - 1) / (2 * rows_per_wg)) >= 2048) rows_per_wg *= 2;
+  hipLaunchKernelGGL((fp8_splitk_reduce_kernel<OUT>), dim3(N / 128, (M + rows_per_wg - 1) / rows_per_wg), dim3(256), 0, stream,
+                     (const float*)planes, S, C, Cs, M, N, rows_per_wg);
   return hipGetLastError();
 }
 
 template <int OUT>
 static hipError_t dispatch_fp8(int tile, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
-                               int M, int N, int K, hipStream_t stream)
+                               int M, int N, int K, int S, float* planes, hipStream_t stream)
 {
   switch (tile) {
-    case LLMMM_TILE_256x256: return launch_fp8<256, 256, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, stream);
-    case LLMMM_TILE_128x256: return launch_fp8<128, 256, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, stream);
-    case LLMMM_TILE_256x128: return launch_fp8<256, 128, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, stream);
-    case LLMMM_TILE_128x128: return launch_fp8<128, 128, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, stream);
+    case LLMMM_TILE_256x256: return launch_fp8<256, 256, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case LLMMM_TILE_128x256: return launch_fp8<128, 256, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case LLMMM_TILE_256x128: return launch_fp8<256, 128, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case LLMMM_TILE_128x128: return launch_fp8<128, 128, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
     default: return hipErrorInvalidValue;
   }
 }
 
 hipError_t fp8_gemm_launch(int out_kind, int tile, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
-                           float* Cs, int M, int N, int K, hipStream_t stream)
+                           float* Cs, int M, int N, int K, int S, float* planes, hipStream_t stream)
 {
   switch (out_kind) {
-    case OUT_F32: return dispatch_fp8<OUT_F32>(tile, A, As, Bt, Bs, C, Cs, M, N, K, stream);
-    case OUT_BF16: return dispatch_fp8<OUT_BF16>(tile, A, As, Bt, Bs, C, Cs, M, N, K, stream);
-    case OUT_FP8Q: return dispatch_fp8<OUT_FP8Q>(tile, A, As, Bt, Bs, C, Cs, M, N, K, stream);
+    case OUT_F32: return dispatch_fp8<OUT_F32>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case OUT_BF16: return dispatch_fp8<OUT_BF16>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case OUT_FP8Q: return dispatch_fp8<OUT_FP8Q>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
     default: return hipErrorInvalidValue;
   }
 }

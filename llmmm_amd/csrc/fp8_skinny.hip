@@ -1,7 +1,7 @@
 // Small-M (decode) FP8 blockwise GEMM for gfx950: weight streaming with deterministic split-K.
 //
 // Same arithmetic and layouts as fp8_gemm.hip (reference math: examples/005.fp8.mm.cu:885-902,
-// fused epilogue examples/005.fp8.mm.opt.cu:401-462) for M <= 64 rows, a range the reference
+// fused epilogue examples/005.fp8.mm.opt.cu:401-462) for M <= 128 rows (in groups of 64), a range the reference
 // does not cover (its launchers require M % 128 == 0, examples/005.fp8.mm.opt.cu:492; split-K
 // is listed as unfinished in README.md:22).
 //
@@ -138,6 +138,8 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   const int i    = lane & 15;
   const int ng   = blockIdx.x;
   const int sp   = blockIdx.y;
+  const int m0   = blockIdx.z * 64;                  // rows are handled in groups of 64: gridDim.z = ceil(M / 64)
+  const int cnt  = ng * gridDim.z + blockIdx.z;      // arrival counter of this (column group, row group)
   const int KB   = K >> 7;
   const int kb0  = sp * KB / S;  // KB * S is small: 32-bit arithmetic (a 64-bit divide costs hundreds of scalar ops)
   const int kb1  = (sp + 1) * KB / S;
@@ -161,7 +163,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   const float*     asp[MBLK];
 #pragma unroll
   for (int mb = 0; mb < MBLK; ++mb) {
-    const int m = min(mb * 16 + i, M - 1);
+    const int m = min(m0 + mb * 16 + i, M - 1);
     ap[mb]      = A + (size_t)m * K + 32 * g;  // same k -> register mapping as the weights: bytes 32g .. 32g+31
     asp[mb]     = As + m;
   }
@@ -210,7 +212,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
     // which costs far more than this kernel's entire run.
 #pragma unroll
     for (int mb = 0; mb < MBLK; ++mb) {
-      const int m = mb * 16 + i;
+      const int m = m0 + mb * 16 + i;
       if (m < M) {
         float* dst = partial + ((size_t)sp * M + m) * N + ncol;
 #pragma unroll
@@ -220,14 +222,14 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): this wave's partial stores are acknowledged
     __syncthreads();
     if (tid == 0) {
-      const unsigned old = __hip_atomic_fetch_add(counters + ng, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned old = __hip_atomic_fetch_add(counters + cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       is_last            = (old == (unsigned)(S - 1));
     }
     __syncthreads();
     if (!is_last) return;
 #pragma unroll
     for (int mb = 0; mb < MBLK; ++mb) {
-      const int m = mb * 16 + i;
+      const int m = m0 + mb * 16 + i;
       f32x4     t = {0.f, 0.f, 0.f, 0.f};
       if (m < M) {
         // fixed order 0..S-1, whoever arrived last; the loads of eight splits are put in flight
@@ -251,14 +253,14 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
       }
       acc[mb] = t;
     }
-    if (tid == 0) __hip_atomic_store(counters + ng, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    if (tid == 0) __hip_atomic_store(counters + cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
   }
 
   if constexpr (OUT == SK_OUT_F32) {
     float* C = (float*)Cv;
 #pragma unroll
     for (int mb = 0; mb < MBLK; ++mb) {
-      const int m = mb * 16 + i;
+      const int m = m0 + mb * 16 + i;
       if (m < M) *(f32x4*)(C + (size_t)m * N + ncol) = acc[mb];
     }
   }
@@ -267,7 +269,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
     typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
     for (int mb = 0; mb < MBLK; ++mb) {
-      const int m = mb * 16 + i;
+      const int m = m0 + mb * 16 + i;
       bf16x4    o;
 #pragma unroll
       for (int r = 0; r < 4; ++r) o[r] = (__bf16)acc[mb][r];
@@ -287,7 +289,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
     __syncthreads();
 #pragma unroll
     for (int mb = 0; mb < MBLK; ++mb) {
-      const int m    = mb * 16 + i;
+      const int m    = m0 + mb * 16 + i;
       float     amax = 0.f;
 #pragma unroll
       for (int w = 0; w < 8; ++w) amax = fmaxf(amax, wave_amax[w][mb][i]);
@@ -306,7 +308,7 @@ template <int MBLK, int OUT, int D>
 static hipError_t launch_skinny(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
                                 int N, int K, int S, float* partial, unsigned* counters, hipStream_t stream)
 {
-  hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D>), dim3(N / 128, S), dim3(512), 0, stream, (const uint8_t*)A, As,
+  hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D>), dim3(N / 128, S, (M + 63) / 64), dim3(512), 0, stream, (const uint8_t*)A, As,
                      (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial, counters);
   return hipGetLastError();
 }
@@ -326,7 +328,7 @@ static hipError_t dispatch_skinny(const void* A, const float* As, const void* Bt
     if (slices >= 4) LLMMM_GO(2, 4);
     LLMMM_GO(2, 2);
   }
-  if (M <= 64) {
+  if (M <= 128) {  // two row groups of (up to) 64 when M > 64
     if (slices >= 4) LLMMM_GO(4, 4);
     LLMMM_GO(4, 2);
   }

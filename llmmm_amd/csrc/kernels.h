@@ -13,11 +13,13 @@ namespace llmmm {
 hipError_t fp16_gemm_launch(int dtype, int b_layout, int tile, const void* A, const void* B, void* C, int M, int N, int K,
                             hipStream_t stream);
 
-// out_kind: 0 = fp32, 1 = bf16, 2 = e4m3 codes + per-1x128 scales.
+// out_kind: 0 = fp32, 1 = bf16, 2 = e4m3 codes + per-1x128 scales.  S > 1 splits K over S
+// workgroups per tile (S <= K/128): `planes` then holds S * M * N floats of partial sums, added
+// in split order by a second kernel that also runs the epilogue.
 hipError_t fp8_gemm_launch(int out_kind, int tile, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
-                           float* Cs, int M, int N, int K, hipStream_t stream);
+                           float* Cs, int M, int N, int K, int S, float* planes, hipStream_t stream);
 
-// M <= 64; S splits of K; partial [S][M][N] fp32 and counters [N/128] are only touched when S > 1.
+// M <= 128 (row groups of 64); S splits of K; partial [S][M][N] fp32 and counters [N/128 * ceil(M/64)] are only touched when S > 1.
 hipError_t fp8_skinny_launch(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
                              int M, int N, int K, int S, float* partial, unsigned* counters, hipStream_t stream);
 

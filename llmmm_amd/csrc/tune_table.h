@@ -14,9 +14,10 @@ struct SkinnyTune {
 struct TileTune {
   int M, N, K;
   int tile;
+  int split_k;  // 0 = heuristic
 };
 
-// FP8 weight-streaming kernel (M <= 64).
+// FP8 weight-streaming kernel (M <= 128, M != 128).
 static const SkinnyTune kSkinnyTune[] = {
   {1, 2560, 4096, 8},
   {16, 2560, 4096, 8},
@@ -34,13 +35,22 @@ static const SkinnyTune kSkinnyTune[] = {
 
 // FP8 MFMA tile kernels (M % 128 == 0).
 static const TileTune kTileTune[] = {
-  {4096, 4096, 4096, 0},
+  {4096, 4096, 4096, 0, 1},
+  {128, 6144, 2560, 3, 3},
+  {2048, 6144, 2560, 0, 1},
+  {128, 2560, 4096, 3, 8},
+  {2048, 2560, 4096, 3, 1},
+  {128, 19456, 2560, 3, 1},
+  {2048, 19456, 2560, 0, 1},
+  {128, 2560, 9728, 3, 8},
+  {2048, 2560, 9728, 0, 3},
 };
 
 // FP16/BF16 MFMA tile kernels.
 static const TileTune kFp16TileTune[] = {
-  {4096, 4096, 4096, 0},
-  {1024, 1024, 1024, 3},
+  {4096, 4096, 4096, 0, 1},
+  {1024, 1024, 1024, 3, 1},
 };
 
 }  // namespace llmmm
+

@@ -4,8 +4,8 @@ of shapes on the GPU at hand and writes ``csrc/tune_table.h`` (compiled into ``l
     python -m llmmm_amd.tune [--write] [--shapes qwen3-4b] [--m 1,16,128,2048]
 
 The reference only hints at such an interface (``tune(N, K)`` in src/mm/fp32/impl.h:20-23, a
-stub that throws).  Candidates: for M <= 64 the split-K factor of the weight-streaming kernel;
-for M % 128 == 0 the MFMA tile.  Timing: HIP events around a HIP graph of back-to-back launches
+stub that throws).  Candidates: for M <= 128 the split-K factor of the weight-streaming kernel;
+for M % 128 == 0 the MFMA tile (M = 128 tries both).  Timing: HIP events around a HIP graph of back-to-back launches
 that rotate over enough weight copies to defeat the caches (decode shapes) -- the same method
 ``bench.py`` uses.  Without ``--write`` the table is only printed.
 """
@@ -59,18 +59,23 @@ def _inputs(M, N, K, copies):
 
 def tune_shape(M, N, K, iters=40, rotate_bytes=768 << 20, verbose=True):
     """Returns (best_tile, best_split, {candidate: ms})."""
-    skinny = M <= 64
+    skinny = M <= 128
     copies = max(2, -(-rotate_bytes // (N * K))) if M <= 128 else 1
     Aq, As, weights = _inputs(M, N, K, copies)
     Cq = torch.empty((M, N), dtype=torch.uint8, device="cuda")
     Cs = torch.empty((N // 128, M), dtype=torch.float32, device="cuda")
-    ws = mm.make_workspace(_lib.OUT_FP8Q, M, N, K)
+    kb = K // 128
+    tile_splits = [x for x in (1, 2, 3, 4, 5, 6, 8) if x <= max(1, kb // 2)]
+    max_split = min(32, kb) if skinny else max(tile_splits)
+    ws = torch.zeros(4096 + max_split * M * N * 4, dtype=torch.uint8, device="cuda")  # zeroed counters + partial planes
+    cands = []
     if skinny:
         kb = K // 128
         cands = [(_lib.TILE_SKINNY, s) for s in sorted({1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 19, 20, 24, 32, kb, kb // 2}) if 1 <= s <= min(32, kb)]
-    else:
-        cands = [(t, 1) for t, (bm, bn) in {_lib.TILE_256x256: (256, 256), _lib.TILE_128x256: (128, 256), _lib.TILE_256x128: (256, 128),
-                                             _lib.TILE_128x128: (128, 128)}.items() if M % bm == 0 and N % bn == 0]
+    if M % 128 == 0:
+        dims = {_lib.TILE_256x256: (256, 256), _lib.TILE_128x256: (128, 256), _lib.TILE_256x128: (256, 128), _lib.TILE_128x128: (128, 128)}
+        cands = (cands if skinny and M % 128 else []) + [(t, x) for t, (bm, bn) in dims.items() if M % bm == 0 and N % bn == 0
+                                                          for x in tile_splits if x == 1 or (M // bm) * (N // bn) * x <= 640]
     results = {}
     for tile, split in cands:
         state = {"i": 0}
@@ -94,13 +99,13 @@ def render_table(skinny_rows, tile_rows, fp16_rows):
            "// (The reference only sketches this interface: `tune(N, K)` in src/mm/fp32/impl.h:20-23.)",
            "#pragma once", '#include "kernels.h"', "", "namespace llmmm {", "",
            "struct SkinnyTune {", "  int m_max;  // entry applies to M <= m_max (entries are ordered by m_max per shape)", "  int N, K;", "  int split_k;", "};",
-           "struct TileTune {", "  int M, N, K;", "  int tile;", "};", "",
-           "// FP8 weight-streaming kernel (M <= 64).", "static const SkinnyTune kSkinnyTune[] = {"]
+           "struct TileTune {", "  int M, N, K;", "  int tile;", "  int split_k;  // 0 = heuristic", "};", "",
+           "// FP8 weight-streaming kernel (M <= 128, M != 128).", "static const SkinnyTune kSkinnyTune[] = {"]
     out += ["  {%d, %d, %d, %d}," % r for r in skinny_rows]
     out += ["};", "", "// FP8 MFMA tile kernels (M % 128 == 0).", "static const TileTune kTileTune[] = {"]
-    out += ["  {%d, %d, %d, %d}," % r for r in tile_rows]
+    out += ["  {%d, %d, %d, %d, %d}," % r for r in tile_rows]
     out += ["};", "", "// FP16/BF16 MFMA tile kernels.", "static const TileTune kFp16TileTune[] = {"]
-    out += ["  {%d, %d, %d, %d}," % r for r in fp16_rows]
+    out += ["  {%d, %d, %d, %d, %d}," % r for r in fp16_rows]
     out += ["};", "", "}  // namespace llmmm", ""]
     return "\n".join(out)
 
@@ -113,17 +118,17 @@ def main():
     args = ap.parse_args()
     torch.cuda.set_device(0)
     ms = [int(x) for x in args.m.split(",")]
-    skinny_rows, tile_rows = [], [(4096, 4096, 4096, _lib.TILE_256x256)]
+    skinny_rows, tile_rows = [], [(4096, 4096, 4096, _lib.TILE_256x256, 1)]
     for name, (N, K) in QWEN3_4B.items():
         for M in ms:
             tile, split, _ = tune_shape(M, N, K, iters=args.iters)
-            if M <= 64:
+            if tile == _lib.TILE_SKINNY:
                 skinny_rows.append((M, N, K, split))
             else:
-                tile_rows.append((M, N, K, tile))
+                tile_rows.append((M, N, K, tile, split))
             torch.cuda.empty_cache()
     skinny_rows.sort(key=lambda r: (r[1], r[2], r[0]))
-    fp16_rows = [(4096, 4096, 4096, _lib.TILE_256x256), (1024, 1024, 1024, _lib.TILE_128x128)]
+    fp16_rows = [(4096, 4096, 4096, _lib.TILE_256x256, 1), (1024, 1024, 1024, _lib.TILE_128x128, 1)]
     text = render_table(skinny_rows, tile_rows, fp16_rows)
     print(text)
     if args.write:

@@ -63,7 +63,7 @@ def test_fp8_validation_without_device():
     args = (FAKE, FAKE, FAKE, FAKE, FAKE, FAKE)
     assert f(2, *args, 128, 100, 256, None, 0, None) == _lib.ERR_NOT_ALIGNED
     assert f(2, *args, 128, 128, 200, None, 0, None) == _lib.ERR_NOT_ALIGNED
-    assert f(2, *args, 100, 128, 256, None, 0, None) == _lib.ERR_NOT_ALIGNED  # 64 < M, M % 128 != 0
+    assert f(2, *args, 200, 128, 256, None, 0, None) == _lib.ERR_NOT_ALIGNED  # 128 < M, M % 128 != 0
     assert f(9, *args, 128, 128, 256, None, 0, None) == _lib.ERR_INVALID_ARGUMENT
     assert f(2, FAKE, FAKE, FAKE, FAKE, FAKE, None, 128, 128, 256, None, 0, None) == _lib.ERR_INVALID_ARGUMENT  # Cs missing
     assert f(0, None, FAKE, FAKE, FAKE, FAKE, None, 128, 128, 256, None, 0, None) == _lib.ERR_INVALID_ARGUMENT
@@ -73,7 +73,7 @@ def test_fp8_validation_without_device():
     assert lib.llmmm_fp8_gemm_ex(2, *args, 16, 256, 1024, FAKE, 4096, ctypes.byref(cfg), None) == _lib.ERR_WORKSPACE
     assert b"workspace" in lib.llmmm_last_error()
     cfg = _lib.GemmCfg(_lib.TILE_SKINNY, 1)
-    assert lib.llmmm_fp8_gemm_ex(2, *args, 128, 256, 1024, None, 0, ctypes.byref(cfg), None) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.llmmm_fp8_gemm_ex(2, *args, 256, 256, 1024, None, 0, ctypes.byref(cfg), None) == _lib.ERR_INVALID_ARGUMENT
 
 
 def test_quant_and_workspace_validation_without_device():
@@ -90,9 +90,9 @@ def test_quant_and_workspace_validation_without_device():
 def test_workspace_sizes_and_config_queries():
     import llmmm_amd
     from llmmm_amd import _lib
-    # the tile kernels never need a workspace; the skinny kernel needs counters + S partial tiles
+    # a shape with a tile per CU never splits and needs no workspace; split configurations need
+    # the counter header + S partial planes
     assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, 4096, 4096, 4096) == 0
-    assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, 128, 6144, 2560) == 0
     for (n, k) in [(6144, 2560), (2560, 4096), (19456, 2560), (2560, 9728)]:
         for m in (1, 16):
             tile, split = llmmm_amd.query_config(_lib.OUT_FP8Q, m, n, k)
@@ -100,10 +100,12 @@ def test_workspace_sizes_and_config_queries():
             assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, m, n, k) >= 4096 + split * m * n * 4
         for m in (128, 2048):
             tile, split = llmmm_amd.query_config(_lib.OUT_FP8Q, m, n, k)
-            assert tile in (_lib.TILE_256x256, _lib.TILE_128x256, _lib.TILE_256x128, _lib.TILE_128x128) and split == 1
+            assert tile in (_lib.TILE_256x256, _lib.TILE_128x256, _lib.TILE_256x128, _lib.TILE_128x128) and 1 <= split <= 8
+            need = 0 if split == 1 else 4096 + split * m * n * 4
+            assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, m, n, k) == need
     assert llmmm_amd.query_config(_lib.OUT_FP8Q, 4096, 4096, 4096) == (_lib.TILE_256x256, 1)
     with pytest.raises(RuntimeError, match="M or N or K are not aligned."):
-        llmmm_amd.query_config(_lib.OUT_FP8Q, 100, 4096, 4096)
+        llmmm_amd.query_config(_lib.OUT_FP8Q, 200, 4096, 4096)
 
 
 def test_python_mirror_raises_like_the_reference():

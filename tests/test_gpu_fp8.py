@@ -25,6 +25,8 @@ def _run_all(lib, Aq, As, Bq, Bs, tile=-1, split_k=0, use_ws=True):
     N = Bq.shape[0]
     t = _gpu(Aq, As, Bq, Bs)
     ws = lib.make_workspace(2, M, N, K) if use_ws else None
+    if use_ws and split_k > 1:  # an explicit split: 4 KiB of counters + split_k partial planes, zero-initialised
+        ws = torch.zeros(4096 + split_k * M * N * 4, dtype=torch.uint8, device="cuda")
     C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
     Cb = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
     Cq = torch.full((M, N), 0x55, dtype=torch.uint8, device="cuda")
@@ -56,6 +58,20 @@ def test_tile_kernels_against_oracle(lib, oracle, tile):
     Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=3)
     ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
     _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, tile=TILES[tile]), ref, "tile " + tile)
+
+
+@pytest.mark.parametrize("tile", ["256x256", "128x128"])
+@pytest.mark.parametrize("split", [2, 3, 7])
+def test_tile_kernels_split_k(lib, oracle, tile, split):
+    """Split-K of the tile kernels: partial planes added in split order by the reduce kernel;
+    uneven slice counts per split (9 slices over 2, 3 and 7 splits)."""
+    M, N, K = 256, 512, 1152
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=77)
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    out = _run_all(lib, Aq, As, Bq, Bs, tile=TILES[tile], split_k=split)
+    _check_all(oracle, out, ref, "tile %s split %d" % (tile, split))
+    again = _run_all(lib, Aq, As, Bq, Bs, tile=TILES[tile], split_k=split)
+    assert all((a == b).all() for a, b in zip(out[1:], again[1:])) and (out[0].view(np.uint32) == again[0].view(np.uint32)).all()
 
 
 @pytest.mark.parametrize("K", [128, 256, 384, 512, 640])
@@ -110,7 +126,7 @@ def test_zero_blocks_give_zero_codes_and_scales(lib, oracle):
     assert np.isfinite(oracle.e4m3_decode(Cq)).all()
 
 
-@pytest.mark.parametrize("M", [1, 2, 15, 16, 17, 33, 64])
+@pytest.mark.parametrize("M", [1, 2, 15, 16, 17, 33, 64, 65, 96, 128])
 @pytest.mark.parametrize("split", [1, 3, 8])
 def test_skinny_kernel_against_oracle(lib, oracle, M, split):
     N, K = 384, 1024
