@@ -85,22 +85,26 @@ LLMMM_API int llmmm_fp16_gemm_ex(int dtype, const void* A, const void* B, void* 
  *                                                                     examples/005.fp8.mm.opt.cu:468-508.
  * C is float* (OUT_F32), bf16* (OUT_BF16) or e4m3 uint8_t* (OUT_FP8Q); Cs is only used (and
  * required) for OUT_FP8Q.  N % 128 == 0 and K % 128 == 0 are required.  M % 128 == 0 runs the
- * MFMA tile kernels (the reference's domain); 1 <= M <= 128 runs the weight-streaming kernel
- * (M = 128: unless a tile is requested through llmmm_fp8_gemm_ex), which may split K: then `workspace` must hold llmmm_fp8_gemm_workspace() bytes, prepared once
- * with llmmm_workspace_init().  With workspace == NULL no split is used.  Other M are rejected
- * as not aligned.  Calls that share a workspace must be ordered on one stream. */
+ * MFMA tile kernels (the reference's domain); 1 <= M < 128 runs the weight-streaming kernel
+ * (so does M = 128 when LLMMM_TILE_SKINNY is requested through llmmm_fp8_gemm_ex).  Other M are
+ * rejected as not aligned.
+ * Split-K: shapes with too few tiles or column groups to fill the GPU split K over several
+ * workgroups; each split stores a plane of fp32 partial sums into `workspace` and a second
+ * kernel adds the planes in split order (a fixed order: results do not depend on timing) and
+ * applies the epilogue.  `workspace` is plain scratch of llmmm_fp8_gemm_workspace() bytes, needs
+ * no initialisation and holds nothing between calls.  With workspace == NULL (or one too small
+ * for the split the library would pick) K is split less or not at all; an explicit
+ * cfg->split_k that does not fit is an error.  Calls that share a workspace must be ordered on
+ * one stream. */
 LLMMM_API int llmmm_fp8_gemm(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
                              int M, int N, int K, void* workspace, size_t workspace_bytes, void* stream);
 LLMMM_API int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
                                 int M, int N, int K, void* workspace, size_t workspace_bytes, const llmmm_gemm_cfg* cfg,
                                 void* stream);
 /* Bytes of workspace that any configuration the library may pick for this shape needs
- * (0 when the shape never splits K).  No reference counterpart: split-K is "still to do" there
- * (README.md:22). */
+ * (0 when the shape never splits K); an explicit split_k = S needs S * M * N * 4 bytes.  No
+ * reference counterpart: split-K is "still to do" there (README.md:22). */
 LLMMM_API size_t llmmm_fp8_gemm_workspace(int out_kind, int M, int N, int K);
-/* Zeroes the arrival counters at the head of a workspace (a small fill kernel, safe to capture
- * in a HIP graph).  Call once after allocating it; the kernels leave the counters at zero. */
-LLMMM_API int llmmm_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 /* The configuration llmmm_fp8_gemm would use for this shape (tune table, then heuristic). */
 LLMMM_API int llmmm_fp8_gemm_query(int out_kind, int M, int N, int K, llmmm_gemm_cfg* cfg);
 

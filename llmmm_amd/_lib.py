@@ -35,7 +35,6 @@ SIGNATURES = {
     "llmmm_fp8_gemm": (_i, [_i, _vp, _fp, _vp, _fp, _vp, _fp, _i, _i, _i, _vp, _sz, _vp]),
     "llmmm_fp8_gemm_ex": (_i, [_i, _vp, _fp, _vp, _fp, _vp, _fp, _i, _i, _i, _vp, _sz, _c.POINTER(GemmCfg), _vp]),
     "llmmm_fp8_gemm_workspace": (_sz, [_i, _i, _i, _i]),
-    "llmmm_workspace_init": (_i, [_vp, _sz, _vp]),
     "llmmm_fp8_gemm_query": (_i, [_i, _i, _i, _i, _c.POINTER(GemmCfg)]),
     "llmmm_quant_fp8": (_i, [_i, _fp, _vp, _fp, _i, _i, _vp]),
     "llmmm_error_string": (_c.c_char_p, [_i]),

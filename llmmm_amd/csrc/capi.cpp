@@ -7,6 +7,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
+#include <stdlib.h>
 #include <stdio.h>
 #include <string.h>
 
@@ -26,7 +27,6 @@ int fail(int code, const char* fmt, ...)
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-constexpr size_t WS_HEADER_BYTES = 4096;  // arrival counters: one uint32 per 128-column group
 constexpr int    MAX_SPLIT_K     = 32;
 constexpr int    NUM_CUS         = 256;   // MI355X
 
@@ -35,16 +35,19 @@ constexpr int SKINNY_MAX_M = 128;  // rows the weight-streaming kernel takes (tw
 int max_split_for(int K) { return (K / 128) < MAX_SPLIT_K ? (K / 128) : MAX_SPLIT_K; }
 
 // Split count for the weight-streaming kernel when the tune table has no entry: about one
-// workgroup (one 128-column group x one split) per CU -- what the measured Qwen3-4B shapes
-// settle on -- every split at least two 128-K slices long, fewer splits when there are many
-// rows (the fp32 partial tiles grow with M).
+// workgroup (one 128-column group x one 64-row group x one split) per CU -- what the measured
+// Qwen3-4B shapes settle on -- every split at least two 128-K slices long, but short enough
+// that the activation rows of a split can be staged in LDS (64 KB: 32 slices of 16 rows).
 int heuristic_split(int M, int N, int K)
 {
   const int groups = (N / 128) * ((M + 63) / 64), kb = K / 128;
   int       s      = (240 + groups / 2) / groups;
-  if (M > 16 && M <= 64) s = (s + 1) / 2;
   if (s > kb / 2) s = kb / 2;
+  const int mblk = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+  const int cap  = 32 / mblk;  // slices whose rows fit the staging area
+  if (s < (kb + cap - 1) / cap) s = (kb + cap - 1) / cap;
   if (s > MAX_SPLIT_K) s = MAX_SPLIT_K;
+  if (s > kb) s = kb;
   if (s < 1) s = 1;
   return s;
 }
@@ -108,27 +111,28 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
 {
   if (M <= 0 || N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "M, N and K must be positive (got %d, %d, %d)", M, N, K);
   if (N % 128 || K % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
-  if (M <= SKINNY_MAX_M && M % 128) {  // M = 128 is better served by a split tile kernel
-    cfg->tile    = LLMMM_TILE_SKINNY;
-    cfg->split_k = 0;
-    for (const auto& e : llmmm::kSkinnyTune)
-      if (e.N == N && e.K == K && M <= e.m_max) {
+  cfg->tile    = -1;
+  cfg->split_k = 0;
+  if (M % 128 == 0)
+    for (const auto& e : llmmm::kTileTune)
+      if (e.M == M && e.N == N && e.K == K) {
+        cfg->tile    = e.tile;
         cfg->split_k = e.split_k;
         break;
       }
-    if (cfg->split_k == 0) cfg->split_k = heuristic_split(M, N, K);
-    return LLMMM_OK;
+  if (cfg->tile < 0 && M <= SKINNY_MAX_M) {
+    for (const auto& e : llmmm::kSkinnyTune)
+      if (e.N == N && e.K == K && M <= e.m_max) {
+        cfg->tile    = LLMMM_TILE_SKINNY;
+        cfg->split_k = e.split_k;
+        break;
+      }
+    if (cfg->tile < 0 && M % 128) cfg->tile = LLMMM_TILE_SKINNY;  // untuned M = 128 goes to a split tile kernel
   }
-  if (M % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
-  cfg->tile    = -1;
-  cfg->split_k = 0;
-  for (const auto& e : llmmm::kTileTune)
-    if (e.M == M && e.N == N && e.K == K) {
-      cfg->tile    = e.tile;
-      cfg->split_k = e.split_k;
-      break;
-    }
-  if (cfg->tile < 0) cfg->tile = heuristic_tile(M, N);
+  if (cfg->tile < 0) {
+    if (M % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+    cfg->tile = heuristic_tile(M, N);
+  }
   if (cfg->tile == LLMMM_TILE_SKINNY) {
     if (cfg->split_k <= 0) cfg->split_k = heuristic_split(M, N, K);
   }
@@ -208,16 +212,7 @@ size_t llmmm_fp8_gemm_workspace(int out_kind, int M, int N, int K)
   // the weight-streaming kernel: room for any split the tuner may try; tile kernels: the split chosen
   const int s = cfg.tile == LLMMM_TILE_SKINNY ? max_split_for(K) : cfg.split_k;
   if (s <= 1) return 0;
-  return WS_HEADER_BYTES + (size_t)s * M * N * sizeof(float);
-}
-
-int llmmm_workspace_init(void* workspace, size_t workspace_bytes, void* stream)
-{
-  if (!workspace || workspace_bytes < WS_HEADER_BYTES) return fail(LLMMM_ERR_WORKSPACE, "workspace must hold at least %zu bytes", WS_HEADER_BYTES);
-  if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
-  const hipError_t e = llmmm::fill_u32_launch((uint32_t*)workspace, 0u, WS_HEADER_BYTES / 4, (hipStream_t)stream);
-  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "workspace init: %s", hipGetErrorString(e));
-  return LLMMM_OK;
+  return (size_t)s * M * N * sizeof(float);
 }
 
 int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
@@ -232,7 +227,6 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
   if (!aligned16(A) || !aligned16(Bt) || !aligned16(C)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
   if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
-  if ((N / 128) * 2 > (int)(WS_HEADER_BYTES / 4)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "N too large");
   if (user) {
     if (user->tile != LLMMM_TILE_AUTO) cfg.tile = user->tile;
     if (user->split_k > 0) cfg.split_k = user->split_k;
@@ -244,16 +238,15 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
     if (split > max_split_for(K)) split = max_split_for(K);
     if (split < 1) split = 1;
     if (!workspace) split = 1;  // documented: no workspace, no split
-    float*    partial  = nullptr;
-    unsigned* counters = nullptr;
+    float* partial = nullptr;
     if (split > 1) {
-      const size_t need = WS_HEADER_BYTES + (size_t)split * M * N * sizeof(float);
+      const size_t need = (size_t)split * M * N * sizeof(float);
       if (workspace_bytes < need) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace_bytes, split, need);
       if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
-      counters = (unsigned*)workspace;
-      partial  = (float*)((char*)workspace + WS_HEADER_BYTES);
+      partial = (float*)workspace;
     }
-    e = llmmm::fp8_skinny_launch(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, split, partial, counters, (hipStream_t)stream);
+    e = llmmm::fp8_skinny_launch(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, split, partial, (hipStream_t)stream);
+    if (e == hipSuccess && split > 1) e = llmmm::fp8_splitk_reduce_launch(out_kind, partial, split, C, Cs, M, N, (hipStream_t)stream);
   }
   else {
     int bm, bn;
@@ -268,14 +261,14 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
     if (split > 1 && !(user && user->split_k > 0)) {
       // a split the library chose itself shrinks to what the caller's workspace holds
       const size_t plane = (size_t)M * N * sizeof(float);
-      const size_t room  = workspace_bytes > WS_HEADER_BYTES ? (workspace_bytes - WS_HEADER_BYTES) / plane : 0;
+      const size_t room  = workspace_bytes / plane;
       if ((size_t)split > room) split = room < 2 ? 1 : (int)room;
     }
     if (split > 1) {
-      const size_t need = WS_HEADER_BYTES + (size_t)split * M * N * sizeof(float);
+      const size_t need = (size_t)split * M * N * sizeof(float);
       if (workspace_bytes < need) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace_bytes, split, need);
       if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
-      planes = (float*)((char*)workspace + WS_HEADER_BYTES);
+      planes = (float*)workspace;
     }
     e = llmmm::fp8_gemm_launch(out_kind, cfg.tile, A, As, Bt, Bs, C, Cs, M, N, K, split, planes, (hipStream_t)stream);
   }

@@ -408,6 +408,16 @@ fp8_splitk_reduce_kernel(const float* __restrict__ planes, int S, void* __restri
 }
 
 // --------------------------------------------------------------------------------------------- host
+template <int OUT>
+static hipError_t launch_reduce(const float* planes, int S, void* C, float* Cs, int M, int N, hipStream_t stream)
+{
+  int rows_per_wg = 8;
+  while (rows_per_wg < 64 && (long)(N / 128) * ((M + 2 * rows_per_wg - 1) / (2 * rows_per_wg)) >= 2048) rows_per_wg *= 2;
+  hipLaunchKernelGGL((fp8_splitk_reduce_kernel<OUT>), dim3(N / 128, (M + rows_per_wg - 1) / rows_per_wg), dim3(256), 0, stream, planes,
+                     S, C, Cs, M, N, rows_per_wg);
+  return hipGetLastError();
+}
+
 template <int BM, int BN, int OUT>
 static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N,
                              int K, int S, float* planes, hipStream_t stream)
@@ -424,11 +434,7 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
                      (const uint8_t*)Bt, Bs, (void*)planes, (float*)nullptr, M, N, K, tiles_m, tiles_n);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  int rows_per_wg = 8;
-  while (rows_per_wg < 64 && (long)(N / 128) * ((M + 2 * rows_per_wg - 1) / (2 * rows_per_wg)) >= 2048) rows_per_wg *= 2;
-  hipLaunchKernelGGL((fp8_splitk_reduce_kernel<OUT>), dim3(N / 128, (M + rows_per_wg - 1) / rows_per_wg), dim3(256), 0, stream,
-                     (const float*)planes, S, C, Cs, M, N, rows_per_wg);
-  return hipGetLastError();
+  return launch_reduce<OUT>(planes, S, C, Cs, M, N, stream);
 }
 
 template <int OUT>
@@ -451,6 +457,16 @@ hipError_t fp8_gemm_launch(int out_kind, int tile, const void* A, const float* A
     case OUT_F32: return dispatch_fp8<OUT_F32>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
     case OUT_BF16: return dispatch_fp8<OUT_BF16>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
     case OUT_FP8Q: return dispatch_fp8<OUT_FP8Q>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t fp8_splitk_reduce_launch(int out_kind, const float* planes, int S, void* C, float* Cs, int M, int N, hipStream_t stream)
+{
+  switch (out_kind) {
+    case OUT_F32: return launch_reduce<OUT_F32>(planes, S, C, Cs, M, N, stream);
+    case OUT_BF16: return launch_reduce<OUT_BF16>(planes, S, C, Cs, M, N, stream);
+    case OUT_FP8Q: return launch_reduce<OUT_FP8Q>(planes, S, C, Cs, M, N, stream);
     default: return hipErrorInvalidValue;
   }
 }

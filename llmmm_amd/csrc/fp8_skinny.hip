@@ -11,9 +11,14 @@
 //    D slots, and reads the MFMA operand back with two conflict-free ds_read_b128.  The
 //    activation rows go straight from global memory (L2) into the other operand's registers.
 //  * A workgroup = 8 waves = one 128-column quantisation group; grid.y = number of K splits.
-//  * split-K: each split writes its fp32 partial tile to the workspace; the workgroup that
-//    arrives last at the group's counter adds the partials in split order 0..S-1 (fixed order,
-//    independent of arrival) and runs the epilogue.  Nobody waits on anybody.
+//  * split-K: each split stores its fp32 plane of partial sums (plain stores) and is done; the
+//    reduce kernel of fp8_gemm.hip, launched behind it, adds the planes in split order 0..S-1
+//    (fixed order, independent of arrival) and runs the epilogue.  An in-kernel "last arriver
+//    reduces" scheme was measured slower: its device-scope stores, counter and re-reads put three
+//    dependent memory round trips on the critical path of every column group.
+//  * The activation rows a workgroup needs (16..64 rows x the K range of its split) are staged
+//    in LDS once, before the loop, whenever they fit beside the ring; every wave then reads its
+//    operand fragments from there instead of re-fetching them from L2 slice by slice.
 #include "device_common.hip.h"
 #include "kernels.h"
 
@@ -35,9 +40,9 @@ __device__ __forceinline__ uint32_t sk_pack_e4m3x4(float a, float b, float c, fl
 // What one 128-K slice needs besides the weights: the activation rows (straight into the MFMA
 // operand registers) and both scales.  Rows beyond M are clamped to M-1 (a valid address, no
 // divergence); their products are computed and never stored.
-template <int MBLK>
+template <int MBLK, bool APRE>
 struct SkinnySlot {
-  i32x4 a[MBLK][2];
+  i32x4 a[APRE ? 1 : MBLK][2];  // unused when the activations were staged in LDS up front (APRE)
   float sa[MBLK];
   float sb;
 };
@@ -46,12 +51,12 @@ struct SkinnySlot {
 // loads of 1 KB each.  A load covers 8 whole rows, so every 128-byte line is fetched by one
 // instruction in full; the SWZ_ROWS16 placement makes the operand read-back conflict-free.
 // One wave-private ring slot = 2 KB; no workgroup barrier is involved.
-constexpr int SKINNY_LOADS_PER_SLOT_BASE = 2;  // LDS-direct loads; + 3 per 16 activation rows
+constexpr int SKINNY_LOADS_PER_SLOT_BASE = 2;  // LDS-direct loads; + 3 (or 1, with APRE) per 16 activation rows
 
 // All vector-memory loads of a slot, in a fixed order, as inline assembly (see device_common.hip.h):
 // the kernel counts them itself.
-template <int MBLK>
-__device__ __forceinline__ void skinny_fetch(SkinnySlot<MBLK>& t, unsigned ring_slot, const uint8_t* wrow, unsigned w_off0,
+template <int MBLK, bool APRE>
+__device__ __forceinline__ void skinny_fetch(SkinnySlot<MBLK, APRE>& t, unsigned ring_slot, const uint8_t* wrow, unsigned w_off0,
                                              unsigned w_off1, const uint8_t* const (&ap)[MBLK], const float* const (&asp)[MBLK],
                                              const float* bsp, int kb, int M)
 {
@@ -59,8 +64,10 @@ __device__ __forceinline__ void skinny_fetch(SkinnySlot<MBLK>& t, unsigned ring_
   asm_load_lds_16B(wrow + (size_t)kb * 128 + w_off1, ring_slot + 1024);
 #pragma unroll
   for (int mb = 0; mb < MBLK; ++mb) {
-    asm_load_16B(t.a[mb][0], ap[mb] + (size_t)kb * 128);
-    asm_load_16B(t.a[mb][1], ap[mb] + (size_t)kb * 128 + 16);
+    if constexpr (!APRE) {
+      asm_load_16B(t.a[mb][0], ap[mb] + (size_t)kb * 128);
+      asm_load_16B(t.a[mb][1], ap[mb] + (size_t)kb * 128 + 16);
+    }
     asm_load_f32(t.sa[mb], asp[mb] + (size_t)kb * M);
   }
   t.sb = bsp[kb];
@@ -68,11 +75,19 @@ __device__ __forceinline__ void skinny_fetch(SkinnySlot<MBLK>& t, unsigned ring_
 
 // s_waitcnt vmcnt(N) that also "touches" the slot's registers, so that nothing reading them can
 // be moved in front of it.
-template <int N, int MBLK>
-__device__ __forceinline__ void skinny_wait(SkinnySlot<MBLK>& t)
+template <int N, int MBLK, bool APRE>
+__device__ __forceinline__ void skinny_wait(SkinnySlot<MBLK, APRE>& t)
 {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-  if constexpr (MBLK == 1)
+  if constexpr (APRE) {
+    if constexpr (MBLK == 1)
+      asm volatile("s_waitcnt vmcnt(%1)" : "+v"(t.sa[0]) : "n"(N) : "memory");
+    else if constexpr (MBLK == 2)
+      asm volatile("s_waitcnt vmcnt(%2)" : "+v"(t.sa[0]), "+v"(t.sa[1]) : "n"(N) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(%4)" : "+v"(t.sa[0]), "+v"(t.sa[1]), "+v"(t.sa[2]), "+v"(t.sa[3]) : "n"(N) : "memory");
+  }
+  else if constexpr (MBLK == 1)
     asm volatile("s_waitcnt vmcnt(%3)" : "+v"(t.a[0][0]), "+v"(t.a[0][1]), "+v"(t.sa[0]) : "n"(N) : "memory");
   else if constexpr (MBLK == 2)
     asm volatile("s_waitcnt vmcnt(%6)"
@@ -87,9 +102,11 @@ __device__ __forceinline__ void skinny_wait(SkinnySlot<MBLK>& t)
                  : "memory");
 }
 
-template <int MBLK>
-__device__ __forceinline__ void skinny_consume(const SkinnySlot<MBLK>& t, const char LLMMM_LDS* ring_slot, int w_rd, bool valid,
-                                               f32x4 (&acc)[MBLK])
+// With APRE the activation fragments come from the workgroup's staged copy: a_slice points at
+// the MBLK x 2 KB block of this slice, a_rd is the lane's SWZ_ROWS16 offset of (row i, chunk 2g).
+template <int MBLK, bool APRE>
+__device__ __forceinline__ void skinny_consume(const SkinnySlot<MBLK, APRE>& t, const char LLMMM_LDS* ring_slot, int w_rd, bool valid,
+                                               f32x4 (&acc)[MBLK], const char LLMMM_LDS* a_slice, int a_rd)
 {
   union {
     i32x4 h[2];
@@ -99,8 +116,14 @@ __device__ __forceinline__ void skinny_consume(const SkinnySlot<MBLK>& t, const 
   wf.h[1] = *(const i32x4 LLMMM_LDS*)(ring_slot + (w_rd ^ 16));
 #pragma unroll
   for (int mb = 0; mb < MBLK; ++mb) {
-    af.h[0]       = t.a[mb][0];
-    af.h[1]       = t.a[mb][1];
+    if constexpr (APRE) {
+      af.h[0] = *(const i32x4 LLMMM_LDS*)(a_slice + mb * 2048 + a_rd);
+      af.h[1] = *(const i32x4 LLMMM_LDS*)(a_slice + mb * 2048 + (a_rd ^ 16));
+    }
+    else {
+      af.h[0] = t.a[mb][0];
+      af.h[1] = t.a[mb][1];
+    }
     const float s = valid ? t.sa[mb] * t.sb : 0.f;
     const f32x4 z = {0.f, 0.f, 0.f, 0.f};
     const f32x4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf.v, af.v, z, 0, 0, 0, 0, 0, 0);
@@ -111,14 +134,18 @@ __device__ __forceinline__ void skinny_consume(const SkinnySlot<MBLK>& t, const 
 
 // D = ring depth = slices in flight per wave.  The host picks the largest D that does not exceed
 // the number of slices of the shortest split.
-template <int MBLK, int OUT, int D>
+// ASTG = bytes of LDS in which the workgroup stages its activation rows for the whole K range
+// of its split before the loop starts (0: the rows are fetched slice by slice into registers).
+template <int MBLK, int OUT, int D, int ASTG>
 __global__ void __launch_bounds__(512)
 fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
                   const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int S,
-                  float* __restrict__ partial, unsigned* __restrict__ counters)
+                  float* __restrict__ partial)
 {
-  constexpr int LOADS = SKINNY_LOADS_PER_SLOT_BASE + 3 * MBLK;  // vector-memory loads per slot, issued in slot order
-  static_assert((D - 1) * LOADS < 64, "vmcnt is a 6-bit counter");
+  constexpr bool APRE  = ASTG > 0;
+  constexpr int  LOADS = SKINNY_LOADS_PER_SLOT_BASE + (APRE ? 1 : 3) * MBLK;  // vector-memory loads per slot, issued in slot order
+  static_assert(D * LOADS < 64, "vmcnt is a 6-bit counter");
+  __shared__ __attribute__((aligned(1024))) char a_stage[APRE ? ASTG : 16];
   // one array per ring slot, so that the compiler can tell the slots apart
   __shared__ __attribute__((aligned(1024))) char ring0[8 * 2048];
   __shared__ __attribute__((aligned(1024))) char ring1[8 * 2048];
@@ -129,7 +156,6 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   __shared__ __attribute__((aligned(1024))) char ring6[D > 4 ? 8 * 2048 : 16];
   __shared__ __attribute__((aligned(1024))) char ring7[D > 4 ? 8 * 2048 : 16];
   __shared__ float    wave_amax[8][MBLK][16];
-  __shared__ unsigned is_last;
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -139,7 +165,6 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   const int ng   = blockIdx.x;
   const int sp   = blockIdx.y;
   const int m0   = blockIdx.z * 64;                  // rows are handled in groups of 64: gridDim.z = ceil(M / 64)
-  const int cnt  = ng * gridDim.z + blockIdx.z;      // arrival counter of this (column group, row group)
   const int KB   = K >> 7;
   const int kb0  = sp * KB / S;  // KB * S is small: 32-bit arithmetic (a 64-bit divide costs hundreds of scalar ops)
   const int kb1  = (sp + 1) * KB / S;
@@ -172,31 +197,55 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
 #pragma unroll
   for (int mb = 0; mb < MBLK; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // Activation staging: the 16*MBLK rows x (kb1 - kb0) slices this workgroup needs, as one
+  // SWZ_ROWS16 tile of MBLK x 2 KB per slice, fetched once by LDS-direct loads of 8 whole rows
+  // (1 KB units dealt round-robin to the waves) instead of once per wave and slice.  They are
+  // the oldest loads in flight, so "at most D*LOADS outstanding" after the ring prologue means
+  // they have landed.
+  const char LLMMM_LDS* const a_tile = (const char LLMMM_LDS*)a_stage;
+  const int                   a_rd   = kmajor_offset<SWZ_ROWS16>(i, 2 * g);
+  if constexpr (APRE) {
+    const unsigned a_addr = (unsigned)(size_t)(char LLMMM_LDS*)a_stage;
+    const int      units  = (kb1 - kb0) * 2 * MBLK;
+    for (int u = wave; u < units; u += 8) {
+      const int j = u / (2 * MBLK), within = u - j * (2 * MBLK);
+      const int r = within * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ kmajor_swz<SWZ_ROWS16>(r);
+      const int m = min(m0 + r, M - 1);
+      asm_load_lds_16B(A + (size_t)m * K + (size_t)(kb0 + j) * 128 + c * 16, a_addr + j * (MBLK * 2048) + within * 1024);
+    }
+  }
+
   // Software pipeline, D slices in flight per wave, all vector-memory loads issued strictly in
   // slot order so that "at most n loads outstanding" pins down which slots have landed.
   // Slice indices beyond the split are clamped to its last slice (a repeated, cached load) and
   // consumed with a zero scale; the last pass issues nothing and counts its waits down.
-  SkinnySlot<MBLK> slot[D];
+  SkinnySlot<MBLK, APRE> slot[D];
 #pragma unroll
   for (int u = 0; u < D; ++u) {
-    skinny_fetch<MBLK>(slot[u], ring_addr[u], wrow, w_off0, w_off1, ap, asp, bsp, min(kb0 + u, kb1 - 1), M);
+    skinny_fetch<MBLK, APRE>(slot[u], ring_addr[u], wrow, w_off0, w_off1, ap, asp, bsp, min(kb0 + u, kb1 - 1), M);
     __builtin_amdgcn_sched_barrier(0);
+  }
+  if constexpr (APRE) {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * LOADS) : "memory");
+    __syncthreads();  // every wave's share of the staged activations is in LDS
   }
   int kb = kb0;
   for (; kb + D < kb1; kb += D) {  // passes followed by another pass: consume a slot, refill it
 #pragma unroll
     for (int u = 0; u < D; ++u) {
-      skinny_wait<(D - 1) * LOADS, MBLK>(slot[u]);
-      skinny_consume<MBLK>(slot[u], ring[u], w_rd, true, acc);
+      skinny_wait<(D - 1) * LOADS, MBLK, APRE>(slot[u]);
+      skinny_consume<MBLK, APRE>(slot[u], ring[u], w_rd, true, acc, a_tile + (kb + u - kb0) * (MBLK * 2048), a_rd);
       __builtin_amdgcn_sched_barrier(0);
-      skinny_fetch<MBLK>(slot[u], ring_addr[u], wrow, w_off0, w_off1, ap, asp, bsp, min(kb + u + D, kb1 - 1), M);
+      skinny_fetch<MBLK, APRE>(slot[u], ring_addr[u], wrow, w_off0, w_off1, ap, asp, bsp, min(kb + u + D, kb1 - 1), M);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
 #define LLMMM_LAST(u)                                                              \
   if constexpr ((u) < D) {                                                         \
-    skinny_wait<(D - 1 - (u)) * LOADS, MBLK>(slot[u]);                             \
-    skinny_consume<MBLK>(slot[u], ring[u], w_rd, kb + (u) < kb1, acc);             \
+    skinny_wait<(D - 1 - (u)) * LOADS, MBLK, APRE>(slot[u]);                       \
+    skinny_consume<MBLK, APRE>(slot[u], ring[u], w_rd, kb + (u) < kb1, acc,        \
+                               a_tile + (min(kb + (u), kb1 - 1) - kb0) * (MBLK * 2048), a_rd); \
     __builtin_amdgcn_sched_barrier(0);                                             \
   }
   LLMMM_LAST(0) LLMMM_LAST(1) LLMMM_LAST(2) LLMMM_LAST(3) LLMMM_LAST(4) LLMMM_LAST(5) LLMMM_LAST(6) LLMMM_LAST(7)
@@ -206,54 +255,14 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   const int ncol = ng * 128 + wave * 16 + 4 * g;
 
   if (S > 1) {
-    // Partials travel through device-coherent (agent-scope, relaxed) stores and loads, which
-    // write through / read past the per-XCD L2.  That makes full release/acquire fences
-    // unnecessary: a fence at agent scope writes back and invalidates the whole L2 of the XCD,
-    // which costs far more than this kernel's entire run.
+    // split-K: this workgroup only stores its plane of partial sums; a second kernel adds the
+    // planes in split order 0..S-1 and runs the epilogue (fixed order, whatever the arrival order)
 #pragma unroll
     for (int mb = 0; mb < MBLK; ++mb) {
       const int m = m0 + mb * 16 + i;
-      if (m < M) {
-        float* dst = partial + ((size_t)sp * M + m) * N + ncol;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) __hip_atomic_store(dst + r, acc[mb][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+      if (m < M) *(f32x4*)(partial + ((size_t)sp * M + m) * N + ncol) = acc[mb];
     }
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): this wave's partial stores are acknowledged
-    __syncthreads();
-    if (tid == 0) {
-      const unsigned old = __hip_atomic_fetch_add(counters + cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      is_last            = (old == (unsigned)(S - 1));
-    }
-    __syncthreads();
-    if (!is_last) return;
-#pragma unroll
-    for (int mb = 0; mb < MBLK; ++mb) {
-      const int m = m0 + mb * 16 + i;
-      f32x4     t = {0.f, 0.f, 0.f, 0.f};
-      if (m < M) {
-        // fixed order 0..S-1, whoever arrived last; the loads of eight splits are put in flight
-        // together (one round trip per batch instead of one per split), the sums stay sequential
-        for (int s0 = 0; s0 < S; s0 += 8) {
-          f32x4 v[8];
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            const int    sc  = (s0 + u < S) ? s0 + u : S - 1;  // clamped duplicate: loaded, not added
-            const float* src = partial + ((size_t)sc * M + m) * N + ncol;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) v[u][r] = __hip_atomic_load(src + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
-#pragma unroll
-          for (int u = 0; u < 8; ++u)
-            if (s0 + u < S) {
-#pragma unroll
-              for (int r = 0; r < 4; ++r) t[r] += v[u][r];
-            }
-        }
-      }
-      acc[mb] = t;
-    }
-    if (tid == 0) __hip_atomic_store(counters + cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    return;
   }
 
   if constexpr (OUT == SK_OUT_F32) {
@@ -304,45 +313,60 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   }
 }
 
-template <int MBLK, int OUT, int D>
+template <int MBLK, int OUT, int D, int ASTG>
 static hipError_t launch_skinny(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
-                                int N, int K, int S, float* partial, unsigned* counters, hipStream_t stream)
+                                int N, int K, int S, float* partial, hipStream_t stream)
 {
-  hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D>), dim3(N / 128, S, (M + 63) / 64), dim3(512), 0, stream, (const uint8_t*)A, As,
-                     (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial, counters);
+  hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D, ASTG>), dim3(N / 128, S, (M + 63) / 64), dim3(512), 0, stream,
+                     (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial);
   return hipGetLastError();
 }
 
+// Ring depth D: the largest that does not exceed the slices of the shortest split.  Activation
+// staging: whenever the rows of the longest split fit next to the ring (28 KB beside the
+// 8-deep ring, 64 KB beside a 4-deep one); otherwise the per-slice register path.
 template <int OUT>
 static hipError_t dispatch_skinny(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
-                                  int N, int K, int S, float* partial, unsigned* counters, hipStream_t stream)
+                                  int N, int K, int S, float* partial, hipStream_t stream)
 {
-  const int slices = (K / 128) / S;  // of the shortest split
-#define LLMMM_GO(MBLK, D) return launch_skinny<MBLK, OUT, D>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, counters, stream)
+  const int KB     = K / 128;
+  const int slices = KB / S;              // of the shortest split
+  const int longest = (KB + S - 1) / S;   // of the longest
+#define LLMMM_GO(MBLK, D, ASTG) return launch_skinny<MBLK, OUT, D, ASTG>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, stream)
   if (M <= 16) {
-    if (slices >= 8) LLMMM_GO(1, 8);
-    if (slices >= 4) LLMMM_GO(1, 4);
-    LLMMM_GO(1, 2);
+    const int need = 2048 * longest;
+    if (slices >= 8 && need <= 28672) LLMMM_GO(1, 8, 28672);
+    if (slices >= 4 && need <= 65536) LLMMM_GO(1, 4, 65536);
+    if (need <= 65536) LLMMM_GO(1, 2, 65536);
+    if (slices >= 8) LLMMM_GO(1, 8, 0);
+    if (slices >= 4) LLMMM_GO(1, 4, 0);
+    LLMMM_GO(1, 2, 0);
   }
   if (M <= 32) {
-    if (slices >= 4) LLMMM_GO(2, 4);
-    LLMMM_GO(2, 2);
+    const int need = 2 * 2048 * longest;
+    if (slices >= 4 && need <= 65536) LLMMM_GO(2, 4, 65536);
+    if (need <= 65536) LLMMM_GO(2, 2, 65536);
+    if (slices >= 4) LLMMM_GO(2, 4, 0);
+    LLMMM_GO(2, 2, 0);
   }
   if (M <= 128) {  // two row groups of (up to) 64 when M > 64
-    if (slices >= 4) LLMMM_GO(4, 4);
-    LLMMM_GO(4, 2);
+    const int need = 4 * 2048 * longest;
+    if (slices >= 4 && need <= 65536) LLMMM_GO(4, 4, 65536);
+    if (need <= 65536) LLMMM_GO(4, 2, 65536);
+    if (slices >= 4) LLMMM_GO(4, 4, 0);
+    LLMMM_GO(4, 2, 0);
   }
 #undef LLMMM_GO
   return hipErrorInvalidValue;
 }
 
 hipError_t fp8_skinny_launch(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
-                             int M, int N, int K, int S, float* partial, unsigned* counters, hipStream_t stream)
+                             int M, int N, int K, int S, float* partial, hipStream_t stream)
 {
   switch (out_kind) {
-    case SK_OUT_F32: return dispatch_skinny<SK_OUT_F32>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, counters, stream);
-    case SK_OUT_BF16: return dispatch_skinny<SK_OUT_BF16>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, counters, stream);
-    case SK_OUT_FP8Q: return dispatch_skinny<SK_OUT_FP8Q>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, counters, stream);
+    case SK_OUT_F32: return dispatch_skinny<SK_OUT_F32>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, stream);
+    case SK_OUT_BF16: return dispatch_skinny<SK_OUT_BF16>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, stream);
+    case SK_OUT_FP8Q: return dispatch_skinny<SK_OUT_FP8Q>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, stream);
     default: return hipErrorInvalidValue;
   }
 }

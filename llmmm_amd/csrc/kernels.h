@@ -19,9 +19,13 @@ hipError_t fp16_gemm_launch(int dtype, int b_layout, int tile, const void* A, co
 hipError_t fp8_gemm_launch(int out_kind, int tile, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
                            float* Cs, int M, int N, int K, int S, float* planes, hipStream_t stream);
 
-// M <= 128 (row groups of 64); S splits of K; partial [S][M][N] fp32 and counters [N/128 * ceil(M/64)] are only touched when S > 1.
+// C = epilogue(planes[0] + planes[1] + ... + planes[S-1]) (that order), planes of M * N floats each.
+hipError_t fp8_splitk_reduce_launch(int out_kind, const float* planes, int S, void* C, float* Cs, int M, int N, hipStream_t stream);
+
+// M <= 128 (row groups of 64); S splits of K.  S == 1: complete result in C / Cs.  S > 1: only the S
+// partial planes `partial` [S][M][N] fp32 are written; run fp8_splitk_reduce_launch behind it.
 hipError_t fp8_skinny_launch(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
-                             int M, int N, int K, int S, float* partial, unsigned* counters, hipStream_t stream);
+                             int M, int N, int K, int S, float* partial, hipStream_t stream);
 
 hipError_t quant_fp8_launch(int quant_m, int transpose, const float* x, void* q, float* scale, int M, int N, hipStream_t stream);
 

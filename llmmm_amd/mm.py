@@ -115,13 +115,11 @@ def workspace_bytes(out_kind, M, N, K):
 
 
 def make_workspace(out_kind, M, N, K, device="cuda", stream=None):
-    """Allocate and initialise a split-K workspace for this shape (None when none is needed)."""
+    """Allocate a split-K workspace for this shape (None when none is needed); plain scratch, no initialisation."""
     n = workspace_bytes(out_kind, M, N, K)
     if n == 0:
         return None
-    ws = torch.empty(n, dtype=torch.uint8, device=device)
-    check(lib.llmmm_workspace_init(ctypes.c_void_p(ws.data_ptr()), n, _stream(stream)))
-    return ws
+    return torch.empty(n, dtype=torch.uint8, device=device)
 
 
 def query_config(out_kind, M, N, K):

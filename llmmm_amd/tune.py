@@ -67,14 +67,14 @@ def tune_shape(M, N, K, iters=40, rotate_bytes=768 << 20, verbose=True):
     kb = K // 128
     tile_splits = [x for x in (1, 2, 3, 4, 5, 6, 8) if x <= max(1, kb // 2)]
     max_split = min(32, kb) if skinny else max(tile_splits)
-    ws = torch.zeros(4096 + max_split * M * N * 4, dtype=torch.uint8, device="cuda")  # zeroed counters + partial planes
+    ws = torch.empty(max_split * M * N * 4, dtype=torch.uint8, device="cuda")  # partial planes
     cands = []
     if skinny:
         kb = K // 128
         cands = [(_lib.TILE_SKINNY, s) for s in sorted({1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 19, 20, 24, 32, kb, kb // 2}) if 1 <= s <= min(32, kb)]
     if M % 128 == 0:
         dims = {_lib.TILE_256x256: (256, 256), _lib.TILE_128x256: (128, 256), _lib.TILE_256x128: (256, 128), _lib.TILE_128x128: (128, 128)}
-        cands = (cands if skinny and M % 128 else []) + [(t, x) for t, (bm, bn) in dims.items() if M % bm == 0 and N % bn == 0
+        cands = (cands if skinny else []) + [(t, x) for t, (bm, bn) in dims.items() if M % bm == 0 and N % bn == 0
                                                           for x in tile_splits if x == 1 or (M // bm) * (N // bn) * x <= 640]
     results = {}
     for tile, split in cands:

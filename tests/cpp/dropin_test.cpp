@@ -93,7 +93,7 @@ int main()
   fails += f8;
   if (!throws_with([&] { LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dAq, dAs, dBq, dBs, dC32, M, 100, K, nullptr); },
                    "M or N or K are not aligned.")) { ++fails; printf("fp8 misaligned N: FAIL\n"); }
-  if (!throws_with([&] { LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(dAq, dAs, dBq, dBs, dCq, dCs, 100, N, K, nullptr); },
+  if (!throws_with([&] { LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(dAq, dAs, dBq, dBs, dCq, dCs, 200, N, K, nullptr); },
                    "M or N or K are not aligned.")) { ++fails; printf("fp8 misaligned M: FAIL\n"); }
   printf(fails ? "DROPIN FAIL (%d)\n" : "DROPIN OK\n", fails);
   return fails ? 1 : 0;

@@ -25,8 +25,8 @@ def _run_all(lib, Aq, As, Bq, Bs, tile=-1, split_k=0, use_ws=True):
     N = Bq.shape[0]
     t = _gpu(Aq, As, Bq, Bs)
     ws = lib.make_workspace(2, M, N, K) if use_ws else None
-    if use_ws and split_k > 1:  # an explicit split: 4 KiB of counters + split_k partial planes, zero-initialised
-        ws = torch.zeros(4096 + split_k * M * N * 4, dtype=torch.uint8, device="cuda")
+    if use_ws and split_k > 1:  # an explicit split: split_k partial planes; poisoned, the library must not rely on their content
+        ws = torch.full((split_k * M * N * 4,), 0xFF, dtype=torch.uint8, device="cuda")
     C = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda")
     Cb = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
     Cq = torch.full((M, N), 0x55, dtype=torch.uint8, device="cuda")
@@ -142,8 +142,7 @@ def test_skinny_without_workspace_does_not_split(lib, oracle):
 
 
 def test_split_k_is_deterministic_and_reusable(lib, oracle):
-    # fixed-order reduction: bit-identical results run after run on the same workspace; the counters
-    # return to zero, so the workspace needs no re-initialisation between calls
+    # fixed-order reduction: bit-identical results run after run on the same (never initialised) workspace
     M, N, K = 16, 2560, 4096
     Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=4)
     t = _gpu(Aq, As, Bq, Bs)
@@ -160,7 +159,6 @@ def test_split_k_is_deterministic_and_reusable(lib, oracle):
     for o in outs[1:]:
         assert all(torch.equal(a, b) for a, b in zip(o, outs[0]))
     assert_fp8_gemm_close(outs[0][2].cpu().numpy(), oracle.fp8_gemm(Aq, As, Bq, Bs), "split-K auto")
-    assert int(ws[:4096].view(torch.int32).abs().sum()) == 0, "arrival counters must be back at zero"
 
 
 @pytest.mark.parametrize("name,N,K", [("qkv", 6144, 2560), ("o", 2560, 4096), ("gate_up", 19456, 2560), ("down", 2560, 9728)])
