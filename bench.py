@@ -38,9 +38,9 @@ QWEN3_4B = {"qkv": (6144, 2560), "o": (2560, 4096), "gate_up": (19456, 2560), "d
 
 def _events_ms(fn, steps, warmup, graph=False):
     """Average duration of one call of fn, HIP events on torch's current stream (the stream
-    every launch below is enqueued on).  With graph=True the `steps` launches are captured into
-    one HIP graph and replayed, so that microsecond kernels are timed back-to-back on the GPU
-    instead of at the pace of the Python launch loop."""
+    every launch below is enqueued on).  With graph=True (every GEMM workload) the `steps` launches
+    are captured into one HIP graph and replayed once inside the timed region, so that kernels are
+    timed back-to-back on the GPU instead of at the pace of the Python launch loop."""
     # Untimed pre-heat: the GPU's clocks take tens of milliseconds of sustained load to settle, far
     # longer than a handful of warm-up launches of a ~100 us kernel; time the settled state.
     t_heat = time.perf_counter()
@@ -58,7 +58,8 @@ def _events_ms(fn, steps, warmup, graph=False):
         with torch.cuda.graph(g):
             for _ in range(steps):
                 fn()
-        g.replay()  # untimed replay: graph upload
+        for _ in range(3):  # untimed replays: graph upload, and the clocks back up after the idle capture
+            g.replay()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         e0.record()
@@ -107,7 +108,7 @@ def bench_fp16(M, N, K, steps, warmup, dtype=torch.float16, b_transposed=False):
     if b_transposed:
         B = B.t().contiguous()
     C = torch.empty((M, N), dtype=dtype, device="cuda")
-    ms, wall = _events_ms(lambda: llmmm_amd.fp16_gemm(A, B, C, b_transposed=b_transposed), steps, warmup)
+    ms, wall = _events_ms(lambda: llmmm_amd.fp16_gemm(A, B, C, b_transposed=b_transposed), steps, warmup, graph=True)
     flops = 2.0 * M * N * K
     return {"ms": ms, "wall_ms": wall, "tflops": flops / ms * 1e-9, "bytes": 2.0 * (M * K + K * N + M * N)}, (A, B, C)
 
@@ -149,7 +150,7 @@ def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0):
         else:
             fns[out](Aq, As, Bq, Bs, C, M, N, K, workspace=ws)
 
-    ms, wall = _events_ms(step, steps, warmup, graph=(M <= 128))
+    ms, wall = _events_ms(step, steps, warmup, graph=True)
     flops = 2.0 * M * N * K
     nbytes = fp8_bytes(M, N, K, out)
     tile, split = llmmm_amd.query_config(kind, M, N, K)

@@ -6,18 +6,23 @@
 //
 // Design (nothing here is translated from the reference's mma.sync/ldmatrix code):
 //  * one workgroup computes a BM x BN tile, one wavefront a 64(m) x 128(n) sub-tile built from
-//    v_mfma_f32_32x32x16_{f16,bf16}; the MFMA is issued with B as the row operand and A as the
-//    column operand so that each lane ends up with 4 consecutive n of one row m (packed stores);
-//  * K advances 32 elements per stage (64 bytes per tile row, (BM+BN)*64 bytes of LDS) and four
-//    stages form a ring that LDS-direct global loads fill three stages ahead of the MFMAs
-//    (no staging registers, no ds_write);
-//  * the single workgroup barrier of a stage sits between its two 16-wide k-steps: by then
-//    every wave has pulled the stage's operands into registers, so the barrier both frees the
-//    stage's buffer for the load of stage +4 and publishes stage +1, whose first fragments are
-//    fetched right behind it -- no wave ever waits on an LDS read it has just issued;
-//  * A (and Bt) tiles are K-major and read with ds_read_b128 through the SWZ_ROW64 placement;
-//    a row-major B tile is kept as [k][n] and read with the transposing ds_read_b64_tr_b16,
-//    its 64-byte column chunks XOR-ed with k&3;
+//    v_mfma_f32_16x16x32_{f16,bf16}.  On this power-limited part the 16x16x32 shape sustains
+//    about 16 % more FLOP/s than 32x32x16 on random operands (same peak, less energy per
+//    FLOP), which is why it is used although it needs twice the instructions.  The MFMA is
+//    issued with B as the row operand and A as the column operand, so that each lane ends up
+//    with 4 consecutive n of one row m;
+//  * K advances 32 elements per stage = one MFMA k-step (64 bytes per tile row, (BM+BN)*64 bytes
+//    of LDS) and four stages form a ring that LDS-direct global loads fill three stages ahead
+//    of the MFMAs (no staging registers, no ds_write);
+//  * the single workgroup barrier of a stage sits in its middle, between the MFMAs of the wave's
+//    left and right 64 columns: by then every wave has pulled the stage's operands into
+//    registers, so the barrier both frees the stage's buffer for the load of stage +4 and
+//    publishes stage +1, whose first fragments are fetched right behind it -- no wave ever waits
+//    on an LDS read it has just issued;
+//  * A (and Bt) tiles are K-major and read with one ds_read_b128 per 16-row fragment (chunk
+//    XOR-ed with row bit 3: conflict-free); a row-major B tile is kept as [k][n] and read with
+//    the transposing ds_read_b64_tr_b16, its 32-byte column chunks XOR-ed with k bits 0, 1, 3;
+//  * the epilogue lays each wave's result out row-major in LDS and stores whole rows;
 //  * workgroup ids are remapped so that the tiles resident on one XCD share A/B panels in its L2.
 #include "device_common.hip.h"
 #include "kernels.h"
@@ -25,16 +30,16 @@
 namespace llmmm {
 
 template <typename T>
-struct Mfma16;
+struct Mfma32;
 template <>
-struct Mfma16<_Float16> {
+struct Mfma32<_Float16> {
   typedef f16x8 vec;
-  static __device__ __forceinline__ f32x16 run(vec x, vec y, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(x, y, c, 0, 0, 0); }
+  static __device__ __forceinline__ f32x4 run(vec x, vec y, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y, c, 0, 0, 0); }
 };
 template <>
-struct Mfma16<__bf16> {
+struct Mfma32<__bf16> {
   typedef bf16x8 vec;
-  static __device__ __forceinline__ f32x16 run(vec x, vec y, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(x, y, c, 0, 0, 0); }
+  static __device__ __forceinline__ f32x4 run(vec x, vec y, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, c, 0, 0, 0); }
 };
 
 template <typename T, int BM, int BN, bool B_NK>
@@ -57,91 +62,108 @@ struct Fp16Tile {
   static constexpr int B_KROWS_PER_LOAD = B_KROWS_PER_GRP * NW;
 };
 
-// Issue the LDS-direct loads of one stage.  `kleft` = K - k0 (elements still to go); a stage
-// whose K range is cut short zero-fills the missing part so that the MFMAs need no masking.
-// All loads of a wave share one per-lane offset: they differ by a wave-uniform row (or k) step
-// that the swizzles do not see.  The loads are inline assembly with the wave-uniform part of the
-// address in SGPRs: no vector ALU work goes into addresses, and the compiler -- which would
-// turn every wait it inserts into "all loads done" while it knows of an LDS-direct load in
-// flight -- never sees them; the kernel places the s_waitcnt vmcnt itself.
+// K-major tile of 64-byte rows read as 16-row fragments: lanes 16g..16g+15 take 16 consecutive
+// rows at chunk g.  Four rows fill a 256-byte bank row; XOR-ing row bit 3 into chunk bit 1 keeps
+// the 16 lanes of every ds_read_b128 pass on 16 different 16-byte slots.
+__device__ __forceinline__ int k64_swz(int r) { return ((r >> 3) & 1) << 1; }
+__device__ __forceinline__ int k64_offset(int r, int c) { return r * 64 + ((c ^ k64_swz(r)) << 4); }
+// [k][n] tile: the 32-byte column chunk of row k is XOR-ed with k bits 0, 1 and 3, which keeps
+// the 4 x 4 row/chunk patches of a transposing 64-bit read on different banks.
+__device__ __forceinline__ int kn_swz(int k) { return (k & 3) | (((k >> 3) & 1) << 2); }
+
+// LDS-direct load as inline assembly with the wave-uniform part of the address in SGPRs: no
+// vector ALU work goes into addresses, and the compiler -- which would turn every wait it
+// inserts into "all loads done" while it knows of an LDS-direct load in flight -- never sees
+// it; the kernel places the s_waitcnt vmcnt itself.
 __device__ __forceinline__ void sload_lds_16B(const void* sbase, unsigned voff, unsigned lds_addr)
 {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr) : "memory");
 }
+
+// Per-lane loader state.  The loads of a wave for the K-major tiles share one byte offset (they
+// differ by a wave-uniform row step that the swizzle does not see); those of the [k][n] tile
+// get one offset each, because their k step may flip the swizzle.
+template <int B_LOADS>
+struct Fp16Loader {
+  unsigned a_off;          // bytes
+  int      a_k;            // k offset (elements) of the lane's chunk inside a stage
+  unsigned b_off[B_LOADS]; // bytes
+  int      b_k[B_LOADS];   // K-major: k offset of the chunk; [k][n]: k row of the lane
+};
+
+// Issue the LDS-direct loads of one stage.  `kleft` = K - k0 (elements still to go); a stage
+// whose K range is cut short zero-fills the missing part so that the MFMAs need no masking.
 template <typename T, int BM, int BN, bool B_NK, bool KTAIL>
 __device__ __forceinline__ void fp16_issue_stage(char LLMMM_LDS* lds, unsigned lds_addr, const T* __restrict__ Ag, const T* __restrict__ Bg,
-                                                 unsigned a_off, int a_k, unsigned b_off, int b_k, int K, int N, int wave,
-                                                 int lane, int kleft)
+                                                 const Fp16Loader<Fp16Tile<T, BM, BN, B_NK>::B_LOADS>& ld, int K, int N, int wave, int lane,
+                                                 int kleft)
 {
   typedef Fp16Tile<T, BM, BN, B_NK> TC;
-  // without a K tail (K % 32 == 0) the loads are unconditional: straight-line code keeps the
-  // compiler's wait-count bookkeeping exact
+  // without a K tail (K % 32 == 0) the loads are unconditional straight-line code
   const bool full = !KTAIL || kleft >= TC::BK;
 #pragma unroll
   for (int i = 0; i < TC::A_LOADS; ++i) {
-    char LLMMM_LDS* dst = lds + (wave + i * TC::NW) * 1024;
-    if (full || a_k < kleft)
-      sload_lds_16B(Ag + (size_t)(TC::ROWS_PER_LOAD * i) * K, a_off * 2u, lds_addr + (wave + i * TC::NW) * 1024);
+    if (full || ld.a_k < kleft)
+      sload_lds_16B(Ag + (size_t)(TC::ROWS_PER_LOAD * i) * K, ld.a_off, lds_addr + (wave + i * TC::NW) * 1024);
     else
-      *(i32x4 LLMMM_LDS*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
+      *(i32x4 LLMMM_LDS*)(lds + (wave + i * TC::NW) * 1024 + lane * 16) = i32x4{0, 0, 0, 0};
   }
-  char LLMMM_LDS* ldsB = lds + TC::A_BYTES;
 #pragma unroll
   for (int i = 0; i < TC::B_LOADS; ++i) {
-    char LLMMM_LDS* dst = ldsB + (wave + i * TC::NW) * 1024;
-    if constexpr (B_NK) {
-      if (full || b_k < kleft)
-        sload_lds_16B(Bg + (size_t)(TC::ROWS_PER_LOAD * i) * K, b_off * 2u, lds_addr + TC::A_BYTES + (wave + i * TC::NW) * 1024);
+    const unsigned dst = TC::A_BYTES + (wave + i * TC::NW) * 1024;
+    if (full || ld.b_k[i] < kleft) {
+      if constexpr (B_NK)
+        sload_lds_16B(Bg + (size_t)(TC::ROWS_PER_LOAD * i) * K, ld.b_off[i], lds_addr + dst);
       else
-        *(i32x4 LLMMM_LDS*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
+        sload_lds_16B(Bg + (size_t)(TC::B_KROWS_PER_LOAD * i) * N, ld.b_off[i], lds_addr + dst);
     }
-    else {
-      if (full || b_k + TC::B_KROWS_PER_LOAD * i < kleft)
-        sload_lds_16B(Bg + (size_t)(TC::B_KROWS_PER_LOAD * i) * N, b_off * 2u, lds_addr + TC::A_BYTES + (wave + i * TC::NW) * 1024);
-      else
-        *(i32x4 LLMMM_LDS*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
-    }
+    else
+      *(i32x4 LLMMM_LDS*)(lds + dst + lane * 16) = i32x4{0, 0, 0, 0};
   }
 }
 
-// Operand fragments of one 16-wide k-step (ks = 0 or 1 inside a stage): a[mf] = 32 rows of A,
-// b[nf] = 32 rows of B^T.
+// The four 16-row A fragments of a stage.
 template <typename T, int BM, int BN, bool B_NK>
-__device__ __forceinline__ void fp16_read_frags(const char LLMMM_LDS* lds, int a_rd, const int (&b_rd)[4], int ks,
-                                                typename Mfma16<T>::vec (&a)[2], typename Mfma16<T>::vec (&b)[4])
+__device__ __forceinline__ void fp16_read_a(const char LLMMM_LDS* lds, int a_rd, typename Mfma32<T>::vec (&a)[4])
+{
+  typedef typename Mfma32<T>::vec vec;
+#pragma unroll
+  for (int mf = 0; mf < 4; ++mf) a[mf] = *(const vec LLMMM_LDS*)(lds + a_rd + mf * 1024);
+}
+// Four 16-column B fragments: nf = 4*half .. 4*half+3.
+template <typename T, int BM, int BN, bool B_NK>
+__device__ __forceinline__ void fp16_read_b(const char LLMMM_LDS* lds, const int (&b_rd)[8], int half, typename Mfma32<T>::vec (&b)[4])
 {
   typedef Fp16Tile<T, BM, BN, B_NK> TC;
-  typedef typename Mfma16<T>::vec   vec;
-  const char LLMMM_LDS*             ldsA = lds;
+  typedef typename Mfma32<T>::vec   vec;
   const char LLMMM_LDS*             ldsB = lds + TC::A_BYTES;
 #pragma unroll
-  for (int mf = 0; mf < 2; ++mf) a[mf] = *(const vec LLMMM_LDS*)(ldsA + (a_rd ^ (ks << 5)) + mf * 2048);
-#pragma unroll
-  for (int nf = 0; nf < 4; ++nf) {
+  for (int q = 0; q < 4; ++q) {
+    const int nf = 4 * half + q;
     if constexpr (B_NK) {
-      b[nf] = *(const vec LLMMM_LDS*)(ldsB + (b_rd[0] ^ (ks << 5)) + nf * 2048);
+      b[q] = *(const vec LLMMM_LDS*)(ldsB + b_rd[0] + nf * 1024);
     }
     else {
       union {
         i16x4 h[2];
         vec   v;
       } u;
-      u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 LLMMM_LDS*)(ldsB + b_rd[nf] + (ks * 16) * TC::B_ROW));
-      u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 LLMMM_LDS*)(ldsB + b_rd[nf] + (ks * 16 + 4) * TC::B_ROW));
-      b[nf]  = u.v;
+      u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 LLMMM_LDS*)(ldsB + b_rd[nf]));
+      u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((i16x4 LLMMM_LDS*)(ldsB + b_rd[nf] + 4 * TC::B_ROW));
+      b[q]   = u.v;
     }
   }
 }
 
-// Half of a k-step: the 4 MFMAs of fragments nf = 2h, 2h+1.
+// 8 MFMAs: fragments nf = 4*half + 2*part, +1 against the four row fragments.
 template <typename T>
-__device__ __forceinline__ void fp16_mfma_half(int h, const typename Mfma16<T>::vec (&a)[2], const typename Mfma16<T>::vec (&b)[4],
-                                               f32x16 (&acc)[4][2])
+__device__ __forceinline__ void fp16_mfma8(int half, int part, const typename Mfma32<T>::vec (&a)[4], const typename Mfma32<T>::vec (&b)[4],
+                                           f32x4 (&acc)[8][4])
 {
 #pragma unroll
-  for (int nf = 2 * h; nf < 2 * h + 2; ++nf)
+  for (int q = 2 * part; q < 2 * part + 2; ++q)
 #pragma unroll
-    for (int mf = 0; mf < 2; ++mf) acc[nf][mf] = Mfma16<T>::run(b[nf], a[mf], acc[nf][mf]);
+    for (int mf = 0; mf < 4; ++mf) acc[4 * half + q][mf] = Mfma32<T>::run(b[q], a[mf], acc[4 * half + q][mf]);
 }
 
 template <typename T, int BM, int BN, bool B_NK, bool KTAIL>
@@ -149,7 +171,7 @@ __global__ void __launch_bounds__((BM / 64) * (BN / 128) * 64)
 fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n)
 {
   typedef Fp16Tile<T, BM, BN, B_NK> TC;
-  typedef typename Mfma16<T>::vec   vec;
+  typedef typename Mfma32<T>::vec   vec;
   __shared__ __attribute__((aligned(1024))) char lds_raw[4 * TC::STAGE];  // the ring of four stages
 
   const int tid  = threadIdx.x;
@@ -161,48 +183,55 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
   tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
 
-  // ---- loader setup
-  const KMajorLane lp    = kmajor_lane<SWZ_ROW64>(wave, lane);
-  const unsigned   a_off = (unsigned)(lp.row * K + lp.chunk * 8);
-  const int        a_k   = lp.chunk * 8;
-  unsigned         b_off;
-  int              b_k;
-  if constexpr (B_NK) {
-    b_off = a_off;
-    b_k   = a_k;
-  }
-  else {
-    const int k     = wave * TC::B_KROWS_PER_GRP + (lane * 16) / TC::B_ROW;
-    const int pbyte = (lane * 16) % TC::B_ROW;
-    const int ch    = (pbyte >> 6) ^ (k & 3);
-    b_off           = (unsigned)(k * N + ((ch << 6) + (pbyte & 63)) / 2);
-    b_k             = k;
+  // ---- loader setup: lane -> what the 16 bytes at (1 KB group base + 16*lane) must hold
+  Fp16Loader<TC::B_LOADS> ld;
+  {
+    const int r = wave * 16 + (lane >> 2);          // tile row of the first group; later groups add 16*NW rows
+    const int c = (lane & 3) ^ k64_swz(r);          // logical chunk placed at physical chunk lane%4
+    ld.a_off    = (unsigned)(r * K + c * 8) * 2u;
+    ld.a_k      = c * 8;
+#pragma unroll
+    for (int i = 0; i < TC::B_LOADS; ++i) {
+      if constexpr (B_NK) {
+        ld.b_off[i] = ld.a_off;
+        ld.b_k[i]   = ld.a_k;
+      }
+      else {
+        const int k     = (wave + i * TC::NW) * TC::B_KROWS_PER_GRP + (lane * 16) / TC::B_ROW;
+        const int pbyte = (lane * 16) % TC::B_ROW;
+        const int ch    = (pbyte >> 5) ^ kn_swz(k);  // logical 32-byte chunk stored at physical chunk pbyte/32
+        // the base pointer of load i already advances by B_KROWS_PER_LOAD * i rows
+        ld.b_off[i] = (unsigned)((k - i * TC::B_KROWS_PER_LOAD) * N + ((ch << 5) + (pbyte & 31)) / 2) * 2u;
+        ld.b_k[i]   = k;
+      }
+    }
   }
   const T* Ag = A + (size_t)m0 * K;
   const T* Bg = B_NK ? B + (size_t)n0 * K : B + n0;
 
-  // ---- operand read setup (byte offsets inside a stage)
-  const int hi   = lane >> 5;
-  const int a_rd = kmajor_offset<SWZ_ROW64>(wm * 64 + (lane & 31), hi);
-  int       b_rd[4];
+  // ---- operand read setup (byte offsets inside a stage).  lane = (g = lane/16, i = lane%16):
+  // row i of a 16-row fragment, k = 8g .. 8g+7
+  const int g    = lane >> 4;
+  const int li   = lane & 15;
+  const int a_rd = k64_offset(wm * 64 + li, g);
+  int       b_rd[8];
   if constexpr (B_NK) {
-    b_rd[0] = kmajor_offset<SWZ_ROW64>(wn * 128 + (lane & 31), hi);
-    b_rd[1] = b_rd[2] = b_rd[3] = 0;
+    b_rd[0] = k64_offset(wn * 128 + li, g);
+#pragma unroll
+    for (int nf = 1; nf < 8; ++nf) b_rd[nf] = 0;
   }
   else {
-    const int blk = lane >> 4, i = lane & 15;
+    // transposing read: inside the 16-lane block, lane j supplies the 8 bytes (4 columns) j%4 of k row 8g + j/4
+    const int k = 8 * g + (li >> 2);
 #pragma unroll
-    for (int nf = 0; nf < 4; ++nf)
-      b_rd[nf] = (8 * (blk >> 1) + (i >> 2)) * TC::B_ROW + (((wn * 4 + nf) ^ (i >> 2)) << 6) + (blk & 1) * 32 + (i & 3) * 8;
+    for (int nf = 0; nf < 8; ++nf) b_rd[nf] = k * TC::B_ROW + (((wn * 8 + nf) ^ kn_swz(k)) << 5) + (li & 3) * 8;
   }
 
-  f32x16 acc[4][2];
+  f32x4 acc[8][4];
 #pragma unroll
-  for (int nf = 0; nf < 4; ++nf)
+  for (int nf = 0; nf < 8; ++nf)
 #pragma unroll
-    for (int mf = 0; mf < 2; ++mf)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[nf][mf][r] = 0.0f;
+    for (int mf = 0; mf < 4; ++mf) acc[nf][mf] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int    KT          = (K + TC::BK - 1) / TC::BK;
   const int    full_stages = K / TC::BK;
@@ -213,9 +242,9 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
   const unsigned        lds_base = (unsigned)(size_t)lds;  // the same buffers as LDS byte addresses, for the loader
   const unsigned ring_addr[4]    = {lds_base, lds_base + TC::STAGE, lds_base + 2 * TC::STAGE, lds_base + 3 * TC::STAGE};
 
-#define LLMMM_ISSUE(stage, buf)                                                                                              \
-  fp16_issue_stage<T, BM, BN, B_NK, KTAIL>(ring[buf], ring_addr[buf], Ag + (size_t)(stage) * TC::BK, Bg + (size_t)(stage) * b_step, a_off, a_k, b_off, \
-                                    b_k, K, N, wave, lane, K - (stage) * TC::BK)
+#define LLMMM_ISSUE(stage, buf)                                                                                                     \
+  fp16_issue_stage<T, BM, BN, B_NK, KTAIL>(ring[buf], ring_addr[buf], Ag + (size_t)(stage) * TC::BK, Bg + (size_t)(stage) * b_step, ld, K, \
+                                           N, wave, lane, K - (stage) * TC::BK)
 
   // prologue: stages 0..2 in flight, stage 0 landed and published, then stage 3 behind the barrier
   LLMMM_ISSUE(0, 0);
@@ -225,21 +254,20 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
   __builtin_amdgcn_s_barrier();
   if (3 < KT) LLMMM_ISSUE(3, 3);
 
-  vec a0[2], b0[4], a1[2], b1[4];
-  fp16_read_frags<T, BM, BN, B_NK>(ring[0], a_rd, b_rd, 0, a0, b0);
+  vec aX[4], aY[4], bL[4], bR[4];  // A fragments of the current / next stage; B fragments of the left / right 64 columns
+  fp16_read_a<T, BM, BN, B_NK>(ring[0], a_rd, aX);
+  fp16_read_b<T, BM, BN, B_NK>(ring[0], b_rd, 0, bL);
 
-  // One stage s (in ring[u]).  STEADY = "stages s+1 .. s+4 exist and are full" (straight-line code).
-  // The LDS reads of the next k-step are issued between the two MFMA halves of the current one:
-  // by the time their data is needed four MFMAs (>= 128 cycles) have been issued behind them.
-  // (While LDS-direct loads are in flight the compiler only ever waits for *all* LDS reads, so a
-  // read must never be issued right before a wait.)
-#define LLMMM_STAGE(STEADY, s, u)                                                                                  \
+  // One stage s (in ring[u]) with its A fragments in aC; aN receives those of stage s+1.
+  // STEADY = "stages s+1 .. s+4 exist and are full" (straight-line code).  LDS reads are always
+  // issued between two groups of 8 MFMAs, a whole group (>= 128 cycles) before their data is used.
+#define LLMMM_STAGE(STEADY, s, u, aC, aN)                                                                          \
   {                                                                                                                \
-    fp16_mfma_half<T>(0, a0, b0, acc);                                                                             \
+    fp16_mfma8<T>(0, 0, aC, bL, acc);                                                                              \
     __builtin_amdgcn_sched_barrier(0);                                                                             \
-    fp16_read_frags<T, BM, BN, B_NK>(ring[u], a_rd, b_rd, 1, a1, b1);                                              \
+    fp16_read_b<T, BM, BN, B_NK>(ring[u], b_rd, 1, bR);                                                            \
     __builtin_amdgcn_sched_barrier(0);                                                                             \
-    fp16_mfma_half<T>(1, a0, b0, acc);                                                                             \
+    fp16_mfma8<T>(0, 1, aC, bL, acc);                                                                              \
     __builtin_amdgcn_sched_barrier(0);                                                                             \
     /* every LDS read of stage s has been issued; once they are back (lgkmcnt(0), part of each wait below) the */ \
     /* barrier hands ring[u] to the loader and publishes stage s+1 */                                             \
@@ -251,33 +279,34 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
       wait_vmcnt<0>();                                                                                             \
     __builtin_amdgcn_s_barrier();                                                                                  \
     if (STEADY || (s) + 4 < KT) LLMMM_ISSUE((s) + 4, u);                                                           \
-    fp16_mfma_half<T>(0, a1, b1, acc);                                                                             \
+    fp16_mfma8<T>(1, 0, aC, bR, acc);                                                                              \
     __builtin_amdgcn_sched_barrier(0);                                                                             \
     /* unconditional: after the last stage this reads a stale buffer and the result is unused */                  \
-    fp16_read_frags<T, BM, BN, B_NK>(ring[((u) + 1) & 3], a_rd, b_rd, 0, a0, b0);                                  \
+    fp16_read_a<T, BM, BN, B_NK>(ring[((u) + 1) & 3], a_rd, aN);                                                   \
+    fp16_read_b<T, BM, BN, B_NK>(ring[((u) + 1) & 3], b_rd, 0, bL);                                                \
     __builtin_amdgcn_sched_barrier(0);                                                                             \
-    fp16_mfma_half<T>(1, a1, b1, acc);                                                                             \
+    fp16_mfma8<T>(1, 1, aC, bR, acc);                                                                              \
     __builtin_amdgcn_sched_barrier(0);                                                                             \
   }
 
   int kt = 0;
   for (; kt + 8 <= full_stages; kt += 4) {
-    LLMMM_STAGE(true, kt + 0, 0)
-    LLMMM_STAGE(true, kt + 1, 1)
-    LLMMM_STAGE(true, kt + 2, 2)
-    LLMMM_STAGE(true, kt + 3, 3)
+    LLMMM_STAGE(true, kt + 0, 0, aX, aY)
+    LLMMM_STAGE(true, kt + 1, 1, aY, aX)
+    LLMMM_STAGE(true, kt + 2, 2, aX, aY)
+    LLMMM_STAGE(true, kt + 3, 3, aY, aX)
   }
   for (; kt < KT; kt += 4) {
-    if (kt + 0 < KT) LLMMM_STAGE(false, kt + 0, 0)
-    if (kt + 1 < KT) LLMMM_STAGE(false, kt + 1, 1)
-    if (kt + 2 < KT) LLMMM_STAGE(false, kt + 2, 2)
-    if (kt + 3 < KT) LLMMM_STAGE(false, kt + 3, 3)
+    if (kt + 0 < KT) LLMMM_STAGE(false, kt + 0, 0, aX, aY)
+    if (kt + 1 < KT) LLMMM_STAGE(false, kt + 1, 1, aY, aX)
+    if (kt + 2 < KT) LLMMM_STAGE(false, kt + 2, 2, aX, aY)
+    if (kt + 3 < KT) LLMMM_STAGE(false, kt + 3, 3, aY, aX)
   }
 #undef LLMMM_STAGE
 #undef LLMMM_ISSUE
 
-  // ---- epilogue: lane holds, for row m = ..+lane%32, the columns 8*(r/4) + 4*(lane/32) + r%4.
-  // Stored straight from this layout, one instruction would write 16 bytes to each of 32 rows,
+  // ---- epilogue: lane (g, li) holds rows m = .. + mf*16 + li, columns nf*16 + 4g + r.
+  // Stored straight from this layout, one instruction would write 8 bytes to each of 16 rows,
   // and the memory pipeline pays per row segment.  Instead every wave lays its 64 x 128 result
   // out row-major (256-byte rows, 16-byte chunks XOR-ed with the row so that the ds_read_b128
   // below is conflict-free) in a private 16 KB piece of the ring and stores whole rows, 16
@@ -287,20 +316,18 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
     typedef T             tx4 __attribute__((ext_vector_type(4)));
     char LLMMM_LDS* const stg = lds + wave * 16384;
 #pragma unroll
-    for (int mf = 0; mf < 2; ++mf) {
-      const int r = mf * 32 + (lane & 31);
+    for (int mf = 0; mf < 4; ++mf) {
+      const int r = mf * 16 + li;
 #pragma unroll
-      for (int nf = 0; nf < 4; ++nf)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const f32x16& v = acc[nf][mf];
-          tx4           o;
-          o[0] = (T)v[4 * q + 0];
-          o[1] = (T)v[4 * q + 1];
-          o[2] = (T)v[4 * q + 2];
-          o[3] = (T)v[4 * q + 3];
-          *(tx4 LLMMM_LDS*)(stg + r * 256 + (((nf * 4 + q) ^ (r & 15)) << 4) + 8 * hi) = o;
-        }
+      for (int nf = 0; nf < 8; ++nf) {
+        const f32x4 v = acc[nf][mf];
+        tx4         o;
+        o[0] = (T)v[0];
+        o[1] = (T)v[1];
+        o[2] = (T)v[2];
+        o[3] = (T)v[3];
+        *(tx4 LLMMM_LDS*)(stg + r * 256 + (((nf * 2 + (g >> 1)) ^ (r & 15)) << 4) + 8 * (g & 1)) = o;
+      }
     }
     T* cbase = C + (size_t)(m0 + wm * 64) * N + n0 + wn * 128;
 #pragma unroll
