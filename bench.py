@@ -176,8 +176,8 @@ def cpu_baseline_fp16(M, N, K, rows):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="fp16_gemm_4096",
                     help="fp16_gemm_4096 (headline) | fp8_gemm_fused_4096 | fp8_gemm_bf16_4096 | bf16_gemm_4096 | "
                          "decode_<qkv|o|gate_up|down>_m<M> | copy_1g (counter calibration only)")
