@@ -40,10 +40,10 @@ int max_split_for(int K) { return (K / 128) < MAX_SPLIT_K ? (K / 128) : MAX_SPLI
 // that the activation rows of a split can be staged in LDS (64 KB: 32 slices of 16 rows).
 int heuristic_split(int M, int N, int K)
 {
-  const int groups = (N / 128) * ((M + 63) / 64), kb = K / 128;
+  const int groups = N / 128, kb = K / 128;
   int       s      = (240 + groups / 2) / groups;
   if (s > kb / 2) s = kb / 2;
-  const int mblk = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+  const int mblk = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
   const int cap  = 32 / mblk;  // slices whose rows fit the staging area
   if (s < (kb + cap - 1) / cap) s = (kb + cap - 1) / cap;
   if (s > MAX_SPLIT_K) s = MAX_SPLIT_K;

@@ -84,8 +84,13 @@ __device__ __forceinline__ void skinny_wait(SkinnySlot<MBLK, APRE>& t)
       asm volatile("s_waitcnt vmcnt(%1)" : "+v"(t.sa[0]) : "n"(N) : "memory");
     else if constexpr (MBLK == 2)
       asm volatile("s_waitcnt vmcnt(%2)" : "+v"(t.sa[0]), "+v"(t.sa[1]) : "n"(N) : "memory");
-    else
+    else if constexpr (MBLK == 4)
       asm volatile("s_waitcnt vmcnt(%4)" : "+v"(t.sa[0]), "+v"(t.sa[1]), "+v"(t.sa[2]), "+v"(t.sa[3]) : "n"(N) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(%8)"
+                   : "+v"(t.sa[0]), "+v"(t.sa[1]), "+v"(t.sa[2]), "+v"(t.sa[3]), "+v"(t.sa[4]), "+v"(t.sa[5]), "+v"(t.sa[6]), "+v"(t.sa[7])
+                   : "n"(N)
+                   : "memory");
   }
   else if constexpr (MBLK == 1)
     asm volatile("s_waitcnt vmcnt(%3)" : "+v"(t.a[0][0]), "+v"(t.a[0][1]), "+v"(t.sa[0]) : "n"(N) : "memory");
@@ -94,7 +99,7 @@ __device__ __forceinline__ void skinny_wait(SkinnySlot<MBLK, APRE>& t)
                  : "+v"(t.a[0][0]), "+v"(t.a[0][1]), "+v"(t.sa[0]), "+v"(t.a[1][0]), "+v"(t.a[1][1]), "+v"(t.sa[1])
                  : "n"(N)
                  : "memory");
-  else
+  else if constexpr (MBLK == 4)
     asm volatile("s_waitcnt vmcnt(%12)"
                  : "+v"(t.a[0][0]), "+v"(t.a[0][1]), "+v"(t.sa[0]), "+v"(t.a[1][0]), "+v"(t.a[1][1]), "+v"(t.sa[1]), "+v"(t.a[2][0]),
                    "+v"(t.a[2][1]), "+v"(t.sa[2]), "+v"(t.a[3][0]), "+v"(t.a[3][1]), "+v"(t.sa[3])
@@ -145,6 +150,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   constexpr bool APRE  = ASTG > 0;
   constexpr int  LOADS = SKINNY_LOADS_PER_SLOT_BASE + (APRE ? 1 : 3) * MBLK;  // vector-memory loads per slot, issued in slot order
   static_assert(D * LOADS < 64, "vmcnt is a 6-bit counter");
+  static_assert(MBLK <= 4 || APRE, "128-row groups only with staged activations");
   __shared__ __attribute__((aligned(1024))) char a_stage[APRE ? ASTG : 16];
   // one array per ring slot, so that the compiler can tell the slots apart
   __shared__ __attribute__((aligned(1024))) char ring0[8 * 2048];
@@ -164,7 +170,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   const int i    = lane & 15;
   const int ng   = blockIdx.x;
   const int sp   = blockIdx.y;
-  const int m0   = blockIdx.z * 64;                  // rows are handled in groups of 64: gridDim.z = ceil(M / 64)
+  const int m0   = blockIdx.z * (MBLK == 8 ? 128 : 64);  // row groups of 64 (of 128 with MBLK = 8): gridDim.z = number of groups
   const int KB   = K >> 7;
   const int kb0  = sp * KB / S;  // KB * S is small: 32-bit arithmetic (a 64-bit divide costs hundreds of scalar ops)
   const int kb1  = (sp + 1) * KB / S;
@@ -317,7 +323,7 @@ template <int MBLK, int OUT, int D, int ASTG>
 static hipError_t launch_skinny(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
                                 int N, int K, int S, float* partial, hipStream_t stream)
 {
-  hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D, ASTG>), dim3(N / 128, S, (M + 63) / 64), dim3(512), 0, stream,
+  hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D, ASTG>), dim3(N / 128, S, MBLK == 8 ? (M + 127) / 128 : (M + 63) / 64), dim3(512), 0, stream,
                      (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial);
   return hipGetLastError();
 }
@@ -348,6 +354,10 @@ static hipError_t dispatch_skinny(const void* A, const float* As, const void* Bt
     if (need <= 65536) LLMMM_GO(2, 2, 65536);
     if (slices >= 4) LLMMM_GO(2, 4, 0);
     LLMMM_GO(2, 2, 0);
+  }
+  if (M > 64 && M <= 128 && 8 * 2048 * longest <= 65536) {  // one pass over the weights for all rows
+    if (slices >= 4) LLMMM_GO(8, 4, 65536);
+    LLMMM_GO(8, 2, 65536);
   }
   if (M <= 128) {  // two row groups of (up to) 64 when M > 64
     const int need = 4 * 2048 * longest;

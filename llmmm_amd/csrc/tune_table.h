@@ -26,10 +26,11 @@ static const SkinnyTune kSkinnyTune[] = {
   {1, 2560, 9728, 10},
   {16, 2560, 9728, 10},
   {64, 2560, 9728, 10},
+  {128, 2560, 9728, 10},
   {1, 6144, 2560, 5},
   {16, 6144, 2560, 5},
   {64, 6144, 2560, 5},
-  {128, 6144, 2560, 3},
+  {128, 6144, 2560, 5},
   {1, 19456, 2560, 1},
   {16, 19456, 2560, 1},
   {64, 19456, 2560, 3},
@@ -42,7 +43,6 @@ static const TileTune kTileTune[] = {
   {2048, 2560, 4096, 3, 1},
   {128, 19456, 2560, 1, 3},
   {2048, 19456, 2560, 0, 1},
-  {128, 2560, 9728, 3, 8},
   {2048, 2560, 9728, 0, 3},
 };
 
