@@ -17,7 +17,7 @@ struct TileTune {
   int split_k;  // 0 = heuristic
 };
 
-// FP8 weight-streaming kernel (M <= 128, M != 128).
+// FP8 weight-streaming kernel (M <= 128).
 static const SkinnyTune kSkinnyTune[] = {
   {1, 2560, 4096, 8},
   {16, 2560, 4096, 8},

@@ -100,7 +100,7 @@ def render_table(skinny_rows, tile_rows, fp16_rows):
            "#pragma once", '#include "kernels.h"', "", "namespace llmmm {", "",
            "struct SkinnyTune {", "  int m_max;  // entry applies to M <= m_max (entries are ordered by m_max per shape)", "  int N, K;", "  int split_k;", "};",
            "struct TileTune {", "  int M, N, K;", "  int tile;", "  int split_k;  // 0 = heuristic", "};", "",
-           "// FP8 weight-streaming kernel (M <= 128, M != 128).", "static const SkinnyTune kSkinnyTune[] = {"]
+           "// FP8 weight-streaming kernel (M <= 128).", "static const SkinnyTune kSkinnyTune[] = {"]
     out += ["  {%d, %d, %d, %d}," % r for r in skinny_rows]
     out += ["};", "", "// FP8 MFMA tile kernels (M % 128 == 0).", "static const TileTune kTileTune[] = {"]
     out += ["  {%d, %d, %d, %d, %d}," % r for r in tile_rows]
