@@ -37,9 +37,11 @@ __device__ __forceinline__ f32x4 mfma_fp8_k128(i32x8 x, i32x8 y)
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, z, 0, 0, 0, 0, 0, 0);
 }
 
-template <int BM, int BN>
+// WM = rows of a wave's sub-tile (64 or 32); its columns are always 128, one quantisation group.
+template <int BM, int BN, int WM>
 struct Fp8Tile {
-  static constexpr int WAVES_M = BM / 64;
+  static constexpr int MF      = WM / 16;  // 16-row fragments per wave
+  static constexpr int WAVES_M = BM / WM;
   static constexpr int WAVES_N = BN / 128;
   static constexpr int NW      = WAVES_M * WAVES_N;
   static constexpr int NT      = NW * 64;
@@ -68,30 +70,33 @@ __device__ __forceinline__ void fp8_load_f32(float& dst, const void* sbase, unsi
 // per-lane offset: load i covers tile rows 8*(wave + i*NW) .. +7, and the SWZ_ROWS16 placement
 // only looks at row bits 0..3, so moving by 8*NW (>= 16) rows changes nothing but the
 // wave-uniform row base.
-template <int BM, int BN, int I>
+template <int BM, int BN, int WM, int I>
 __device__ __forceinline__ void fp8_issue_load(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned lane_off, int K, int wave)
 {
-  typedef Fp8Tile<BM, BN> TC;
+  typedef Fp8Tile<BM, BN, WM> TC;
   if constexpr (I < TC::A_LOADS)
     fp8_load_lds_16B(Ag + (size_t)(8 * TC::NW * I) * K, lane_off, lds_stage + (wave + I * TC::NW) * 1024);
   else if constexpr (I < TC::A_LOADS + TC::B_LOADS)
     fp8_load_lds_16B(Bg + (size_t)(8 * TC::NW * (I - TC::A_LOADS)) * K, lane_off, lds_stage + TC::A_BYTES + (wave + (I - TC::A_LOADS) * TC::NW) * 1024);
 }
-template <int BM, int BN, int FIRST, int COUNT>
+template <int BM, int BN, int WM, int FIRST, int COUNT>
 __device__ __forceinline__ void fp8_issue_loads(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned lane_off, int K, int wave)
 {
   if constexpr (COUNT > 0) {
-    fp8_issue_load<BM, BN, FIRST>(lds_stage, Ag, Bg, lane_off, K, wave);
-    fp8_issue_loads<BM, BN, FIRST + 1, COUNT - 1>(lds_stage, Ag, Bg, lane_off, K, wave);
+    fp8_issue_load<BM, BN, WM, FIRST>(lds_stage, Ag, Bg, lane_off, K, wave);
+    fp8_issue_loads<BM, BN, WM, FIRST + 1, COUNT - 1>(lds_stage, Ag, Bg, lane_off, K, wave);
   }
 }
 // The slice scales of the lane's four 16-row fragments and of the wave's column group.
-__device__ __forceinline__ void fp8_issue_scales(float (&sa)[4], float& sb, const float* As_slice, unsigned row_off, const float* Bs_elem, unsigned zero)
+template <int MF>
+__device__ __forceinline__ void fp8_issue_scales(float (&sa)[MF], float& sb, const float* As_slice, unsigned row_off, const float* Bs_elem, unsigned zero)
 {
   fp8_load_f32<0>(sa[0], As_slice, row_off);
   fp8_load_f32<64>(sa[1], As_slice, row_off);
-  fp8_load_f32<128>(sa[2], As_slice, row_off);
-  fp8_load_f32<192>(sa[3], As_slice, row_off);
+  if constexpr (MF == 4) {
+    fp8_load_f32<128>(sa[2], As_slice, row_off);
+    fp8_load_f32<192>(sa[3], As_slice, row_off);
+  }
   fp8_load_f32<0>(sb, Bs_elem, zero);
 }
 
@@ -117,50 +122,52 @@ struct Fp8Next {
   const float*   Bs_elem;    // &Bs[nb, kb_next]
 };
 
-// One 128-K slice of the wave's 64 x 128 sub-tile.  s[mf] = As[kb, row] * Bs[nb, kb].
+// One 128-K slice of the wave's WM x 128 sub-tile.  s[mf] = As[kb, row] * Bs[nb, kb].
 // With LOAD, the next stage's loads go out two or more per fragment step during the first four
 // steps (spread, so that no wave sits in the memory pipeline's issue queue while its matrix
 // work waits, and early enough to land within the slice), its scales during the fifth.
-template <int BM, int BN, bool LOAD>
+template <int BM, int BN, int WM, bool LOAD>
 __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int a_rd0, int a_rd1, int b_rd0, int b_rd1,
-                                                  const float (&s)[4], f32x4 (&acc)[8][4], const Fp8Next& nx, unsigned lane_off,
-                                                  unsigned row_off, unsigned zero, int K, int wave, float (&sa_next)[4], float& sb_next)
+                                                  const float (&s)[WM / 16], f32x4 (&acc)[8][WM / 16], const Fp8Next& nx, unsigned lane_off,
+                                                  unsigned row_off, unsigned zero, int K, int wave, float (&sa_next)[WM / 16],
+                                                  float& sb_next)
 {
-  typedef Fp8Tile<BM, BN> TC;
+  constexpr int MF = WM / 16;
+  typedef Fp8Tile<BM, BN, WM> TC;
   constexpr int           NL   = TC::A_LOADS + TC::B_LOADS;
   constexpr int           LPG  = (NL + 3) / 4;
   const char LLMMM_LDS*   ldsA = lds;
   const char LLMMM_LDS*   ldsB = lds + TC::A_BYTES;
-  i32x8                   a[4], b[2];
-  f32x4                   p[2][4];
+  i32x8                   a[MF], b[2];
+  f32x4                   p[2][MF];
   b[0] = fp8_read_frag(ldsB, b_rd0, b_rd1, 0);
 #pragma unroll
-  for (int mf = 0; mf < 4; ++mf) a[mf] = fp8_read_frag(ldsA, a_rd0, a_rd1, mf * 2048);
+  for (int mf = 0; mf < MF; ++mf) a[mf] = fp8_read_frag(ldsA, a_rd0, a_rd1, mf * 2048);
 #pragma unroll
   for (int nf = 0; nf < 8; ++nf) {
     const int cur = nf & 1;
     if (nf + 1 < 8) b[cur ^ 1] = fp8_read_frag(ldsB, b_rd0, b_rd1, (nf + 1) * 2048);
     if constexpr (LOAD) {
-      if (nf == 0) fp8_issue_loads<BM, BN, 0, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
-      if (nf == 1) fp8_issue_loads<BM, BN, LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
-      if (nf == 2) fp8_issue_loads<BM, BN, 2 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
-      if (nf == 3) fp8_issue_loads<BM, BN, 3 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
-      if (nf == 4) fp8_issue_scales(sa_next, sb_next, nx.As_slice, row_off, nx.Bs_elem, zero);
+      if (nf == 0) fp8_issue_loads<BM, BN, WM, 0, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
+      if (nf == 1) fp8_issue_loads<BM, BN, WM, LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
+      if (nf == 2) fp8_issue_loads<BM, BN, WM, 2 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
+      if (nf == 3) fp8_issue_loads<BM, BN, WM, 3 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
+      if (nf == 4) fp8_issue_scales<MF>(sa_next, sb_next, nx.As_slice, row_off, nx.Bs_elem, zero);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int mf = 0; mf < 4; ++mf) p[cur][mf] = mfma_fp8_k128(b[cur], a[mf]);
+    for (int mf = 0; mf < MF; ++mf) p[cur][mf] = mfma_fp8_k128(b[cur], a[mf]);
     if (nf > 0) {
 #pragma unroll
-      for (int mf = 0; mf < 4; ++mf)
+      for (int mf = 0; mf < MF; ++mf)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[nf - 1][mf][r] = __builtin_fmaf(p[cur ^ 1][mf][r], s[mf], acc[nf - 1][mf][r]);
       // Pin the promotion here (an empty asm the optimiser cannot move or sink), then ask for
       // MFMA, 4 FMA, MFMA, 4 FMA ...: the FMAs of fragment nf-1 run under the MFMAs of fragment nf.
 #pragma unroll
-      for (int mf = 0; mf < 4; ++mf) asm volatile("" : "+v"(acc[nf - 1][mf]));
+      for (int mf = 0; mf < MF; ++mf) asm volatile("" : "+v"(acc[nf - 1][mf]));
 #pragma unroll
-      for (int mf = 0; mf < 4; ++mf) {
+      for (int mf = 0; mf < MF; ++mf) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
       }
@@ -168,11 +175,11 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int
     __builtin_amdgcn_sched_barrier(0);
   }
 #pragma unroll
-  for (int mf = 0; mf < 4; ++mf)
+  for (int mf = 0; mf < MF; ++mf)
 #pragma unroll
     for (int r = 0; r < 4; ++r) acc[7][mf][r] = __builtin_fmaf(p[1][mf][r], s[mf], acc[7][mf][r]);
 #pragma unroll
-  for (int mf = 0; mf < 4; ++mf) asm volatile("" : "+v"(acc[7][mf]));
+  for (int mf = 0; mf < MF; ++mf) asm volatile("" : "+v"(acc[7][mf]));
 }
 
 __device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float d)
@@ -188,13 +195,14 @@ __device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float
   return (uint32_t)v;
 }
 
-template <int BM, int BN, int OUT>
-__global__ void __launch_bounds__((BM / 64) * (BN / 128) * 64)
+template <int BM, int BN, int WM, int OUT>
+__global__ void __launch_bounds__((BM / WM) * (BN / 128) * 64)
 fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
                 const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int tiles_m,
                 int tiles_n)
 {
-  typedef Fp8Tile<BM, BN> TC;
+  typedef Fp8Tile<BM, BN, WM> TC;
+  constexpr int MF = TC::MF;
   __shared__ __attribute__((aligned(1024))) char lds[2 * TC::STAGE];
 
   const int tid  = threadIdx.x;
@@ -222,46 +230,49 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   // operand reads: lane = (g = lane/16, i = lane%16) takes row i of a 16-row fragment and the
   // 32 bytes k = 32g .. 32g+31 (chunks 2g and 2g+1)
   const int g     = lane >> 4;
-  const int a_rd0 = kmajor_offset<SWZ_ROWS16>(wm * 64 + (lane & 15), 2 * g), a_rd1 = a_rd0 ^ 16;
+  const int a_rd0 = kmajor_offset<SWZ_ROWS16>(wm * WM + (lane & 15), 2 * g), a_rd1 = a_rd0 ^ 16;
   const int b_rd0 = kmajor_offset<SWZ_ROWS16>(wn * 128 + (lane & 15), 2 * g), b_rd1 = b_rd0 ^ 16;
 
-  f32x4 acc[8][4];
+  f32x4 acc[8][MF];
 #pragma unroll
   for (int nf = 0; nf < 8; ++nf)
 #pragma unroll
-    for (int mf = 0; mf < 4; ++mf) acc[nf][mf] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int mf = 0; mf < MF; ++mf) acc[nf][mf] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // scales: As[kb*M + m] for the lane's 4 rows, Bs[(n/128)*KB + kb] for the wave's column group
-  const int      mrow    = m0 + wm * 64 + (lane & 15);
+  const int      mrow    = m0 + wm * WM + (lane & 15);
   const unsigned row_off = (unsigned)mrow * 4u;
   const float*   Bsp     = Bs + (size_t)((n0 >> 7) + wn) * KB + kb0;
   const float*   Asl     = As + (size_t)kb0 * M;
   unsigned       zero    = 0;
   asm volatile("" : "+v"(zero));  // a VGPR holding 0: the per-lane offset of the wave-uniform Bs load
-  float sa_next[4], sb_next;
+  float sa_next[MF], sb_next;
 
   const unsigned lds0 = (unsigned)(size_t)(char LLMMM_LDS*)lds;
   char LLMMM_LDS* const s0 = (char LLMMM_LDS*)lds;
 
-  fp8_issue_loads<BM, BN, 0, TC::A_LOADS + TC::B_LOADS>(lds0, Ag, Bg, lane_off, K, wave);
-  fp8_issue_scales(sa_next, sb_next, Asl, row_off, Bsp, zero);
+  fp8_issue_loads<BM, BN, WM, 0, TC::A_LOADS + TC::B_LOADS>(lds0, Ag, Bg, lane_off, K, wave);
+  fp8_issue_scales<MF>(sa_next, sb_next, Asl, row_off, Bsp, zero);
 
   // One slice: wait for this wave's loads of the slice (all of them were issued at least half a
   // slice ago), meet the other waves, then compute it while the loads of the next one go out.
 #define LLMMM_FP8_SLICE(LOAD, CUR, NXT_LDS, KC)                                                                                   \
   {                                                                                                                               \
     wait_vmcnt<0>();                                                                                                              \
-    asm volatile("" : "+v"(sa_next[0]), "+v"(sa_next[1]), "+v"(sa_next[2]), "+v"(sa_next[3]), "+v"(sb_next));                     \
+    if constexpr (MF == 4)                                                                                                        \
+      asm volatile("" : "+v"(sa_next[0]), "+v"(sa_next[1]), "+v"(sa_next[2]), "+v"(sa_next[MF - 1]), "+v"(sb_next));              \
+    else                                                                                                                          \
+      asm volatile("" : "+v"(sa_next[0]), "+v"(sa_next[1]), "+v"(sb_next));                                                       \
     __syncthreads();                                                                                                              \
-    float s[4];                                                                                                                   \
-    _Pragma("unroll") for (int mf = 0; mf < 4; ++mf) s[mf] = sa_next[mf] * sb_next;                                               \
+    float s[MF];                                                                                                                  \
+    _Pragma("unroll") for (int mf = 0; mf < MF; ++mf) s[mf] = sa_next[mf] * sb_next;                                               \
     Fp8Next nx;                                                                                                                   \
     nx.lds_stage = NXT_LDS;                                                                                                       \
     nx.Ag        = Ag + (size_t)((KC) + 1) * 128;                                                                                 \
     nx.Bg        = Bg + (size_t)((KC) + 1) * 128;                                                                                 \
     nx.As_slice  = Asl + (size_t)((KC) + 1) * M;                                                                                  \
     nx.Bs_elem   = Bsp + (KC) + 1;                                                                                                \
-    fp8_compute_stage<BM, BN, LOAD>(CUR, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, row_off, zero, K, wave, sa_next,       \
+    fp8_compute_stage<BM, BN, WM, LOAD>(CUR, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, row_off, zero, K, wave, sa_next,       \
                                     sb_next);                                                                                     \
   }
 
@@ -276,18 +287,18 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   // ---- epilogue.  lane (g, i): row m = .. + mf*16 + i, columns n = nf*16 + 4g + r.
   // Written straight from this layout, one store instruction would touch 16 rows with 16..64
   // bytes each; the memory pipeline pays per row segment, not per byte.  So every wave first
-  // lays its 64 x 128 result out row-major in a private 16 KB piece of the (now idle) operand
+  // lays its WM x 128 result out row-major in a private 16 KB piece of the (now idle) operand
   // buffers -- 16-byte chunks XOR-ed with row bits so that neither the writes nor the
   // ds_read_b128 reads conflict -- and stores it back out 16 bytes per lane, whole rows at a time.
   __syncthreads();  // every wave is done reading the last operand stage
   char LLMMM_LDS* const stg  = s0 + wave * 16384;
-  const int             row0 = m0 + wm * 64;
+  const int             row0 = m0 + wm * WM;
   const int             col0 = n0 + wn * 128;
   const int             li   = lane & 15;
   if constexpr (OUT == OUT_F32) {
     float* C = (float*)Cv + (size_t)sp * M * N;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {  // 32 rows x 512 B per round
+    for (int h = 0; h < MF / 2; ++h) {  // 32 rows x 512 B per round
 #pragma unroll
       for (int mfl = 0; mfl < 2; ++mfl) {
         const int r = mfl * 16 + li;
@@ -306,7 +317,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
     __bf16* C = (__bf16*)Cv;
     typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int mf = 0; mf < 4; ++mf) {
+    for (int mf = 0; mf < MF; ++mf) {
       const int r = mf * 16 + li;
 #pragma unroll
       for (int nf = 0; nf < 8; ++nf) {
@@ -317,7 +328,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
       }
     }
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
+    for (int j = 0; j < WM / 4; ++j) {
       const int   r = 4 * j + (lane >> 4), c = lane & 15;
       const i32x4 v = *(const i32x4 LLMMM_LDS*)(stg + r * 256 + ((c ^ (r & 15)) << 4));
       *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 8) = v;
@@ -326,7 +337,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   else {
     uint8_t* C = (uint8_t*)Cv;
 #pragma unroll
-    for (int mf = 0; mf < 4; ++mf) {
+    for (int mf = 0; mf < MF; ++mf) {
       float amax = 0.f;
 #pragma unroll
       for (int nf = 0; nf < 8; ++nf)
@@ -345,7 +356,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
       if (g == 0) Cs[(size_t)((n0 >> 7) + wn) * M + row0 + r] = scale;
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < WM / 8; ++j) {
       const int   r = 8 * j + (lane >> 3), c = lane & 7;
       const i32x4 v = *(const i32x4 LLMMM_LDS*)(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
       *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 16) = v;
@@ -418,19 +429,19 @@ static hipError_t launch_reduce(const float* planes, int S, void* C, float* Cs, 
   return hipGetLastError();
 }
 
-template <int BM, int BN, int OUT>
+template <int BM, int BN, int WM, int OUT>
 static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N,
                              int K, int S, float* planes, hipStream_t stream)
 {
-  typedef Fp8Tile<BM, BN> TC;
+  typedef Fp8Tile<BM, BN, WM> TC;
   const int tiles_m = M / BM, tiles_n = N / BN;
   if (S <= 1) {
-    hipLaunchKernelGGL((fp8_gemm_kernel<BM, BN, OUT>), dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As,
+    hipLaunchKernelGGL((fp8_gemm_kernel<BM, BN, WM, OUT>), dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As,
                        (const uint8_t*)Bt, Bs, C, Cs, M, N, K, tiles_m, tiles_n);
     return hipGetLastError();
   }
   // split-K: S partial planes from the fp32 instantiation, then the ordered sum + epilogue
-  hipLaunchKernelGGL((fp8_gemm_kernel<BM, BN, OUT_F32>), dim3(tiles_m * tiles_n, S), dim3(TC::NT), 0, stream, (const uint8_t*)A, As,
+  hipLaunchKernelGGL((fp8_gemm_kernel<BM, BN, WM, OUT_F32>), dim3(tiles_m * tiles_n, S), dim3(TC::NT), 0, stream, (const uint8_t*)A, As,
                      (const uint8_t*)Bt, Bs, (void*)planes, (float*)nullptr, M, N, K, tiles_m, tiles_n);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
@@ -442,10 +453,10 @@ static hipError_t dispatch_fp8(int tile, const void* A, const float* As, const v
                                int M, int N, int K, int S, float* planes, hipStream_t stream)
 {
   switch (tile) {
-    case LLMMM_TILE_256x256: return launch_fp8<256, 256, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
-    case LLMMM_TILE_128x256: return launch_fp8<128, 256, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
-    case LLMMM_TILE_256x128: return launch_fp8<256, 128, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
-    case LLMMM_TILE_128x128: return launch_fp8<128, 128, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case LLMMM_TILE_256x256: return launch_fp8<256, 256, 64, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case LLMMM_TILE_128x256: return launch_fp8<128, 256, 64, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case LLMMM_TILE_256x128: return launch_fp8<256, 128, 64, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case LLMMM_TILE_128x128: return launch_fp8<128, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);  // four 32-row waves
     default: return hipErrorInvalidValue;
   }
 }

@@ -26,7 +26,6 @@ static const SkinnyTune kSkinnyTune[] = {
   {1, 2560, 9728, 10},
   {16, 2560, 9728, 10},
   {64, 2560, 9728, 10},
-  {128, 2560, 9728, 10},
   {1, 6144, 2560, 5},
   {16, 6144, 2560, 5},
   {64, 6144, 2560, 5},
@@ -41,9 +40,10 @@ static const TileTune kTileTune[] = {
   {4096, 4096, 4096, 0, 1},
   {2048, 6144, 2560, 0, 1},
   {2048, 2560, 4096, 3, 1},
-  {128, 19456, 2560, 1, 3},
+  {128, 19456, 2560, 3, 1},
   {2048, 19456, 2560, 0, 1},
-  {2048, 2560, 9728, 0, 3},
+  {128, 2560, 9728, 3, 8},
+  {2048, 2560, 9728, 3, 1},
 };
 
 // FP16/BF16 MFMA tile kernels.
