@@ -250,7 +250,10 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
   LLMMM_ISSUE(0, 0);
   if (1 < KT) LLMMM_ISSUE(1, 1);
   if (2 < KT) LLMMM_ISSUE(2, 2);
-  wait_vmcnt<0>();
+  if (!KTAIL && 2 < KT)
+    wait_vmcnt<2 * TC::LOADS>();  // only stage 0 has to be here; stages 1 and 2 stay in flight
+  else
+    wait_vmcnt<0>();
   __builtin_amdgcn_s_barrier();
   if (3 < KT) LLMMM_ISSUE(3, 3);
 

@@ -195,6 +195,16 @@ __device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float
   return (uint32_t)v;
 }
 
+// The same conversion without the clamp, for values that are known to lie within +-448 * (1 + 2^-22):
+// the fused epilogue's C * (448 / amax), whose magnitude cannot exceed the row's own amax * (448 / amax).
+// Anything below 464 rounds to 448, so the codes are those of pack_e4m3x4; 128 v_med3 per lane are saved.
+__device__ __forceinline__ uint32_t pack_e4m3x4_in_range(float a, float b, float c, float d)
+{
+  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  v     = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+  return (uint32_t)v;
+}
+
 template <int BM, int BN, int WM, int OUT>
 __global__ void __launch_bounds__((BM / WM) * (BN / 128) * 64)
 fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
@@ -351,7 +361,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
 #pragma unroll
       for (int nf = 0; nf < 8; ++nf) {
         const f32x4 v = acc[nf][mf];
-        *(uint32_t LLMMM_LDS*)(stg + r * 128 + ((nf ^ ((r >> 1) & 7)) << 4) + 4 * g) = pack_e4m3x4(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+        *(uint32_t LLMMM_LDS*)(stg + r * 128 + ((nf ^ ((r >> 1) & 7)) << 4) + 4 * g) = pack_e4m3x4_in_range(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
       }
       if (g == 0) Cs[(size_t)((n0 >> 7) + wn) * M + row0 + r] = scale;
     }
