@@ -7,7 +7,6 @@
 
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
-#include <stdlib.h>
 #include <stdio.h>
 #include <string.h>
 
@@ -30,12 +29,12 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 constexpr int    MAX_SPLIT_K     = 32;
 constexpr int    NUM_CUS         = 256;   // MI355X
 
-constexpr int SKINNY_MAX_M = 128;  // rows the weight-streaming kernel takes (two groups of 64)
+constexpr int SKINNY_MAX_M = 128;  // rows the weight-streaming kernel takes
 
 int max_split_for(int K) { return (K / 128) < MAX_SPLIT_K ? (K / 128) : MAX_SPLIT_K; }
 
 // Split count for the weight-streaming kernel when the tune table has no entry: about one
-// workgroup (one 128-column group x one 64-row group x one split) per CU -- what the measured
+// workgroup (one 128-column group x one split) per CU -- what the measured
 // Qwen3-4B shapes settle on -- every split at least two 128-K slices long, but short enough
 // that the activation rows of a split can be staged in LDS (64 KB: 32 slices of 16 rows).
 int heuristic_split(int M, int N, int K)

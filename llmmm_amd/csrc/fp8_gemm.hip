@@ -301,25 +301,21 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   // buffers -- 16-byte chunks XOR-ed with row bits so that neither the writes nor the
   // ds_read_b128 reads conflict -- and stores it back out 16 bytes per lane, whole rows at a time.
   __syncthreads();  // every wave is done reading the last operand stage
-  char LLMMM_LDS* const stg  = s0 + wave * 16384;
+  char LLMMM_LDS* const stg  = s0 + wave * (WM * 256);  // WM rows of up to 256 bytes; fp32 goes 16 rows at a time
   const int             row0 = m0 + wm * WM;
   const int             col0 = n0 + wn * 128;
   const int             li   = lane & 15;
   if constexpr (OUT == OUT_F32) {
     float* C = (float*)Cv + (size_t)sp * M * N;
 #pragma unroll
-    for (int h = 0; h < MF / 2; ++h) {  // 32 rows x 512 B per round
+    for (int mf = 0; mf < MF; ++mf) {  // 16 rows x 512 B per round
 #pragma unroll
-      for (int mfl = 0; mfl < 2; ++mfl) {
-        const int r = mfl * 16 + li;
+      for (int nf = 0; nf < 8; ++nf) *(f32x4 LLMMM_LDS*)(stg + li * 512 + (((nf * 4 + g) ^ ((li & 7) << 1)) << 4)) = acc[nf][mf];
 #pragma unroll
-        for (int nf = 0; nf < 8; ++nf) *(f32x4 LLMMM_LDS*)(stg + r * 512 + (((nf * 4 + g) ^ ((r & 7) << 1)) << 4)) = acc[nf][2 * h + mfl];
-      }
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
+      for (int j = 0; j < 8; ++j) {
         const int   r = 2 * j + (lane >> 5), c = lane & 31;
         const f32x4 v = *(const f32x4 LLMMM_LDS*)(stg + r * 512 + ((c ^ ((r & 7) << 1)) << 4));
-        *(f32x4*)(C + (size_t)(row0 + 32 * h + r) * N + col0 + c * 4) = v;
+        *(f32x4*)(C + (size_t)(row0 + 16 * mf + r) * N + col0 + c * 4) = v;
       }
     }
   }
