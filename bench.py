@@ -183,7 +183,7 @@ def main():
                          "decode_<qkv|o|gate_up|down>_m<M> | copy_1g (counter calibration only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table")
-    ap.add_argument("--cpu-rows", type=int, default=2048)
+    ap.add_argument("--cpu-rows", type=int, default=4096)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (every box has one GPU); run with --gpus 1",
