@@ -458,11 +458,12 @@ template <int OUT>
 static hipError_t dispatch_fp8(int tile, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
                                int M, int N, int K, int S, float* planes, hipStream_t stream)
 {
+  // the 256 x 256 tile uses eight 64-row waves; the smaller tiles 32-row waves (twice the waves per SIMD)
   switch (tile) {
     case LLMMM_TILE_256x256: return launch_fp8<256, 256, 64, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
-    case LLMMM_TILE_128x256: return launch_fp8<128, 256, 64, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
-    case LLMMM_TILE_256x128: return launch_fp8<256, 128, 64, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
-    case LLMMM_TILE_128x128: return launch_fp8<128, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);  // four 32-row waves
+    case LLMMM_TILE_128x256: return launch_fp8<128, 256, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case LLMMM_TILE_256x128: return launch_fp8<256, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case LLMMM_TILE_128x128: return launch_fp8<128, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
     default: return hipErrorInvalidValue;
   }
 }
