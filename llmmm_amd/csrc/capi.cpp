@@ -59,9 +59,9 @@ int heuristic_tile(int M, int N)
     int   id, bm, bn, per_cu;
     float eff;
   } cand[] = {{LLMMM_TILE_256x256, 256, 256, 1, 1.00f},
-              {LLMMM_TILE_128x256, 128, 256, 1, 0.88f},
-              {LLMMM_TILE_256x128, 256, 128, 1, 0.88f},
-              {LLMMM_TILE_128x128, 128, 128, 2, 0.75f}};
+              {LLMMM_TILE_128x256, 128, 256, 1, 0.85f},
+              {LLMMM_TILE_256x128, 256, 128, 1, 0.85f},
+              {LLMMM_TILE_128x128, 128, 128, 2, 0.90f}};
   int   best      = -1;
   float best_cost = 0.f;
   for (const auto& c : cand) {
