@@ -124,15 +124,18 @@ def fp8_bytes(M, N, K, out):
     return b
 
 
-def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0):
+def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0, preshuffled=False):
     """out in {"f32","bf16","fp8q"}.  With rotate_bytes > 0 the launches cycle through enough
-    distinct weight copies to exceed that many bytes, so weights stream from HBM, not from cache."""
+    distinct weight copies to exceed that many bytes, so weights stream from HBM, not from cache.
+    preshuffled: the weights are permuted once, outside the timed region, into MFMA operand order."""
     import llmmm_amd
     from llmmm_amd import _lib
     copies = 1
     if rotate_bytes:
         copies = max(2, int(np.ceil(rotate_bytes / float(N * K))))
     Aq, As, weights = fp8_inputs(M, N, K, copies=copies)
+    if preshuffled:
+        weights = [(llmmm_amd.preshuffle_weight(bq), bs) for bq, bs in weights]
     kind = {"f32": _lib.OUT_F32, "bf16": _lib.OUT_BF16, "fp8q": _lib.OUT_FP8Q}[out]
     cdt = {"f32": torch.float32, "bf16": torch.bfloat16, "fp8q": torch.uint8}[out]
     C = torch.empty((M, N), dtype=cdt, device="cuda")
@@ -146,9 +149,10 @@ def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0):
         Bq, Bs = weights[state["i"] % copies]
         state["i"] += 1
         if out == "fp8q":
-            llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(Aq, As, Bq, Bs, C, Cs, M, N, K, workspace=ws)
+            llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(Aq, As, Bq, Bs, C, Cs, M, N, K, workspace=ws,
+                                                                                       b_preshuffled=preshuffled)
         else:
-            fns[out](Aq, As, Bq, Bs, C, M, N, K, workspace=ws)
+            fns[out](Aq, As, Bq, Bs, C, M, N, K, workspace=ws, b_preshuffled=preshuffled)
 
     ms, wall = _events_ms(step, steps, warmup, graph=True)
     flops = 2.0 * M * N * K
@@ -180,7 +184,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="fp16_gemm_4096",
                     help="fp16_gemm_4096 (headline) | fp8_gemm_fused_4096 | fp8_gemm_bf16_4096 | bf16_gemm_4096 | "
-                         "decode_<qkv|o|gate_up|down>_m<M> | copy_1g (counter calibration only)")
+                         "decode_<qkv|o|gate_up|down>_m<M>[_pre] (_pre: weights pre-shuffled offline) | copy_1g (counter calibration only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table")
     ap.add_argument("--cpu-rows", type=int, default=4096)
@@ -225,19 +229,20 @@ def main():
         cfg = {"workload": "FP8 e4m3 blockwise GEMM M=N=K=4096 (A 1x128, B 128x128 scales), output %s" % out, "M": M, "N": N, "K": K}
     elif w.startswith("decode_"):
         import re
-        mo = re.fullmatch(r"decode_(qkv|o|gate_up|down)_m(\d+)", w)
+        mo = re.fullmatch(r"decode_(qkv|o|gate_up|down)_m(\d+)(_pre)?", w)
         if not mo:
             print("unknown workload", w, file=sys.stderr)
             sys.exit(2)
         name, M = mo.group(1), int(mo.group(2))
         N, K = QWEN3_4B[name]
-        r = bench_fp8(M, N, K, "fp8q", args.steps, args.warmup, rotate_bytes=768 << 20)
+        pre = mo.group(3) is not None
+        r = bench_fp8(M, N, K, "fp8q", args.steps, args.warmup, rotate_bytes=768 << 20, preshuffled=pre)
         dtype = "fp8"
         roof = {"bound": "hbm", "achieved": r["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": r["gbs"] / PEAK_HBM_GBS, "traffic": None,
                 "kernel": "fp8_skinny_kernel split_k=%d" % r["split_k"]}
         value, unit = r["gbs"], "GB/s"
-        cfg = {"workload": "Qwen3-4B %s projection, FP8 blockwise GEMM + fused C quant, M=%d N=%d K=%d, weights rotated over %d "
-                           "copies" % (name, M, N, K, r["weight_copies"]), "M": M, "N": N, "K": K}
+        cfg = {"workload": "Qwen3-4B %s projection, FP8 blockwise GEMM + fused C quant, M=%d N=%d K=%d, %s weights rotated over %d "
+                           "copies" % (name, M, N, K, "pre-shuffled" if pre else "row-major", r["weight_copies"]), "M": M, "N": N, "K": K}
     else:
         print("unknown workload", w, file=sys.stderr)
         sys.exit(2)
@@ -267,9 +272,9 @@ def main():
             x = bench_fp8(4096, 4096, 4096, out, s2, w2)
             shapes.append({"name": "fp8_gemm_4096_" + out, "ms": x["ms"], "tflops": x["tflops"], "frac_of_fp8_peak": x["tflops"] / PEAK_TFLOPS["fp8"]})
         for name, (n, k) in QWEN3_4B.items():
-            for m in (1, 16, 128, 2048):
-                x = bench_fp8(m, n, k, "fp8q", s2 * 2 if m <= 16 else s2, w2, rotate_bytes=(768 << 20) if m <= 128 else 0)
-                e = {"name": "qwen3_4b_%s_m%d" % (name, m), "M": m, "N": n, "K": k, "us": x["ms"] * 1e3, "tflops": x["tflops"],
+            for m, pre in ((1, False), (1, True), (16, False), (16, True), (128, False), (128, True), (2048, False), (2048, True)):
+                x = bench_fp8(m, n, k, "fp8q", s2 * 2 if m <= 16 else s2, w2, rotate_bytes=(768 << 20) if m <= 128 else 0, preshuffled=pre)
+                e = {"name": "qwen3_4b_%s_m%d%s" % (name, m, "_preshuffled" if pre else ""), "M": m, "N": n, "K": k, "us": x["ms"] * 1e3, "tflops": x["tflops"],
                      "frac_of_fp8_peak": x["tflops"] / PEAK_TFLOPS["fp8"], "tile": x["tile"], "split_k": x["split_k"]}
                 if m <= 128:
                     e.update({"hbm_gbs": x["gbs"], "frac_of_hbm_peak": x["gbs"] / PEAK_HBM_GBS, "weight_copies": x["weight_copies"]})

@@ -53,8 +53,7 @@ extern "C" {
 #define LLMMM_QUANT_128x128_T 3 /* <128,128,true>               scale[(n/128)*M + m/128] */
 
 /* Kernel selection for llmmm_fp8_gemm_ex / llmmm_fp16_gemm_ex (the auto-tune driver's knobs).
- * tile: LLMMM_TILE_AUTO or one of the explicit ids; split_k: 0 = auto, >= 1 explicit
- * (only the skinny kernel splits K). */
+ * tile: LLMMM_TILE_AUTO or one of the explicit ids; split_k: 0 = auto, >= 1 explicit. */
 #define LLMMM_TILE_AUTO (-1)
 #define LLMMM_TILE_256x256 0
 #define LLMMM_TILE_128x256 1
@@ -62,9 +61,14 @@ extern "C" {
 #define LLMMM_TILE_128x128 3
 #define LLMMM_TILE_SKINNY 8 /* M <= 128 weight-streaming kernel */
 
+/* Weight layout of the FP8 GEMM's B operand (llmmm_gemm_cfg.b_layout). */
+#define LLMMM_FP8_B_ROWS 0        /* Bt[N,K] row-major, the reference layout (examples/005.fp8.mm.cu:157) */
+#define LLMMM_FP8_B_PRESHUFFLED 1 /* the image llmmm_fp8_preshuffle_b writes */
+
 typedef struct llmmm_gemm_cfg {
   int tile;
   int split_k;
+  int b_layout; /* FP8 only: LLMMM_FP8_B_ROWS (0, the default) or LLMMM_FP8_B_PRESHUFFLED; the FP16 GEMM ignores it */
 } llmmm_gemm_cfg;
 
 /* ---- FP16 / BF16 GEMM -------------------------------------------------------------------
@@ -114,6 +118,25 @@ LLMMM_API int llmmm_fp8_gemm_query(int out_kind, int M, int N, int K, llmmm_gemm
  *                float* scale, int M, int N, cudaStream_t)             examples/005.fp8.mm.cu:547-563.
  * x [M,N] fp32 -> q [M,N] e4m3 + scales (layout per `kind`).  Any M; N % 4 == 0. */
 LLMMM_API int llmmm_quant_fp8(int kind, const float* x, void* q, float* scale, int M, int N, void* stream);
+
+/* ---- offline layout helpers --------------------------------------------------------------
+ * llmmm_fp8_preshuffle_b takes the role of  construct_m16n8k32_B_layout(dst, src_transposed, N, K,
+ * stream)  (src/base/base.h:13, src/base/base.cu:222-271): a one-off permutation of the weights
+ * Bt[N,K] e4m3 into the order the matrix instructions consume them in.  The byte order is this
+ * library's (MFMA 16x16x128 on gfx950), not the reference's mma.m16n8k32 one: Bp consists of
+ * 2 KB blocks, block (n/16, k/128) at ((n/16) * (K/128) + k/128) * 2048, each the LDS image of
+ * its 16 rows x 128 bytes (16-byte chunk c of row r at r*128 + ((c ^ swz(r)) << 4), with
+ * swz(r) = ((r >> 1) & 7) ^ ((((r >> 2) ^ (r >> 3)) & 1) << 1)).  Every FP8 GEMM entry point
+ * accepts it through cfg->b_layout = LLMMM_FP8_B_PRESHUFFLED, with the scales Bs unchanged;
+ * results are bit-identical to the row-major layout's.  llmmm_fp8_unshuffle_b is the exact inverse.
+ * N % 16 == 0 and K % 128 == 0 (the reference's text "K must be greater than 0 and divisible by
+ * 128." is left in llmmm_last_error); src and dst must not overlap.
+ * llmmm_transpose replaces  transpose_matrix__aligned_128<T>(dst, src, M, N, stream)
+ * (src/base/base.h:9, src/base/base.cu:124-153) for sizeof(T) = 1 (e4m3) and 4 (float):
+ * dst[n*M+m] = src[m*N+n]; M % 128 == 0 and N % 128 == 0 ("M or N can't be divided 128."). */
+LLMMM_API int llmmm_fp8_preshuffle_b(const void* Bt, void* Bp, int N, int K, void* stream);
+LLMMM_API int llmmm_fp8_unshuffle_b(const void* Bp, void* Bt, int N, int K, void* stream);
+LLMMM_API int llmmm_transpose(int elem_size, const void* src, void* dst, int M, int N, void* stream);
 
 /* ---- misc ------------------------------------------------------------------------------- */
 LLMMM_API const char* llmmm_error_string(int code); /* the reference's exception texts for codes 1 and 2 */

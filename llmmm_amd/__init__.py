@@ -5,6 +5,7 @@
 """
 from . import _lib  # noqa: F401  (raises if libllmmm.so has not been built)
 from .mm import (  # noqa: F401
+    construct_mfma_B_layout,
     fp16_gemm,
     fp16_mm,
     fp8_blockwise_symmetric_quantization,
@@ -12,8 +13,11 @@ from .mm import (  # noqa: F401
     fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16,
     fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32,
     make_workspace,
+    preshuffle_weight,
     quantize_activation,
     quantize_weight,
     query_config,
+    restore_B_layout,
+    transpose_matrix__aligned_128,
     workspace_bytes,
 )

@@ -19,11 +19,12 @@ DTYPE_F16, DTYPE_BF16 = 0, 1
 B_ROW_MAJOR, B_TRANSPOSED = 0, 1
 OUT_F32, OUT_BF16, OUT_FP8Q = 0, 1, 2
 QUANT_1x128_T, QUANT_128x128, QUANT_1x128, QUANT_128x128_T = 0, 1, 2, 3
+FP8_B_ROWS, FP8_B_PRESHUFFLED = 0, 1
 TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_SKINNY = -1, 0, 1, 2, 3, 8
 
 
 class GemmCfg(ctypes.Structure):
-    _fields_ = [("tile", ctypes.c_int), ("split_k", ctypes.c_int)]
+    _fields_ = [("tile", ctypes.c_int), ("split_k", ctypes.c_int), ("b_layout", ctypes.c_int)]
 
 
 # name -> (restype, argtypes); must list every symbol include/llmmm.h declares
@@ -37,6 +38,9 @@ SIGNATURES = {
     "llmmm_fp8_gemm_workspace": (_sz, [_i, _i, _i, _i]),
     "llmmm_fp8_gemm_query": (_i, [_i, _i, _i, _i, _c.POINTER(GemmCfg)]),
     "llmmm_quant_fp8": (_i, [_i, _fp, _vp, _fp, _i, _i, _vp]),
+    "llmmm_fp8_preshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
+    "llmmm_fp8_unshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
+    "llmmm_transpose": (_i, [_i, _vp, _vp, _i, _i, _vp]),
     "llmmm_error_string": (_c.c_char_p, [_i]),
     "llmmm_last_error": (_c.c_char_p, []),
     "llmmm_version": (_i, []),
@@ -46,11 +50,15 @@ SIGNATURES = {
 def load():
     if not os.path.exists(LIB_PATH):
         raise ImportError(
-            "%s is missing: build it with `python -m llmmm_amd.build` (hipcc, gfx950). "
+            "%s is missing: build it with `python llmmm_amd/build.py` (hipcc, gfx950). "
             "There is no fallback path." % LIB_PATH)
     lib = ctypes.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
-        fn = getattr(lib, name)
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            raise ImportError("%s lacks %s: it is older than the sources, rebuild it with "
+                              "`python llmmm_amd/build.py`" % (LIB_PATH, name)) from None
         fn.restype, fn.argtypes = res, args
     return lib
 
@@ -61,11 +69,11 @@ lib = load()
 def check(code):
     """Turn a status code into the exception the reference's launchers throw.
 
-    Codes 1 and 2 carry the reference's own texts (src/mm/fp16/mm.cu:15-21)."""
+    Codes 1 and 2 carry the reference's own texts (src/mm/fp16/mm.cu:15-21, src/base/base.cu:127-129, :265-267)."""
     if code == OK:
         return
     text = lib.llmmm_error_string(code).decode()
     detail = lib.llmmm_last_error().decode()
     if code in (ERR_NOT_ALIGNED, ERR_UNSUPPORTED_TYPE):
-        raise RuntimeError(text)
+        raise RuntimeError(detail or text)  # the detail is the reference's text for the entry point that failed
     raise RuntimeError("%s: %s" % (text, detail) if detail else text)

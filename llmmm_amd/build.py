@@ -1,7 +1,8 @@
 """Builds ``libllmmm.so`` (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
 
-``python -m llmmm_amd.build`` or ``llmmm_amd.build.build()``.  hipcc cross-compiles without a
-GPU; the resulting library sits next to this file so that it travels with the source tree.
+``python llmmm_amd/build.py`` (run as a script: importing the package needs the library this
+builds).  hipcc cross-compiles without a GPU; the resulting library sits next to this file so
+that it travels with the source tree.
 """
 import os
 import subprocess
@@ -26,6 +27,7 @@ SOURCES = {
     "fp8_gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "fp8_skinny.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "quant_fp8.hip": [],
+    "layout.hip": [],
     "capi.cpp": ["-x", "hip"],
 }
 

@@ -110,8 +110,9 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
 {
   if (M <= 0 || N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "M, N and K must be positive (got %d, %d, %d)", M, N, K);
   if (N % 128 || K % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
-  cfg->tile    = -1;
-  cfg->split_k = 0;
+  cfg->tile     = -1;
+  cfg->split_k  = 0;
+  cfg->b_layout = LLMMM_FP8_B_ROWS;
   if (M % 128 == 0)
     for (const auto& e : llmmm::kTileTune)
       if (e.M == M && e.N == N && e.K == K) {
@@ -229,6 +230,9 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
   if (user) {
     if (user->tile != LLMMM_TILE_AUTO) cfg.tile = user->tile;
     if (user->split_k > 0) cfg.split_k = user->split_k;
+    if (user->b_layout != LLMMM_FP8_B_ROWS && user->b_layout != LLMMM_FP8_B_PRESHUFFLED)
+      return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown B layout %d", user->b_layout);
+    cfg.b_layout = user->b_layout;
   }
   hipError_t e;
   if (cfg.tile == LLMMM_TILE_SKINNY) {
@@ -244,7 +248,7 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
       if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
       partial = (float*)workspace;
     }
-    e = llmmm::fp8_skinny_launch(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, split, partial, (hipStream_t)stream);
+    e = llmmm::fp8_skinny_launch(out_kind, cfg.b_layout, A, As, Bt, Bs, C, Cs, M, N, K, split, partial, (hipStream_t)stream);
     if (e == hipSuccess && split > 1) e = llmmm::fp8_splitk_reduce_launch(out_kind, partial, split, C, Cs, M, N, (hipStream_t)stream);
   }
   else {
@@ -269,7 +273,7 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
       if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
       planes = (float*)workspace;
     }
-    e = llmmm::fp8_gemm_launch(out_kind, cfg.tile, A, As, Bt, Bs, C, Cs, M, N, K, split, planes, (hipStream_t)stream);
+    e = llmmm::fp8_gemm_launch(out_kind, cfg.tile, cfg.b_layout, A, As, Bt, Bs, C, Cs, M, N, K, split, planes, (hipStream_t)stream);
   }
   if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "fp8 gemm launch: %s", hipGetErrorString(e));
   return LLMMM_OK;
@@ -293,6 +297,40 @@ int llmmm_quant_fp8(int kind, const float* x, void* q, float* scale, int M, int 
   const int transpose = (kind == LLMMM_QUANT_1x128_T || kind == LLMMM_QUANT_128x128_T) ? 1 : 0;
   const hipError_t e  = llmmm::quant_fp8_launch(quant_m, transpose, x, q, scale, M, N, (hipStream_t)stream);
   if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "quantiser launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
+static int preshuffle(int inverse, const void* src, void* dst, int N, int K, void* stream)
+{
+  if (N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "N and K must be positive (got %d, %d)", N, K);
+  if (K % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "K must be greater than 0 and divisible by 128.");
+  if (N % 16) return fail(LLMMM_ERR_NOT_ALIGNED, "N must be divisible by 16.");
+  if (!src || !dst) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (!aligned16(src) || !aligned16(dst)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+  if ((long)N * K >= (1L << 31)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
+  const char *a = (const char*)src, *b = (const char*)dst;
+  if (a < b + (size_t)N * K && b < a + (size_t)N * K) return fail(LLMMM_ERR_INVALID_ARGUMENT, "source and destination overlap");
+  const hipError_t e = llmmm::fp8_preshuffle_launch(inverse, src, dst, N, K, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "pre-shuffle launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
+int llmmm_fp8_preshuffle_b(const void* Bt, void* Bp, int N, int K, void* stream) { return preshuffle(0, Bt, Bp, N, K, stream); }
+int llmmm_fp8_unshuffle_b(const void* Bp, void* Bt, int N, int K, void* stream) { return preshuffle(1, Bp, Bt, N, K, stream); }
+
+int llmmm_transpose(int elem_size, const void* src, void* dst, int M, int N, void* stream)
+{
+  if (elem_size != 1 && elem_size != 4) return fail(LLMMM_ERR_UNSUPPORTED_TYPE, "T is not supported.");
+  if (M <= 0 || N <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "M and N must be positive (got %d, %d)", M, N);
+  if (M % 128 || N % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N can't be divided 128.");
+  if (!src || !dst) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 3u) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 4-byte aligned");
+  if ((long)M * N >= (1L << 31)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
+  const size_t bytes = (size_t)M * N * elem_size;
+  const char * a = (const char*)src, *b = (const char*)dst;
+  if (a < b + bytes && b < a + bytes) return fail(LLMMM_ERR_INVALID_ARGUMENT, "source and destination overlap");
+  const hipError_t e = llmmm::transpose_launch(elem_size, src, dst, M, N, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "transpose launch: %s", hipGetErrorString(e));
   return LLMMM_OK;
 }
 

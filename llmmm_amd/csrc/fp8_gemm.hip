@@ -70,21 +70,27 @@ __device__ __forceinline__ void fp8_load_f32(float& dst, const void* sbase, unsi
 // per-lane offset: load i covers tile rows 8*(wave + i*NW) .. +7, and the SWZ_ROWS16 placement
 // only looks at row bits 0..3, so moving by 8*NW (>= 16) rows changes nothing but the
 // wave-uniform row base.
+//
+// Pre-shuffled weights (layout.hip) hold the same LDS image as consecutive 1 KB half blocks: half
+// block h of row group rg and slice kb at ((rg * K/128 + kb) * 2 + h) * 1024.  Rows 8*NW apart
+// are then 8*NW*K bytes apart as well, so only the per-lane offset (16 * lane instead of
+// row * K + chunk * 16, the wave's own rows folded into the base) and the step from slice to
+// slice (2048 instead of 128 bytes) differ between the two layouts.
 template <int BM, int BN, int WM, int I>
-__device__ __forceinline__ void fp8_issue_load(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned lane_off, int K, int wave)
+__device__ __forceinline__ void fp8_issue_load(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned a_off, unsigned b_off, int K, int wave)
 {
   typedef Fp8Tile<BM, BN, WM> TC;
   if constexpr (I < TC::A_LOADS)
-    fp8_load_lds_16B(Ag + (size_t)(8 * TC::NW * I) * K, lane_off, lds_stage + (wave + I * TC::NW) * 1024);
+    fp8_load_lds_16B(Ag + (size_t)(8 * TC::NW * I) * K, a_off, lds_stage + (wave + I * TC::NW) * 1024);
   else if constexpr (I < TC::A_LOADS + TC::B_LOADS)
-    fp8_load_lds_16B(Bg + (size_t)(8 * TC::NW * (I - TC::A_LOADS)) * K, lane_off, lds_stage + TC::A_BYTES + (wave + (I - TC::A_LOADS) * TC::NW) * 1024);
+    fp8_load_lds_16B(Bg + (size_t)(8 * TC::NW * (I - TC::A_LOADS)) * K, b_off, lds_stage + TC::A_BYTES + (wave + (I - TC::A_LOADS) * TC::NW) * 1024);
 }
 template <int BM, int BN, int WM, int FIRST, int COUNT>
-__device__ __forceinline__ void fp8_issue_loads(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned lane_off, int K, int wave)
+__device__ __forceinline__ void fp8_issue_loads(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned a_off, unsigned b_off, int K, int wave)
 {
   if constexpr (COUNT > 0) {
-    fp8_issue_load<BM, BN, WM, FIRST>(lds_stage, Ag, Bg, lane_off, K, wave);
-    fp8_issue_loads<BM, BN, WM, FIRST + 1, COUNT - 1>(lds_stage, Ag, Bg, lane_off, K, wave);
+    fp8_issue_load<BM, BN, WM, FIRST>(lds_stage, Ag, Bg, a_off, b_off, K, wave);
+    fp8_issue_loads<BM, BN, WM, FIRST + 1, COUNT - 1>(lds_stage, Ag, Bg, a_off, b_off, K, wave);
   }
 }
 // The slice scales of the lane's four 16-row fragments and of the wave's column group.
@@ -129,7 +135,7 @@ struct Fp8Next {
 template <int BM, int BN, int WM, bool LOAD>
 __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int a_rd0, int a_rd1, int b_rd0, int b_rd1,
                                                   const float (&s)[WM / 16], f32x4 (&acc)[8][WM / 16], const Fp8Next& nx, unsigned lane_off,
-                                                  unsigned row_off, unsigned zero, int K, int wave, float (&sa_next)[WM / 16],
+                                                  unsigned b_lane_off, unsigned row_off, unsigned zero, int K, int wave, float (&sa_next)[WM / 16],
                                                   float& sb_next)
 {
   constexpr int MF = WM / 16;
@@ -148,10 +154,10 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int
     const int cur = nf & 1;
     if (nf + 1 < 8) b[cur ^ 1] = fp8_read_frag(ldsB, b_rd0, b_rd1, (nf + 1) * 2048);
     if constexpr (LOAD) {
-      if (nf == 0) fp8_issue_loads<BM, BN, WM, 0, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
-      if (nf == 1) fp8_issue_loads<BM, BN, WM, LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
-      if (nf == 2) fp8_issue_loads<BM, BN, WM, 2 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
-      if (nf == 3) fp8_issue_loads<BM, BN, WM, 3 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, K, wave);
+      if (nf == 0) fp8_issue_loads<BM, BN, WM, 0, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, wave);
+      if (nf == 1) fp8_issue_loads<BM, BN, WM, LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, wave);
+      if (nf == 2) fp8_issue_loads<BM, BN, WM, 2 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, wave);
+      if (nf == 3) fp8_issue_loads<BM, BN, WM, 3 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, wave);
       if (nf == 4) fp8_issue_scales<MF>(sa_next, sb_next, nx.As_slice, row_off, nx.Bs_elem, zero);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -205,7 +211,8 @@ __device__ __forceinline__ uint32_t pack_e4m3x4_in_range(float a, float b, float
   return (uint32_t)v;
 }
 
-template <int BM, int BN, int WM, int OUT>
+// BPRE: Bt is the pre-shuffled image of the weights (layout.hip) instead of row-major [N, K].
+template <int BM, int BN, int WM, int OUT, bool BPRE>
 __global__ void __launch_bounds__((BM / WM) * (BN / 128) * 64)
 fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
                 const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int tiles_m,
@@ -235,7 +242,11 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const KMajorLane lp       = kmajor_lane<SWZ_ROWS16>(wave, lane);
   const unsigned   lane_off = (unsigned)(lp.row * K + lp.chunk * 16);
   const uint8_t*   Ag       = A + (size_t)m0 * K + (size_t)kb0 * 128;
-  const uint8_t*   Bg       = Bt + (size_t)n0 * K + (size_t)kb0 * 128;
+  // pre-shuffled: row 8*wave of the tile starts half block (wave & 1) of row group n0/16 + wave/2
+  constexpr int    B_KSTEP    = BPRE ? 2048 : 128;  // bytes from one slice to the next
+  const unsigned   b_lane_off = BPRE ? (unsigned)lane * 16u : lane_off;
+  const uint8_t*   Bg         = BPRE ? Bt + (size_t)(n0 + 16 * (wave >> 1)) * K + (wave & 1) * 1024 + (size_t)kb0 * 2048
+                                     : Bt + (size_t)n0 * K + (size_t)kb0 * 128;
 
   // operand reads: lane = (g = lane/16, i = lane%16) takes row i of a 16-row fragment and the
   // 32 bytes k = 32g .. 32g+31 (chunks 2g and 2g+1)
@@ -261,7 +272,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const unsigned lds0 = (unsigned)(size_t)(char LLMMM_LDS*)lds;
   char LLMMM_LDS* const s0 = (char LLMMM_LDS*)lds;
 
-  fp8_issue_loads<BM, BN, WM, 0, TC::A_LOADS + TC::B_LOADS>(lds0, Ag, Bg, lane_off, K, wave);
+  fp8_issue_loads<BM, BN, WM, 0, TC::A_LOADS + TC::B_LOADS>(lds0, Ag, Bg, lane_off, b_lane_off, K, wave);
   fp8_issue_scales<MF>(sa_next, sb_next, Asl, row_off, Bsp, zero);
 
   // One slice: wait for this wave's loads of the slice (all of them were issued at least half a
@@ -279,10 +290,10 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
     Fp8Next nx;                                                                                                                   \
     nx.lds_stage = NXT_LDS;                                                                                                       \
     nx.Ag        = Ag + (size_t)((KC) + 1) * 128;                                                                                 \
-    nx.Bg        = Bg + (size_t)((KC) + 1) * 128;                                                                                 \
+    nx.Bg        = Bg + (size_t)((KC) + 1) * B_KSTEP;                                                                               \
     nx.As_slice  = Asl + (size_t)((KC) + 1) * M;                                                                                  \
     nx.Bs_elem   = Bsp + (KC) + 1;                                                                                                \
-    fp8_compute_stage<BM, BN, WM, LOAD>(CUR, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, row_off, zero, K, wave, sa_next,       \
+    fp8_compute_stage<BM, BN, WM, LOAD>(CUR, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, b_lane_off, row_off, zero, K, wave, sa_next, \
                                     sb_next);                                                                                     \
   }
 
@@ -437,18 +448,20 @@ static hipError_t launch_reduce(const float* planes, int S, void* C, float* Cs, 
 
 template <int BM, int BN, int WM, int OUT>
 static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N,
-                             int K, int S, float* planes, hipStream_t stream)
+                             int K, int S, float* planes, bool bpre, hipStream_t stream)
 {
   typedef Fp8Tile<BM, BN, WM> TC;
   const int tiles_m = M / BM, tiles_n = N / BN;
   if (S <= 1) {
-    hipLaunchKernelGGL((fp8_gemm_kernel<BM, BN, WM, OUT>), dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As,
-                       (const uint8_t*)Bt, Bs, C, Cs, M, N, K, tiles_m, tiles_n);
+    const auto kernel = bpre ? fp8_gemm_kernel<BM, BN, WM, OUT, true> : fp8_gemm_kernel<BM, BN, WM, OUT, false>;
+    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs,
+                       M, N, K, tiles_m, tiles_n);
     return hipGetLastError();
   }
   // split-K: S partial planes from the fp32 instantiation, then the ordered sum + epilogue
-  hipLaunchKernelGGL((fp8_gemm_kernel<BM, BN, WM, OUT_F32>), dim3(tiles_m * tiles_n, S), dim3(TC::NT), 0, stream, (const uint8_t*)A, As,
-                     (const uint8_t*)Bt, Bs, (void*)planes, (float*)nullptr, M, N, K, tiles_m, tiles_n);
+  const auto kernel = bpre ? fp8_gemm_kernel<BM, BN, WM, OUT_F32, true> : fp8_gemm_kernel<BM, BN, WM, OUT_F32, false>;
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, S), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs,
+                     (void*)planes, (float*)nullptr, M, N, K, tiles_m, tiles_n);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   return launch_reduce<OUT>(planes, S, C, Cs, M, N, stream);
@@ -456,25 +469,26 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
 
 template <int OUT>
 static hipError_t dispatch_fp8(int tile, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
-                               int M, int N, int K, int S, float* planes, hipStream_t stream)
+                               int M, int N, int K, int S, float* planes, bool bpre, hipStream_t stream)
 {
   // the 256 x 256 tile uses eight 64-row waves; the smaller tiles 32-row waves (twice the waves per SIMD)
   switch (tile) {
-    case LLMMM_TILE_256x256: return launch_fp8<256, 256, 64, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
-    case LLMMM_TILE_128x256: return launch_fp8<128, 256, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
-    case LLMMM_TILE_256x128: return launch_fp8<256, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
-    case LLMMM_TILE_128x128: return launch_fp8<128, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case LLMMM_TILE_256x256: return launch_fp8<256, 256, 64, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
+    case LLMMM_TILE_128x256: return launch_fp8<128, 256, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
+    case LLMMM_TILE_256x128: return launch_fp8<256, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
+    case LLMMM_TILE_128x128: return launch_fp8<128, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
     default: return hipErrorInvalidValue;
   }
 }
 
-hipError_t fp8_gemm_launch(int out_kind, int tile, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
-                           float* Cs, int M, int N, int K, int S, float* planes, hipStream_t stream)
+hipError_t fp8_gemm_launch(int out_kind, int tile, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs,
+                           void* C, float* Cs, int M, int N, int K, int S, float* planes, hipStream_t stream)
 {
+  const bool bpre = b_layout == LLMMM_FP8_B_PRESHUFFLED;
   switch (out_kind) {
-    case OUT_F32: return dispatch_fp8<OUT_F32>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
-    case OUT_BF16: return dispatch_fp8<OUT_BF16>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
-    case OUT_FP8Q: return dispatch_fp8<OUT_FP8Q>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, stream);
+    case OUT_F32: return dispatch_fp8<OUT_F32>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
+    case OUT_BF16: return dispatch_fp8<OUT_BF16>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
+    case OUT_FP8Q: return dispatch_fp8<OUT_FP8Q>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
     default: return hipErrorInvalidValue;
   }
 }

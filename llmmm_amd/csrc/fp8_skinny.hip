@@ -56,12 +56,12 @@ constexpr int SKINNY_LOADS_PER_SLOT_BASE = 2;  // LDS-direct loads; + 3 (or 1, w
 // All vector-memory loads of a slot, in a fixed order, as inline assembly (see device_common.hip.h):
 // the kernel counts them itself.
 template <int MBLK, bool APRE>
-__device__ __forceinline__ void skinny_fetch(SkinnySlot<MBLK, APRE>& t, unsigned ring_slot, const uint8_t* wrow, unsigned w_off0,
-                                             unsigned w_off1, const uint8_t* const (&ap)[MBLK], const float* const (&asp)[MBLK],
+__device__ __forceinline__ void skinny_fetch(SkinnySlot<MBLK, APRE>& t, unsigned ring_slot, const uint8_t* wrow, int w_kstep,
+                                             unsigned w_off0, unsigned w_off1, const uint8_t* const (&ap)[MBLK], const float* const (&asp)[MBLK],
                                              const float* bsp, int kb, int M)
 {
-  asm_load_lds_16B(wrow + (size_t)kb * 128 + w_off0, ring_slot);
-  asm_load_lds_16B(wrow + (size_t)kb * 128 + w_off1, ring_slot + 1024);
+  asm_load_lds_16B(wrow + (size_t)kb * w_kstep + w_off0, ring_slot);
+  asm_load_lds_16B(wrow + (size_t)kb * w_kstep + w_off1, ring_slot + 1024);
 #pragma unroll
   for (int mb = 0; mb < MBLK; ++mb) {
     if constexpr (!APRE) {
@@ -145,7 +145,7 @@ template <int MBLK, int OUT, int D, int ASTG>
 __global__ void __launch_bounds__(512)
 fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
                   const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int S,
-                  float* __restrict__ partial)
+                  float* __restrict__ partial, int bpre)
 {
   constexpr bool APRE  = ASTG > 0;
   constexpr int  LOADS = SKINNY_LOADS_PER_SLOT_BASE + (APRE ? 1 : 3) * MBLK;  // vector-memory loads per slot, issued in slot order
@@ -184,10 +184,14 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   for (int u = 0; u < 8; ++u) ring_addr[u] = __builtin_amdgcn_readfirstlane((unsigned)(size_t)ring[u]);
 
   // weights: loader lane -> (row, chunk) of the 1 KB group it fills; reader lane (g, i) -> row i, chunks 2g, 2g+1
+  // pre-shuffled weights (bpre, layout.hip): the wave's 16 rows x 128 bytes of a slice are one 2 KB block that
+  // already is the ring slot's image, and the blocks of consecutive slices follow each other
   const uint8_t*   wrow = Bt + (size_t)(ng * 128 + wave * 16) * K;
   const KMajorLane l0   = kmajor_lane<SWZ_ROWS16>(0, lane);
   const KMajorLane l1   = kmajor_lane<SWZ_ROWS16>(1, lane);
-  const unsigned   w_off0 = (unsigned)(l0.row * K + l0.chunk * 16), w_off1 = (unsigned)(l1.row * K + l1.chunk * 16);
+  const unsigned   w_off0   = bpre ? (unsigned)lane * 16u : (unsigned)(l0.row * K + l0.chunk * 16);
+  const unsigned   w_off1   = bpre ? 1024u + (unsigned)lane * 16u : (unsigned)(l1.row * K + l1.chunk * 16);
+  const int        w_kstep  = bpre ? 2048 : 128;
   const int        w_rd   = kmajor_offset<SWZ_ROWS16>(i, 2 * g);
   const float*     bsp    = Bs + (size_t)ng * KB;
   const uint8_t*   ap[MBLK];
@@ -229,7 +233,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   SkinnySlot<MBLK, APRE> slot[D];
 #pragma unroll
   for (int u = 0; u < D; ++u) {
-    skinny_fetch<MBLK, APRE>(slot[u], ring_addr[u], wrow, w_off0, w_off1, ap, asp, bsp, min(kb0 + u, kb1 - 1), M);
+    skinny_fetch<MBLK, APRE>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb0 + u, kb1 - 1), M);
     __builtin_amdgcn_sched_barrier(0);
   }
   if constexpr (APRE) {
@@ -243,7 +247,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
       skinny_wait<(D - 1) * LOADS, MBLK, APRE>(slot[u]);
       skinny_consume<MBLK, APRE>(slot[u], ring[u], w_rd, true, acc, a_tile + (kb + u - kb0) * (MBLK * 2048), a_rd);
       __builtin_amdgcn_sched_barrier(0);
-      skinny_fetch<MBLK, APRE>(slot[u], ring_addr[u], wrow, w_off0, w_off1, ap, asp, bsp, min(kb + u + D, kb1 - 1), M);
+      skinny_fetch<MBLK, APRE>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb + u + D, kb1 - 1), M);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -321,10 +325,10 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
 
 template <int MBLK, int OUT, int D, int ASTG>
 static hipError_t launch_skinny(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
-                                int N, int K, int S, float* partial, hipStream_t stream)
+                                int N, int K, int S, float* partial, int bpre, hipStream_t stream)
 {
   hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D, ASTG>), dim3(N / 128, S, MBLK == 8 ? (M + 127) / 128 : (M + 63) / 64), dim3(512), 0, stream,
-                     (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial);
+                     (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial, bpre);
   return hipGetLastError();
 }
 
@@ -333,12 +337,12 @@ static hipError_t launch_skinny(const void* A, const float* As, const void* Bt, 
 // 8-deep ring, 64 KB beside a 4-deep one); otherwise the per-slice register path.
 template <int OUT>
 static hipError_t dispatch_skinny(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
-                                  int N, int K, int S, float* partial, hipStream_t stream)
+                                  int N, int K, int S, float* partial, int bpre, hipStream_t stream)
 {
   const int KB     = K / 128;
   const int slices = KB / S;              // of the shortest split
   const int longest = (KB + S - 1) / S;   // of the longest
-#define LLMMM_GO(MBLK, D, ASTG) return launch_skinny<MBLK, OUT, D, ASTG>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, stream)
+#define LLMMM_GO(MBLK, D, ASTG) return launch_skinny<MBLK, OUT, D, ASTG>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, bpre, stream)
   if (M <= 16) {
     const int need = 2048 * longest;
     if (slices >= 8 && need <= 28672) LLMMM_GO(1, 8, 28672);
@@ -370,13 +374,14 @@ static hipError_t dispatch_skinny(const void* A, const float* As, const void* Bt
   return hipErrorInvalidValue;
 }
 
-hipError_t fp8_skinny_launch(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
-                             int M, int N, int K, int S, float* partial, hipStream_t stream)
+hipError_t fp8_skinny_launch(int out_kind, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
+                             float* Cs, int M, int N, int K, int S, float* partial, hipStream_t stream)
 {
+  const int bpre = b_layout == LLMMM_FP8_B_PRESHUFFLED;
   switch (out_kind) {
-    case SK_OUT_F32: return dispatch_skinny<SK_OUT_F32>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, stream);
-    case SK_OUT_BF16: return dispatch_skinny<SK_OUT_BF16>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, stream);
-    case SK_OUT_FP8Q: return dispatch_skinny<SK_OUT_FP8Q>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, stream);
+    case SK_OUT_F32: return dispatch_skinny<SK_OUT_F32>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, bpre, stream);
+    case SK_OUT_BF16: return dispatch_skinny<SK_OUT_BF16>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, bpre, stream);
+    case SK_OUT_FP8Q: return dispatch_skinny<SK_OUT_FP8Q>(A, As, Bt, Bs, C, Cs, M, N, K, S, partial, bpre, stream);
     default: return hipErrorInvalidValue;
   }
 }

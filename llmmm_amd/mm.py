@@ -128,7 +128,7 @@ def query_config(out_kind, M, N, K):
     return cfg.tile, cfg.split_k
 
 
-def _fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, workspace, tile, split_k, stream):
+def _fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, workspace, tile, split_k, stream, b_preshuffled=False):
     kb = K // 128 if K % 128 == 0 else 0
     c_dtypes = {_lib.OUT_F32: (torch.float32,), _lib.OUT_BF16: (torch.bfloat16,), _lib.OUT_FP8Q: _FP8_DTYPES}[out_kind]
     a_p = _ptr(A, "A", _FP8_DTYPES, M * K)
@@ -138,26 +138,66 @@ def _fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, workspace, tile, split_k,
     c_p = _ptr(C, "C", c_dtypes, M * N)
     cs_p = _ptr(Cs, "C_scale_transposed", (torch.float32,), ((N + 127) // 128) * M) if out_kind == _lib.OUT_FP8Q else None
     ws_p, ws_n = (ctypes.c_void_p(workspace.data_ptr()), workspace.numel() * workspace.element_size()) if workspace is not None else (None, 0)
-    cfg = GemmCfg(tile, split_k)
+    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS)
     check(lib.llmmm_fp8_gemm_ex(out_kind, a_p, as_p, b_p, bs_p, c_p, cs_p, M, N, K, ws_p, ws_n, ctypes.byref(cfg), _stream(stream)))
 
 
 def fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(A, A_scale_transposed, B_transposed, B_scale_transposed, C, M, N, K,
-                                                             stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0):
-    """examples/005.fp8.mm.cu:217-246.  C [M,N] float32."""
-    _fp8_gemm(_lib.OUT_F32, A, A_scale_transposed, B_transposed, B_scale_transposed, C, None, M, N, K, workspace, tile, split_k, stream)
+                                                             stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0,
+                                                             b_preshuffled=False):
+    """examples/005.fp8.mm.cu:217-246.  C [M,N] float32.  ``b_preshuffled``: B_transposed is the image written by
+    :func:`construct_mfma_B_layout` instead of row-major [N,K] (same results, bit for bit)."""
+    _fp8_gemm(_lib.OUT_F32, A, A_scale_transposed, B_transposed, B_scale_transposed, C, None, M, N, K, workspace, tile, split_k, stream,
+              b_preshuffled)
 
 
 def fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(A, A_scale_transposed, B_transposed, B_scale_transposed, C, M, N, K,
-                                                             stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0):
+                                                             stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0,
+                                                             b_preshuffled=False):
     """The fp32 variant's result rounded to bfloat16 (no reference kernel; same signature)."""
-    _fp8_gemm(_lib.OUT_BF16, A, A_scale_transposed, B_transposed, B_scale_transposed, C, None, M, N, K, workspace, tile, split_k, stream)
+    _fp8_gemm(_lib.OUT_BF16, A, A_scale_transposed, B_transposed, B_scale_transposed, C, None, M, N, K, workspace, tile, split_k, stream,
+              b_preshuffled)
 
 
 def fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(A, A_scale_transposed, B_transposed, B_scale_transposed, C,
                                                                      C_scale_transposed, M, N, K, stream=None, workspace=None,
-                                                                     tile=_lib.TILE_AUTO, split_k=0):
+                                                                     tile=_lib.TILE_AUTO, split_k=0, b_preshuffled=False):
     """examples/005.fp8.mm.cu:2467-2500 / examples/005.fp8.mm.opt.cu:468-508.  C e4m3 codes [M,N],
     C_scale_transposed float32 [N/128, M]."""
     _fp8_gemm(_lib.OUT_FP8Q, A, A_scale_transposed, B_transposed, B_scale_transposed, C, C_scale_transposed, M, N, K, workspace, tile,
-              split_k, stream)
+              split_k, stream, b_preshuffled)
+
+
+# ------------------------------------------------------------------------------------- offline layout helpers
+def construct_mfma_B_layout(dst, src_transposed, N, K, stream=None):
+    """The role of ``LLMMM::construct_m16n8k32_B_layout(dst, src_transposed, N, K, stream)``
+    (src/base/base.h:13, src/base/base.cu:222-271): the weights Bt [N,K] e4m3, permuted once into the order the
+    matrix instructions read them in -- here the 16x16x128 MFMA operand image of gfx950, consumed by the FP8 GEMMs
+    with ``b_preshuffled=True``.  Raises RuntimeError("K must be greater than 0 and divisible by 128.") like the
+    reference (base.cu:265-267)."""
+    check(lib.llmmm_fp8_preshuffle_b(_ptr(src_transposed, "src_transposed", _FP8_DTYPES, N * K), _ptr(dst, "dst", _FP8_DTYPES, N * K), N, K,
+                                     _stream(stream)))
+
+
+def restore_B_layout(dst_transposed, src, N, K, stream=None):
+    """Exact inverse of :func:`construct_mfma_B_layout` (the reference checks its permutation the same way,
+    examples/005.fp8.mm.opt.cu:710-765)."""
+    check(lib.llmmm_fp8_unshuffle_b(_ptr(src, "src", _FP8_DTYPES, N * K), _ptr(dst_transposed, "dst_transposed", _FP8_DTYPES, N * K), N, K,
+                                    _stream(stream)))
+
+
+def preshuffle_weight(bq, stream=None):
+    """Bt [N,K] e4m3 codes -> a new tensor holding the pre-shuffled image (same shape and dtype)."""
+    N, K = bq.shape
+    out = torch.empty_like(bq)
+    construct_mfma_B_layout(out, bq, N, K, stream)
+    return out
+
+
+def transpose_matrix__aligned_128(dst, src, M, N, stream=None):
+    """``LLMMM::transpose_matrix__aligned_128<T>(dst, src, M, N, stream)`` (src/base/base.cu:124-153): dst [N,M] =
+    transpose of src [M,N] for 1-byte (e4m3) and 4-byte (float) elements.  Raises
+    RuntimeError("M or N can't be divided 128.") unless both are multiples of 128 (base.cu:127-129)."""
+    if src.dtype != dst.dtype or src.element_size() not in (1, 4):
+        raise RuntimeError("T is not supported.")
+    check(lib.llmmm_transpose(src.element_size(), _ptr(src, "src", numel=M * N), _ptr(dst, "dst", numel=M * N), M, N, _stream(stream)))

@@ -134,7 +134,7 @@ def main():
     if args.write:
         with open(os.path.join(HERE, "csrc", "tune_table.h"), "w") as f:
             f.write(text)
-        print("wrote csrc/tune_table.h -- rebuild with `python -m llmmm_amd.build`", file=sys.stderr)
+        print("wrote csrc/tune_table.h -- rebuild with `python llmmm_amd/build.py`", file=sys.stderr)
 
 
 if __name__ == "__main__":

@@ -230,3 +230,53 @@ def requant_c_1x128(C, reciprocal=True, zero_guard=True):
     _lib.oracle_requant_c_1x128(_p(C, ctypes.c_float), _p(Cq, ctypes.c_uint8), _p(Cs, ctypes.c_float), M, N,
                                 int(reciprocal), int(zero_guard))
     return Cq, Cs
+
+
+# ----------------------------------------------------------------------------- offline layouts
+def operand_swizzle_rows16(r):
+    """Chunk XOR of row r (0..15) in the 16-row x 128-byte MFMA operand image of the pre-shuffled
+    weights: 16-byte chunk c of row r sits at r*128 + ((c ^ swz(r)) << 4)."""
+    r = np.asarray(r)
+    return ((r >> 1) & 7) ^ ((((r >> 2) ^ (r >> 3)) & 1) << 1)
+
+
+def preshuffle_b(Bt):
+    """The pre-shuffled image of Bt [N,K] (1-byte elements; N % 16 == 0, K % 128 == 0), returned in Bt's shape.
+
+    The MI355X counterpart of construct_m16n8k32_B_layout (src/base/base.cu:222-271): block
+    (n/16, k/128) of 2 KB at ((n/16) * (K/128) + k/128) * 2048 holds its 16 rows x 128 bytes with the
+    chunks of row r XOR-ed by operand_swizzle_rows16(r).  Pinned by tests/test_oracle_layout.py
+    (bijection, block and row confinement, conflict-free operand reads) and, on the GPU, by the
+    bit-identity of GEMM results over both layouts."""
+    Bt = _u8(Bt)
+    N, K = Bt.shape
+    if N % 16 or K % 128:
+        raise RuntimeError("K must be greater than 0 and divisible by 128." if K % 128 else "N must be divisible by 16.")
+    src = Bt.reshape(N // 16, 16, K // 128, 8, 16).transpose(0, 2, 1, 3, 4)  # [rg, kb, r, c, byte]
+    out = np.empty_like(src)
+    r = np.arange(16)
+    swz = operand_swizzle_rows16(r)
+    for c in range(8):
+        out[:, :, r, c ^ swz, :] = src[:, :, r, c, :]
+    return np.ascontiguousarray(out).reshape(N, K)
+
+
+def unshuffle_b(Bp):
+    """Inverse of preshuffle_b."""
+    Bp = _u8(Bp)
+    N, K = Bp.shape
+    img = Bp.reshape(N // 16, K // 128, 16, 8, 16)
+    out = np.empty_like(img)
+    r = np.arange(16)
+    swz = operand_swizzle_rows16(r)
+    for c in range(8):
+        out[:, :, r, c, :] = img[:, :, r, c ^ swz, :]
+    return np.ascontiguousarray(out.transpose(0, 2, 1, 3, 4)).reshape(N, K)
+
+
+def transpose_aligned_128(src):
+    """transpose_matrix__aligned_128 (src/base/base.cu:124-153): dst[n, m] = src[m, n], M and N multiples of 128."""
+    M, N = src.shape
+    if M % 128 or N % 128:
+        raise RuntimeError("M or N can't be divided 128.")
+    return np.ascontiguousarray(src.T)

@@ -3,6 +3,7 @@
 // driven the way test/fp16_mm_test.cc drives them: raw device pointers, nullptr stream, sync outside.
 // Checks the reference's closed-form known answers (A = I corner; B = I) and the exception texts.
 #include "llmmm/mm/fp16/mm.h"
+#include "llmmm/base/base.h"
 #include "llmmm/mm/fp8/mm.h"
 
 #include <hip/hip_runtime.h>
@@ -95,6 +96,38 @@ int main()
                    "M or N or K are not aligned.")) { ++fails; printf("fp8 misaligned N: FAIL\n"); }
   if (!throws_with([&] { LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(dAq, dAs, dBq, dBs, dCq, dCs, 200, N, K, nullptr); },
                    "M or N or K are not aligned.")) { ++fails; printf("fp8 misaligned M: FAIL\n"); }
+  // ---- layout helpers (src/base/base.h:8-13): transpose twice == identity and == the host transpose
+  // (test/transpose_matrix__aligned_128_test.cc:16-35 compares bytes the same way); pre-shuffle + GEMM == GEMM
+  {
+    LLMMM::fp8_t *dT, *dTT, *dBp, *dBack, *dCq2;
+    float*        dCs2;
+    CHECK(hipMalloc(&dT, M * K)); CHECK(hipMalloc(&dTT, M * K)); CHECK(hipMalloc(&dBp, N * K)); CHECK(hipMalloc(&dBack, N * K));
+    CHECK(hipMalloc(&dCq2, M * N)); CHECK(hipMalloc(&dCs2, (N / 128) * M * 4));
+    LLMMM::transpose_matrix__aligned_128(dT, dAq, M, K, nullptr);
+    LLMMM::transpose_matrix__aligned_128(dTT, dT, K, M, nullptr);
+    LLMMM::construct_m16n8k32_B_layout(dBp, dBq, N, K, nullptr);
+    LLMMM::restore_B_layout(dBack, dBp, N, K, nullptr);
+    llmmm_gemm_cfg cfg = {LLMMM_TILE_AUTO, 0, LLMMM_FP8_B_PRESHUFFLED};
+    if (llmmm_fp8_gemm_ex(LLMMM_OUT_FP8Q, dAq, dAs, dBp, dBs, dCq2, dCs2, M, N, K, nullptr, 0, &cfg, nullptr) != LLMMM_OK) ++fails;
+    CHECK(hipDeviceSynchronize());
+    std::vector<unsigned char> hT(M * K), hTT(M * K), hBq(N * K), hBack(N * K), hCq2(M * N);
+    CHECK(hipMemcpy(hT.data(), dT, hT.size(), hipMemcpyDeviceToHost));
+    CHECK(hipMemcpy(hTT.data(), dTT, hTT.size(), hipMemcpyDeviceToHost));
+    CHECK(hipMemcpy(hBq.data(), dBq, hBq.size(), hipMemcpyDeviceToHost));
+    CHECK(hipMemcpy(hBack.data(), dBack, hBack.size(), hipMemcpyDeviceToHost));
+    CHECK(hipMemcpy(hCq2.data(), dCq2, hCq2.size(), hipMemcpyDeviceToHost));
+    int fl = 0;
+    for (int m = 0; m < M; ++m)
+      for (int k = 0; k < K; ++k)
+        if (hT[(size_t)k * M + m] != hAq[(size_t)m * K + k]) ++fl;
+    if (memcmp(hTT.data(), hAq.data(), hAq.size()) != 0) ++fl;
+    if (memcmp(hBack.data(), hBq.data(), hBq.size()) != 0) ++fl;
+    if (memcmp(hCq2.data(), hCq.data(), hCq.size()) != 0) ++fl;
+    printf("transpose / pre-shuffle round trips, GEMM over pre-shuffled weights: %s\n", fl ? "FAIL" : "ok");
+    fails += fl;
+    if (!throws_with([&] { LLMMM::transpose_matrix__aligned_128(dT, dAq, 100, K, nullptr); }, "M or N can't be divided 128.")) { ++fails; printf("transpose misaligned: FAIL\n"); }
+    if (!throws_with([&] { LLMMM::construct_m16n8k32_B_layout(dBp, dBq, N, 100, nullptr); }, "K must be greater than 0 and divisible by 128.")) { ++fails; printf("layout misaligned K: FAIL\n"); }
+  }
   printf(fails ? "DROPIN FAIL (%d)\n" : "DROPIN OK\n", fails);
   return fails ? 1 : 0;
 }

@@ -140,3 +140,32 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".cpp", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "import oracle" not in text and "from oracle" not in text and "liboracle" not in text, f
+
+
+def test_layout_helpers_validation_without_device():
+    """Texts of src/base/base.cu:127-129 ("M or N can't be divided 128.") and :265-267 ("K must be ...")."""
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    A, B = ctypes.c_void_p(0x100000), ctypes.c_void_p(0x900000)
+    for f in (lib.llmmm_fp8_preshuffle_b, lib.llmmm_fp8_unshuffle_b):
+        assert f(A, B, 128, 100, None) == _lib.ERR_NOT_ALIGNED
+        assert lib.llmmm_last_error() == b"K must be greater than 0 and divisible by 128."
+        assert f(A, B, 24, 128, None) == _lib.ERR_NOT_ALIGNED
+        assert f(A, B, 0, 128, None) == _lib.ERR_INVALID_ARGUMENT
+        assert f(None, B, 128, 128, None) == _lib.ERR_INVALID_ARGUMENT
+        assert f(A, ctypes.c_void_p(0x900004), 128, 128, None) == _lib.ERR_INVALID_ARGUMENT
+        assert f(A, A, 128, 128, None) == _lib.ERR_INVALID_ARGUMENT  # in place
+        assert f(A, ctypes.c_void_p(0x100000 + 128 * 64), 128, 128, None) == _lib.ERR_INVALID_ARGUMENT  # overlap
+    t = lib.llmmm_transpose
+    assert t(1, A, B, 128, 100, None) == _lib.ERR_NOT_ALIGNED
+    assert lib.llmmm_last_error() == b"M or N can't be divided 128."
+    assert t(4, A, B, 200, 128, None) == _lib.ERR_NOT_ALIGNED
+    assert t(2, A, B, 128, 128, None) == _lib.ERR_UNSUPPORTED_TYPE
+    assert t(4, A, A, 128, 128, None) == _lib.ERR_INVALID_ARGUMENT
+    assert t(4, None, B, 128, 128, None) == _lib.ERR_INVALID_ARGUMENT
+    # an unknown weight layout is rejected before any launch
+    cfg = _lib.GemmCfg(_lib.TILE_AUTO, 0, 7)
+    args = (FAKE, FAKE, FAKE, FAKE, FAKE, FAKE)
+    assert lib.llmmm_fp8_gemm_ex(2, *args, 128, 128, 256, None, 0, ctypes.byref(cfg), None) == _lib.ERR_INVALID_ARGUMENT
+    q = _lib.GemmCfg(5, 5, 5)
+    assert lib.llmmm_fp8_gemm_query(2, 128, 128, 256, ctypes.byref(q)) == _lib.OK and q.b_layout == _lib.FP8_B_ROWS

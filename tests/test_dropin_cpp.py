@@ -17,7 +17,7 @@ def test_shims_compile_and_link():
 
 @pytest.mark.gpu
 def test_dropin_known_answers_on_gpu():
-    assert os.path.exists(BIN), "tests/cpp/dropin_test has not been built (python -m llmmm_amd.build)"
+    assert os.path.exists(BIN), "tests/cpp/dropin_test has not been built (python llmmm_amd/build.py)"
     res = subprocess.run([BIN], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     print(res.stdout)
     assert res.returncode == 0 and "DROPIN OK" in res.stdout, res.stdout
