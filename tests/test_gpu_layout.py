@@ -83,7 +83,7 @@ def _run_three(lib, t, M, N, K, tile, split_k, pre):
 
 
 @pytest.mark.parametrize("tile,M,split_k", [("256x256", 512, 1), ("128x256", 384, 1), ("256x128", 512, 1), ("128x128", 384, 1),
-                                             ("256x256", 256, 3), ("128x128", 128, 2),
+                                             ("256x256", 256, 3), ("128x128", 128, 2), ("128x256", 128, 1), ("256x128", 256, 1), ("256x256", 256, 1),
                                              ("skinny", 1, 1), ("skinny", 16, 3), ("skinny", 33, 1), ("skinny", 64, 8),
                                              ("skinny", 100, 1), ("skinny", 128, 3)])
 def test_gemm_bit_identical_over_both_weight_layouts(lib, oracle, tile, M, split_k):
