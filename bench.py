@@ -115,7 +115,9 @@ def bench_fp16(M, N, K, steps, warmup, dtype=torch.float16, b_transposed=False):
 
 def fp8_bytes(M, N, K, out):
     b = M * K + N * K + 4.0 * (M * K / 128 + (N / 128) * (K / 128))
-    if out == "fp8q":
+    if out == "swiglu":
+        b += M * N / 2 + 4.0 * M * N / 256
+    elif out == "fp8q":
         b += M * N + 4.0 * M * N / 128
     elif out == "bf16":
         b += 2.0 * M * N
@@ -136,10 +138,11 @@ def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0, preshuffled=False):
     Aq, As, weights = fp8_inputs(M, N, K, copies=copies)
     if preshuffled:
         weights = [(llmmm_amd.preshuffle_weight(bq), bs) for bq, bs in weights]
-    kind = {"f32": _lib.OUT_F32, "bf16": _lib.OUT_BF16, "fp8q": _lib.OUT_FP8Q}[out]
-    cdt = {"f32": torch.float32, "bf16": torch.bfloat16, "fp8q": torch.uint8}[out]
-    C = torch.empty((M, N), dtype=cdt, device="cuda")
-    Cs = torch.empty((N // 128, M), dtype=torch.float32, device="cuda")
+    kind = {"f32": _lib.OUT_F32, "bf16": _lib.OUT_BF16, "fp8q": _lib.OUT_FP8Q, "swiglu": _lib.OUT_FP8Q_SWIGLU}[out]
+    cdt = {"f32": torch.float32, "bf16": torch.bfloat16, "fp8q": torch.uint8, "swiglu": torch.uint8}[out]
+    n_out = N // 2 if out == "swiglu" else N
+    C = torch.empty((M, n_out), dtype=cdt, device="cuda")
+    Cs = torch.empty((max(1, n_out // 128), M), dtype=torch.float32, device="cuda")
     ws = llmmm_amd.make_workspace(kind, M, N, K)
     fns = {"f32": llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32,
            "bf16": llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16}
@@ -148,7 +151,10 @@ def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0, preshuffled=False):
     def step():
         Bq, Bs = weights[state["i"] % copies]
         state["i"] += 1
-        if out == "fp8q":
+        if out == "swiglu":
+            llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(Aq, As, Bq, Bs, C, Cs, M, N, K, workspace=ws,
+                                                                                               b_preshuffled=preshuffled)
+        elif out == "fp8q":
             llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(Aq, As, Bq, Bs, C, Cs, M, N, K, workspace=ws,
                                                                                        b_preshuffled=preshuffled)
         else:
@@ -280,6 +286,16 @@ def main():
                     e.update({"hbm_gbs": x["gbs"], "frac_of_hbm_peak": x["gbs"] / PEAK_HBM_GBS, "weight_copies": x["weight_copies"]})
                 shapes.append(e)
                 torch.cuda.empty_cache()
+        # the gate_up projection with the SwiGLU activation fused in front of the C quantisation (output N/2 wide)
+        n, k = QWEN3_4B["gate_up"]
+        for m in (1, 16, 128, 2048):
+            x = bench_fp8(m, n, k, "swiglu", s2 * 2 if m <= 16 else s2, w2, rotate_bytes=(768 << 20) if m <= 128 else 0)
+            e = {"name": "qwen3_4b_gate_up_swiglu_m%d" % m, "M": m, "N": n, "K": k, "us": x["ms"] * 1e3, "tflops": x["tflops"],
+                 "frac_of_fp8_peak": x["tflops"] / PEAK_TFLOPS["fp8"], "tile": x["tile"], "split_k": x["split_k"]}
+            if m <= 128:
+                e.update({"hbm_gbs": x["gbs"], "frac_of_hbm_peak": x["gbs"] / PEAK_HBM_GBS, "weight_copies": x["weight_copies"]})
+            shapes.append(e)
+            torch.cuda.empty_cache()
         line["shapes"] = shapes
 
     if not args.no_cpu:

@@ -46,6 +46,8 @@ extern "C" {
 #define LLMMM_OUT_F32 0  /* ...__output_fp32              examples/005.fp8.mm.cu:217-225 */
 #define LLMMM_OUT_BF16 1 /* same result rounded to bf16 (no reference kernel; RNE cast of the fp32 result) */
 #define LLMMM_OUT_FP8Q 2 /* ...__C_1x128__output_fp8      examples/005.fp8.mm.cu:2467-2476 */
+#define LLMMM_OUT_FP8Q_SWIGLU 3 /* SiLU(gate) * up, then the same 1x128 quantisation; no reference kernel: the
+                                   fusion the reference plans next (README.md:16).  See llmmm_fp8_gemm. */
 
 #define LLMMM_QUANT_1x128_T 0   /* <1,128,true>    activations: scale[(n/128)*M + m]           examples/005.fp8.mm.cu:2686 */
 #define LLMMM_QUANT_128x128 1   /* <128,128,false> weights:     scale[(m/128)*ceil(N/128)+n/128] examples/005.fp8.mm.cu:2739 */
@@ -92,6 +94,12 @@ LLMMM_API int llmmm_fp16_gemm_ex(int dtype, const void* A, const void* B, void* 
  * MFMA tile kernels (the reference's domain); 1 <= M < 128 runs the weight-streaming kernel
  * (so does M = 128 when LLMMM_TILE_SKINNY is requested through llmmm_fp8_gemm_ex).  Other M are
  * rejected as not aligned.
+ * LLMMM_OUT_FP8Q_SWIGLU (the gate_up projection of a gated MLP): Bt holds the gate rows in [0, N/2) and the
+ * up rows in [N/2, N) (N % 256 == 0; Bs covers all N rows as usual).  With C32 = the fp32 result above,
+ * h[m,j] = silu(C32[m,j]) * C32[m,N/2+j], silu(x) = x / (1 + exp(-x)) in fp32 (hardware exp2 and
+ * reciprocal, each within about an ulp), and the output is h quantised per 1x128 like OUT_FP8Q:
+ * C = e4m3 uint8_t[M, N/2], Cs = float[(N/2)/128, M].  For M <= 128 this output always goes
+ * through the workspace (at least one plane of M * N floats is required).
  * Split-K: shapes with too few tiles or column groups to fill the GPU split K over several
  * workgroups; each split stores a plane of fp32 partial sums into `workspace` and a second
  * kernel adds the planes in split order (a fixed order: results do not depend on timing) and

@@ -74,4 +74,18 @@ inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(con
                                          N, K, nullptr, 0, (void*)stream));
 }
 
+// The gate_up projection of a gated MLP with silu(gate) * up fused in front of the C quantisation -- the
+// fusion the reference plans (README.md:16), no reference kernel.  B_transposed [N,K]: gate rows in
+// [0, N/2), up rows in [N/2, N); C [M, N/2] e4m3, C_scale_transposed [N/256, M].  M % 128 == 0 through
+// this signature (smaller M needs a workspace: llmmm_fp8_gemm with LLMMM_OUT_FP8Q_SWIGLU).
+inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(const fp8_t* A, const float* A_scale_transposed,
+                                                                                     const fp8_t* B_transposed,
+                                                                                     const float* B_scale_transposed, fp8_t* C,
+                                                                                     float* C_scale_transposed, int M, int N, int K,
+                                                                                     hipStream_t stream)
+{
+  detail8::throw_on_error(llmmm_fp8_gemm(LLMMM_OUT_FP8Q_SWIGLU, A, A_scale_transposed, B_transposed, B_scale_transposed, C,
+                                         C_scale_transposed, M, N, K, nullptr, 0, (void*)stream));
+}
+
 }  // namespace LLMMM

@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libllmmm.so")
 OK, ERR_NOT_ALIGNED, ERR_UNSUPPORTED_TYPE, ERR_INVALID_ARGUMENT, ERR_WORKSPACE, ERR_RUNTIME = range(6)
 DTYPE_F16, DTYPE_BF16 = 0, 1
 B_ROW_MAJOR, B_TRANSPOSED = 0, 1
-OUT_F32, OUT_BF16, OUT_FP8Q = 0, 1, 2
+OUT_F32, OUT_BF16, OUT_FP8Q, OUT_FP8Q_SWIGLU = 0, 1, 2, 3
 QUANT_1x128_T, QUANT_128x128, QUANT_1x128, QUANT_128x128_T = 0, 1, 2, 3
 FP8_B_ROWS, FP8_B_PRESHUFFLED = 0, 1
 TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_SKINNY = -1, 0, 1, 2, 3, 8

@@ -141,6 +141,33 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
   return LLMMM_OK;
 }
 
+// The SwiGLU output.  In the tile kernels the activation is either fused into the epilogue of a 256-column tile
+// (whose two halves are the gate and the up columns of the same outputs), or -- with a 128-column tile, or
+// whenever K is split -- applied by the reduce kernel to fp32 planes in the workspace.  The second way costs a
+// round trip of M * N floats, which only pays while that is small and the 256-column tiles would leave
+// most of the chip idle (decode-sized M).
+constexpr size_t SWIGLU_PLANE_LIMIT = 16u << 20;
+
+int choose_fp8_out(int out_kind, int M, int N, int K, llmmm_gemm_cfg* cfg)
+{
+  const int rc = choose_fp8(M, N, K, cfg);
+  if (rc) return rc;
+  if (out_kind == LLMMM_OUT_FP8Q_SWIGLU) {
+    if (N % 256) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+    if (cfg->tile != LLMMM_TILE_SKINNY && cfg->split_k <= 1) {
+      const bool narrow      = cfg->tile == LLMMM_TILE_256x128 || cfg->tile == LLMMM_TILE_128x128;
+      const long wide_tiles  = (long)(M / 128) * (N / 256);
+      const bool small_plane = (size_t)M * N * sizeof(float) <= SWIGLU_PLANE_LIMIT;
+      if (small_plane && wide_tiles < NUM_CUS / 2) {
+        if (!narrow) cfg->tile = LLMMM_TILE_128x128;  // through one fp32 plane, twice the workgroups
+      }
+      else if (narrow)
+        cfg->tile = (M % 256 == 0 && (long)(M / 256) * (N / 256) >= NUM_CUS) ? LLMMM_TILE_256x256 : LLMMM_TILE_128x256;
+    }
+  }
+  return LLMMM_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -198,32 +225,34 @@ int llmmm_fp16_gemm(int dtype, const void* A, const void* B, void* C, int M, int
 
 int llmmm_fp8_gemm_query(int out_kind, int M, int N, int K, llmmm_gemm_cfg* cfg)
 {
-  if (out_kind < LLMMM_OUT_F32 || out_kind > LLMMM_OUT_FP8Q) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown output kind %d", out_kind);
+  if (out_kind < LLMMM_OUT_F32 || out_kind > LLMMM_OUT_FP8Q_SWIGLU) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown output kind %d", out_kind);
   if (!cfg) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null cfg");
-  return choose_fp8(M, N, K, cfg);
+  return choose_fp8_out(out_kind, M, N, K, cfg);
 }
 
 size_t llmmm_fp8_gemm_workspace(int out_kind, int M, int N, int K)
 {
-  (void)out_kind;
   if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
   llmmm_gemm_cfg cfg;
-  if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
+  if (choose_fp8_out(out_kind, M, N, K, &cfg) != LLMMM_OK) return 0;
   // the weight-streaming kernel: room for any split the tuner may try; tile kernels: the split chosen
-  const int s = cfg.tile == LLMMM_TILE_SKINNY ? max_split_for(K) : cfg.split_k;
-  if (s <= 1) return 0;
-  return (size_t)s * M * N * sizeof(float);
+  const int  s       = cfg.tile == LLMMM_TILE_SKINNY ? max_split_for(K) : cfg.split_k;
+  const bool narrow  = cfg.tile == LLMMM_TILE_256x128 || cfg.tile == LLMMM_TILE_128x128;
+  const bool a_plane = out_kind == LLMMM_OUT_FP8Q_SWIGLU && (cfg.tile == LLMMM_TILE_SKINNY || narrow);  // SwiGLU outside a 256-column tile
+  if (s <= 1 && !a_plane) return 0;
+  return (size_t)(s < 1 ? 1 : s) * M * N * sizeof(float);
 }
 
 int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
                       int N, int K, void* workspace, size_t workspace_bytes, const llmmm_gemm_cfg* user, void* stream)
 {
-  if (out_kind < LLMMM_OUT_F32 || out_kind > LLMMM_OUT_FP8Q) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown output kind %d", out_kind);
+  if (out_kind < LLMMM_OUT_F32 || out_kind > LLMMM_OUT_FP8Q_SWIGLU) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown output kind %d", out_kind);
+  const bool     swiglu = out_kind == LLMMM_OUT_FP8Q_SWIGLU;
   llmmm_gemm_cfg cfg;
-  const int      rc = choose_fp8(M, N, K, &cfg);
+  const int      rc = choose_fp8_out(out_kind, M, N, K, &cfg);
   if (rc) return rc;
   if (!A || !As || !Bt || !Bs || !C) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
-  if (out_kind == LLMMM_OUT_FP8Q && !Cs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "C_scale_transposed is required for fp8 output");
+  if ((out_kind == LLMMM_OUT_FP8Q || swiglu) && !Cs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "C_scale_transposed is required for fp8 output");
   if (!aligned16(A) || !aligned16(Bt) || !aligned16(C)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
   if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
@@ -242,14 +271,20 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
     if (split < 1) split = 1;
     if (!workspace) split = 1;  // documented: no workspace, no split
     float* partial = nullptr;
-    if (split > 1) {
+    if (swiglu && !workspace) return fail(LLMMM_ERR_WORKSPACE, "the SwiGLU output at M <= %d needs a workspace of at least M * N floats", SKINNY_MAX_M);
+    if (split > 1 && !(user && user->split_k > 0)) {
+      // a split the library chose itself shrinks to what the caller's workspace holds
+      const size_t room = workspace_bytes / ((size_t)M * N * sizeof(float));
+      if ((size_t)split > room) split = room < 2 ? 1 : (int)room;
+    }
+    if (split > 1 || swiglu) {
       const size_t need = (size_t)split * M * N * sizeof(float);
       if (workspace_bytes < need) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace_bytes, split, need);
       if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
       partial = (float*)workspace;
     }
-    e = llmmm::fp8_skinny_launch(out_kind, cfg.b_layout, A, As, Bt, Bs, C, Cs, M, N, K, split, partial, (hipStream_t)stream);
-    if (e == hipSuccess && split > 1) e = llmmm::fp8_splitk_reduce_launch(out_kind, partial, split, C, Cs, M, N, (hipStream_t)stream);
+    e = llmmm::fp8_skinny_launch(partial ? LLMMM_OUT_F32 : out_kind, cfg.b_layout, A, As, Bt, Bs, C, Cs, M, N, K, split, partial, (hipStream_t)stream);
+    if (e == hipSuccess && partial) e = llmmm::fp8_splitk_reduce_launch(out_kind, partial, split, C, Cs, M, N, (hipStream_t)stream);
   }
   else {
     int bm, bn;
@@ -267,7 +302,14 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
       const size_t room  = workspace_bytes / plane;
       if ((size_t)split > room) split = room < 2 ? 1 : (int)room;
     }
-    if (split > 1) {
+    if (swiglu && split <= 1 && bn != 256 && (!workspace || workspace_bytes < (size_t)M * N * sizeof(float))) {
+      // no room for the fp32 plane a 128-column tile needs: the fused epilogue of a 256-column tile instead
+      if (user && user->tile != LLMMM_TILE_AUTO)
+        return fail(LLMMM_ERR_WORKSPACE, "the SwiGLU output from a 128-column tile needs a workspace of M * N floats");
+      cfg.tile = LLMMM_TILE_128x256;
+      bn       = 256;
+    }
+    if (split > 1 || (swiglu && bn != 256)) {
       const size_t need = (size_t)split * M * N * sizeof(float);
       if (workspace_bytes < need) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace_bytes, split, need);
       if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");

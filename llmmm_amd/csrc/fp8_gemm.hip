@@ -29,7 +29,7 @@
 
 namespace llmmm {
 
-enum { OUT_F32 = 0, OUT_BF16 = 1, OUT_FP8Q = 2 };
+enum { OUT_F32 = 0, OUT_BF16 = 1, OUT_FP8Q = 2, OUT_SWIGLU = 3 };
 
 __device__ __forceinline__ f32x4 mfma_fp8_k128(i32x8 x, i32x8 y)
 {
@@ -85,24 +85,26 @@ __device__ __forceinline__ void fp8_load_f32(float& dst, const void* sbase, unsi
 // row * K + chunk * 16, the wave's own rows folded into the base) and the step from slice to
 // slice (2048 instead of 128 bytes) differ between the two layouts.
 template <int BM, int BN, int WM, bool BNT, int I>
-__device__ __forceinline__ void fp8_issue_load(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned a_off, unsigned b_off, int K, int wave)
+__device__ __forceinline__ void fp8_issue_load(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned a_off, unsigned b_off, int K, size_t b_hi, int wave)
 {
   typedef Fp8Tile<BM, BN, WM> TC;
+  // b_hi: extra byte offset of the tile's upper half of weight rows (0 unless the two halves come from different row ranges)
+  const size_t b_skip = I - TC::A_LOADS >= TC::B_LOADS / 2 ? b_hi : 0;
   if constexpr (I < TC::A_LOADS)
     fp8_load_lds_16B(Ag + (size_t)(8 * TC::NW * I) * K, a_off, lds_stage + (wave + I * TC::NW) * 1024);
   else if constexpr (I < TC::A_LOADS + TC::B_LOADS) {
     if constexpr (BNT)
-      fp8_load_lds_16B_nt(Bg + (size_t)(8 * TC::NW * (I - TC::A_LOADS)) * K, b_off, lds_stage + TC::A_BYTES + (wave + (I - TC::A_LOADS) * TC::NW) * 1024);
+      fp8_load_lds_16B_nt(Bg + (size_t)(8 * TC::NW * (I - TC::A_LOADS)) * K + b_skip, b_off, lds_stage + TC::A_BYTES + (wave + (I - TC::A_LOADS) * TC::NW) * 1024);
     else
-      fp8_load_lds_16B(Bg + (size_t)(8 * TC::NW * (I - TC::A_LOADS)) * K, b_off, lds_stage + TC::A_BYTES + (wave + (I - TC::A_LOADS) * TC::NW) * 1024);
+      fp8_load_lds_16B(Bg + (size_t)(8 * TC::NW * (I - TC::A_LOADS)) * K + b_skip, b_off, lds_stage + TC::A_BYTES + (wave + (I - TC::A_LOADS) * TC::NW) * 1024);
   }
 }
 template <int BM, int BN, int WM, bool BNT, int FIRST, int COUNT>
-__device__ __forceinline__ void fp8_issue_loads(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned a_off, unsigned b_off, int K, int wave)
+__device__ __forceinline__ void fp8_issue_loads(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned a_off, unsigned b_off, int K, size_t b_hi, int wave)
 {
   if constexpr (COUNT > 0) {
-    fp8_issue_load<BM, BN, WM, BNT, FIRST>(lds_stage, Ag, Bg, a_off, b_off, K, wave);
-    fp8_issue_loads<BM, BN, WM, BNT, FIRST + 1, COUNT - 1>(lds_stage, Ag, Bg, a_off, b_off, K, wave);
+    fp8_issue_load<BM, BN, WM, BNT, FIRST>(lds_stage, Ag, Bg, a_off, b_off, K, b_hi, wave);
+    fp8_issue_loads<BM, BN, WM, BNT, FIRST + 1, COUNT - 1>(lds_stage, Ag, Bg, a_off, b_off, K, b_hi, wave);
   }
 }
 // The slice scales of the lane's four 16-row fragments and of the wave's column group.
@@ -147,7 +149,7 @@ struct Fp8Next {
 template <int BM, int BN, int WM, bool BNT, bool LOAD>
 __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int a_rd0, int a_rd1, int b_rd0, int b_rd1,
                                                   const float (&s)[WM / 16], f32x4 (&acc)[8][WM / 16], const Fp8Next& nx, unsigned lane_off,
-                                                  unsigned b_lane_off, unsigned row_off, unsigned zero, int K, int wave, float (&sa_next)[WM / 16],
+                                                  unsigned b_lane_off, unsigned row_off, unsigned zero, int K, size_t b_hi, int wave, float (&sa_next)[WM / 16],
                                                   float& sb_next)
 {
   constexpr int MF = WM / 16;
@@ -166,10 +168,10 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int
     const int cur = nf & 1;
     if (nf + 1 < 8) b[cur ^ 1] = fp8_read_frag(ldsB, b_rd0, b_rd1, (nf + 1) * 2048);
     if constexpr (LOAD) {
-      if (nf == 0) fp8_issue_loads<BM, BN, WM, BNT, 0, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, wave);
-      if (nf == 1) fp8_issue_loads<BM, BN, WM, BNT, LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, wave);
-      if (nf == 2) fp8_issue_loads<BM, BN, WM, BNT, 2 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, wave);
-      if (nf == 3) fp8_issue_loads<BM, BN, WM, BNT, 3 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, wave);
+      if (nf == 0) fp8_issue_loads<BM, BN, WM, BNT, 0, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
+      if (nf == 1) fp8_issue_loads<BM, BN, WM, BNT, LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
+      if (nf == 2) fp8_issue_loads<BM, BN, WM, BNT, 2 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
+      if (nf == 3) fp8_issue_loads<BM, BN, WM, BNT, 3 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
       if (nf == 4) fp8_issue_scales<MF>(sa_next, sb_next, nx.As_slice, row_off, nx.Bs_elem, zero);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -223,6 +225,64 @@ __device__ __forceinline__ uint32_t pack_e4m3x4_in_range(float a, float b, float
   return (uint32_t)v;
 }
 
+// silu(g) * u with the hardware's exp2 and reciprocal (each within about one ulp of fp32): far below the
+// resolution of the e4m3 codes the result is quantised to.  g -> -inf gives -0, g -> +inf gives g * u.
+__device__ __forceinline__ float silu_mul(float g, float u)
+{
+  const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896340736f);  // exp(-g)
+  return g * __builtin_amdgcn_rcpf(1.f + e) * u;
+}
+
+// SwiGLU exchange: the fragments mf = SEND0 .. SEND0 + MF/2 - 1 go to the partner wave through LDS, lane for lane.
+template <int MF, int SEND0>
+__device__ __forceinline__ void swiglu_send(const f32x4 (&acc)[8][MF], char LLMMM_LDS* region, int lane)
+{
+#pragma unroll
+  for (int nf = 0; nf < 8; ++nf)
+#pragma unroll
+    for (int h = 0; h < MF / 2; ++h) *(f32x4 LLMMM_LDS*)(region + ((h * 8 + nf) * 64 + lane) * 16) = acc[nf][SEND0 + h];
+}
+
+// The kept fragments mf = KEEP0 .. (own values: gate if IS_GATE, else up) meet the partner's values of the same
+// rows and columns: h = silu(gate) * up, then the fused 1x128 quantisation of h exactly as for plain C
+// (examples/005.fp8.mm.opt.cu:401-462), staged row-major in `stg` and stored as whole 128-byte rows.
+template <int MF, int KEEP0, bool IS_GATE>
+__device__ __forceinline__ void swiglu_finish(const f32x4 (&acc)[8][MF], const f32x4 (&other)[8][MF / 2], char LLMMM_LDS* stg, uint8_t* C,
+                                              float* Cs_col, int ldc, int row0, int col0, int lane)
+{
+  constexpr int MH = MF / 2;
+  const int     g = lane >> 4, li = lane & 15;
+#pragma unroll
+  for (int h = 0; h < MH; ++h) {
+    f32x4 v[8];
+    float amax = 0.f;
+#pragma unroll
+    for (int nf = 0; nf < 8; ++nf)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float mine = acc[nf][KEEP0 + h][q], theirs = other[nf][h][q];
+        v[nf][q]         = IS_GATE ? silu_mul(mine, theirs) : silu_mul(theirs, mine);
+        amax             = fmaxf(amax, __builtin_fabsf(v[nf][q]));
+      }
+    amax              = wave_xor_max(amax, 16);
+    amax              = wave_xor_max(amax, 32);
+    const float scale = amax / 448.f;
+    const float inv   = amax > 0.f ? 448.f / amax : 0.f;
+    const int   r     = h * 16 + li;
+#pragma unroll
+    for (int nf = 0; nf < 8; ++nf)
+      *(uint32_t LLMMM_LDS*)(stg + r * 128 + ((nf ^ ((r >> 1) & 7)) << 4) + 4 * g) =
+        pack_e4m3x4_in_range(v[nf][0] * inv, v[nf][1] * inv, v[nf][2] * inv, v[nf][3] * inv);
+    if (g == 0) Cs_col[row0 + KEEP0 * 16 + r] = scale;
+  }
+#pragma unroll
+  for (int j = 0; j < MH * 2; ++j) {
+    const int   r = 8 * j + (lane >> 3), c = lane & 7;
+    const i32x4 x = *(const i32x4 LLMMM_LDS*)(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
+    *(i32x4*)(C + (size_t)(row0 + KEEP0 * 16 + r) * ldc + col0 + c * 16) = x;
+  }
+}
+
 // BMODE bit 0 (BPRE): Bt is the pre-shuffled image of the weights (layout.hip) instead of row-major [N, K].
 // BMODE bit 1 (BNT): the weight loads carry the non-temporal hint (one tile row: every weight byte is read once).
 template <int BM, int BN, int WM, int OUT, int BMODE>
@@ -243,8 +303,13 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const int wn   = wave / TC::WAVES_M;
   int       tm, tn;
   tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
-  const int KB = K >> 7;
+  // SwiGLU output: the tile's two 128-column halves are the gate columns n0 .. n0+127 and the up columns
+  // N/2 + n0 .. of the same 128 output columns, so the weight rows of the upper half start N/2 - 128 rows further on
+  constexpr bool SWIGLU = OUT == OUT_SWIGLU;
+  static_assert(!SWIGLU || BN == 256, "the SwiGLU epilogue pairs the two 128-column halves of a 256-wide tile");
+  const int    m0   = tm * BM, n0 = SWIGLU ? tn * 128 : tn * BN;
+  const size_t b_hi = SWIGLU ? (size_t)((N >> 1) - 128) * K : 0;
+  const int    KB   = K >> 7;
   // split-K: gridDim.y workgroups share a tile, each taking a contiguous run of slices and (the
   // host only splits the fp32 instantiation) writing its partial sums to its own [M, N] plane
   // of C; a second kernel adds the planes in order.  gridDim.y == 1: the whole K range.
@@ -277,7 +342,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   // scales: As[kb*M + m] for the lane's 4 rows, Bs[(n/128)*KB + kb] for the wave's column group
   const int      mrow    = m0 + wm * WM + (lane & 15);
   const unsigned row_off = (unsigned)mrow * 4u;
-  const float*   Bsp     = Bs + (size_t)((n0 >> 7) + wn) * KB + kb0;
+  const float*   Bsp     = Bs + (size_t)((n0 >> 7) + (SWIGLU ? wn * (N >> 8) : wn)) * KB + kb0;
   const float*   Asl     = As + (size_t)kb0 * M;
   unsigned       zero    = 0;
   asm volatile("" : "+v"(zero));  // a VGPR holding 0: the per-lane offset of the wave-uniform Bs load
@@ -286,7 +351,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const unsigned lds0 = (unsigned)(size_t)(char LLMMM_LDS*)lds;
   char LLMMM_LDS* const s0 = (char LLMMM_LDS*)lds;
 
-  fp8_issue_loads<BM, BN, WM, BNT, 0, TC::A_LOADS + TC::B_LOADS>(lds0, Ag, Bg, lane_off, b_lane_off, K, wave);
+  fp8_issue_loads<BM, BN, WM, BNT, 0, TC::A_LOADS + TC::B_LOADS>(lds0, Ag, Bg, lane_off, b_lane_off, K, b_hi, wave);
   fp8_issue_scales<MF>(sa_next, sb_next, Asl, row_off, Bsp, zero);
 
   // One slice: wait for this wave's loads of the slice (all of them were issued at least half a
@@ -307,7 +372,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
     nx.Bg        = Bg + (size_t)((KC) + 1) * B_KSTEP;                                                                               \
     nx.As_slice  = Asl + (size_t)((KC) + 1) * M;                                                                                  \
     nx.Bs_elem   = Bsp + (KC) + 1;                                                                                                \
-    fp8_compute_stage<BM, BN, WM, BNT, LOAD>(CUR, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, b_lane_off, row_off, zero, K, wave, sa_next, \
+    fp8_compute_stage<BM, BN, WM, BNT, LOAD>(CUR, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, b_lane_off, row_off, zero, K, b_hi, wave, sa_next, \
                                     sb_next);                                                                                     \
   }
 
@@ -364,6 +429,32 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
       const i32x4 v = *(const i32x4 LLMMM_LDS*)(stg + r * 256 + ((c ^ (r & 15)) << 4));
       *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 8) = v;
     }
+  }
+  else if constexpr (OUT == OUT_SWIGLU) {
+    // Waves (wm, 0) hold the gate half and waves (wm, 1) the up half of the same WM rows x 128 output columns.
+    // Each sends the partner the 16-row fragments it does not keep (the gate wave keeps the first half of them,
+    // the up wave the second), so that all eight waves share the activation work and each owns whole rows.
+    constexpr int         MH      = MF / 2;
+    char LLMMM_LDS* const xmine   = s0 + wave * (MH * 8192);
+    const int             partner = wm + (1 - wn) * TC::WAVES_M;
+    const char LLMMM_LDS* xtheirs = s0 + partner * (MH * 8192);
+    if (wn == 0)
+      swiglu_send<MF, MH>(acc, xmine, lane);
+    else
+      swiglu_send<MF, 0>(acc, xmine, lane);
+    __syncthreads();
+    f32x4 other[8][MH];
+#pragma unroll
+    for (int nf = 0; nf < 8; ++nf)
+#pragma unroll
+      for (int h = 0; h < MH; ++h) other[nf][h] = *(const f32x4 LLMMM_LDS*)(xtheirs + ((h * 8 + nf) * 64 + lane) * 16);
+    __syncthreads();  // every wave has read its partner's fragments: the regions are free for the output staging
+    uint8_t*  C    = (uint8_t*)Cv;
+    const int half = N >> 1;
+    if (wn == 0)
+      swiglu_finish<MF, 0, true>(acc, other, xmine, C, Cs + (size_t)tn * M, half, row0, n0, lane);
+    else
+      swiglu_finish<MF, MH, false>(acc, other, xmine, C, Cs + (size_t)tn * M, half, row0, n0, lane);
   }
   else {
     uint8_t* C = (uint8_t*)Cv;
@@ -424,6 +515,20 @@ fp8_splitk_reduce_kernel(const float* __restrict__ planes, int S, void* __restri
       for (int u = 0; u < 4; ++u)
         if (s0 + u < S) v += t[u];
     }
+    if constexpr (OUT == OUT_SWIGLU) {
+      // v = the gate columns; the up columns of the same outputs lie N/2 further on.  h = silu(gate) * up.
+      f32x4 up = {0.f, 0.f, 0.f, 0.f};
+      for (int s0 = 0; s0 < S; s0 += 4) {
+        f32x4 t[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) t[u] = __builtin_nontemporal_load((const f32x4*)(src + (N >> 1) + (size_t)min(s0 + u, S - 1) * plane));
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (s0 + u < S) up += t[u];
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = silu_mul(v[q], up[q]);
+    }
     if constexpr (OUT == OUT_F32) {
       *(f32x4*)((float*)Cv + (size_t)m * N + n) = v;
     }
@@ -434,7 +539,8 @@ fp8_splitk_reduce_kernel(const float* __restrict__ planes, int S, void* __restri
       for (int q = 0; q < 4; ++q) o[q] = (__bf16)v[q];
       *(bf16x4*)((__bf16*)Cv + (size_t)m * N + n) = o;
     }
-    else {
+    else {  // e4m3 codes + 1x128 scales, of C or (SwiGLU) of h, whose rows are N/2 wide
+      const int ldc = OUT == OUT_SWIGLU ? (N >> 1) : N;
       float a = fmaxf(fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1])), fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
       a       = wave_xor_max(a, 1);
       a       = wave_xor_max(a, 2);
@@ -443,7 +549,7 @@ fp8_splitk_reduce_kernel(const float* __restrict__ planes, int S, void* __restri
       a       = wave_xor_max(a, 16);
       const float scale = a / 448.f;
       const float inv   = a > 0.f ? 448.f / a : 0.f;
-      *(uint32_t*)((uint8_t*)Cv + (size_t)m * N + n) = pack_e4m3x4(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+      *(uint32_t*)((uint8_t*)Cv + (size_t)m * ldc + n) = pack_e4m3x4(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
       if (l32 == 0) Cs[(size_t)nb * M + m] = scale;
     }
   }
@@ -453,9 +559,10 @@ fp8_splitk_reduce_kernel(const float* __restrict__ planes, int S, void* __restri
 template <int OUT>
 static hipError_t launch_reduce(const float* planes, int S, void* C, float* Cs, int M, int N, hipStream_t stream)
 {
-  int rows_per_wg = 8;
-  while (rows_per_wg < 64 && (long)(N / 128) * ((M + 2 * rows_per_wg - 1) / (2 * rows_per_wg)) >= 2048) rows_per_wg *= 2;
-  hipLaunchKernelGGL((fp8_splitk_reduce_kernel<OUT>), dim3(N / 128, (M + rows_per_wg - 1) / rows_per_wg), dim3(256), 0, stream, planes,
+  const int groups      = OUT == OUT_SWIGLU ? N / 256 : N / 128;  // 128-column groups of the output
+  int       rows_per_wg = 8;
+  while (rows_per_wg < 64 && (long)groups * ((M + 2 * rows_per_wg - 1) / (2 * rows_per_wg)) >= 2048) rows_per_wg *= 2;
+  hipLaunchKernelGGL((fp8_splitk_reduce_kernel<OUT>), dim3(groups, (M + rows_per_wg - 1) / rows_per_wg), dim3(256), 0, stream, planes,
                      S, C, Cs, M, N, rows_per_wg);
   return hipGetLastError();
 }
@@ -478,13 +585,20 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
   typedef Fp8Tile<BM, BN, WM> TC;
   const int tiles_m = M / BM, tiles_n = N / BN;
   const int bmode   = (bpre ? 1 : 0) | (tiles_m == 1 ? 2 : 0);
-  if (S <= 1) {
-    const auto kernel = pick_kernel<BM, BN, WM, OUT>(bmode);
-    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs,
-                       M, N, K, tiles_m, tiles_n);
-    return hipGetLastError();
+  if (S <= 1 && planes == nullptr) {
+    if constexpr (OUT == OUT_SWIGLU && BN != 256) {
+      return hipErrorInvalidValue;  // unsplit SwiGLU needs a 256-wide tile (the host picks one)
+    }
+    else {
+      const auto kernel = pick_kernel<BM, BN, WM, OUT>(bmode);
+      hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs,
+                         M, N, K, tiles_m, tiles_n);
+      return hipGetLastError();
+    }
   }
-  // split-K: S partial planes from the fp32 instantiation, then the ordered sum + epilogue
+  // split-K (or planes != nullptr with S = 1: an epilogue that only the second kernel has): S partial planes from
+  // the fp32 instantiation, then the ordered sum + epilogue
+  if (S < 1) S = 1;
   const auto kernel = pick_kernel<BM, BN, WM, OUT_F32>(bmode);
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, S), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs,
                      (void*)planes, (float*)nullptr, M, N, K, tiles_m, tiles_n);
@@ -515,6 +629,7 @@ hipError_t fp8_gemm_launch(int out_kind, int tile, int b_layout, const void* A, 
     case OUT_F32: return dispatch_fp8<OUT_F32>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
     case OUT_BF16: return dispatch_fp8<OUT_BF16>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
     case OUT_FP8Q: return dispatch_fp8<OUT_FP8Q>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
+    case OUT_SWIGLU: return dispatch_fp8<OUT_SWIGLU>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -525,6 +640,7 @@ hipError_t fp8_splitk_reduce_launch(int out_kind, const float* planes, int S, vo
     case OUT_F32: return launch_reduce<OUT_F32>(planes, S, C, Cs, M, N, stream);
     case OUT_BF16: return launch_reduce<OUT_BF16>(planes, S, C, Cs, M, N, stream);
     case OUT_FP8Q: return launch_reduce<OUT_FP8Q>(planes, S, C, Cs, M, N, stream);
+    case OUT_SWIGLU: return launch_reduce<OUT_SWIGLU>(planes, S, C, Cs, M, N, stream);
     default: return hipErrorInvalidValue;
   }
 }

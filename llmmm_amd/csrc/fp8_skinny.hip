@@ -272,9 +272,10 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   // lane (g, i): row m = mb*16 + i, columns ncol .. ncol+3
   const int ncol = ng * 128 + wave * 16 + 4 * g;
 
-  if (S > 1) {
-    // split-K: this workgroup only stores its plane of partial sums; a second kernel adds the
-    // planes in split order 0..S-1 and runs the epilogue (fixed order, whatever the arrival order)
+  if (partial != nullptr) {
+    // split-K (or an epilogue that lives in the second kernel only, S >= 1): this workgroup only stores its
+    // plane of partial sums; a second kernel adds the planes in split order 0..S-1 and runs the
+    // epilogue (fixed order, whatever the arrival order)
 #pragma unroll
     for (int mb = 0; mb < MBLK; ++mb) {
       const int m = m0 + mb * 16 + i;

@@ -13,9 +13,10 @@ namespace llmmm {
 hipError_t fp16_gemm_launch(int dtype, int b_layout, int tile, const void* A, const void* B, void* C, int M, int N, int K,
                             hipStream_t stream);
 
-// out_kind: 0 = fp32, 1 = bf16, 2 = e4m3 codes + per-1x128 scales.  S > 1 splits K over S
+// out_kind: 0 = fp32, 1 = bf16, 2 = e4m3 codes + per-1x128 scales, 3 = SwiGLU (silu(C[:, :N/2]) * C[:, N/2:]) as codes + scales.  S > 1 splits K over S
 // workgroups per tile (S <= K/128): `planes` then holds S * M * N floats of partial sums, added
-// in split order by a second kernel that also runs the epilogue.
+// in split order by a second kernel that also runs the epilogue.  planes != nullptr with S == 1 takes the
+// same two-kernel route through one plane (the SwiGLU output from a 128-column tile).
 // b_layout: LLMMM_FP8_B_ROWS (Bt[N,K] row-major) or LLMMM_FP8_B_PRESHUFFLED (the image fp8_preshuffle_launch writes).
 hipError_t fp8_gemm_launch(int out_kind, int tile, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs,
                            void* C, float* Cs, int M, int N, int K, int S, float* planes, hipStream_t stream);
@@ -23,8 +24,8 @@ hipError_t fp8_gemm_launch(int out_kind, int tile, int b_layout, const void* A, 
 // C = epilogue(planes[0] + planes[1] + ... + planes[S-1]) (that order), planes of M * N floats each.
 hipError_t fp8_splitk_reduce_launch(int out_kind, const float* planes, int S, void* C, float* Cs, int M, int N, hipStream_t stream);
 
-// M <= 128 (row groups of 64); S splits of K.  S == 1: complete result in C / Cs.  S > 1: only the S
-// partial planes `partial` [S][M][N] fp32 are written; run fp8_splitk_reduce_launch behind it.
+// M <= 128 (row groups of 64); S splits of K.  partial == nullptr (S must be 1): complete result in C / Cs.
+// Otherwise only the S partial planes `partial` [S][M][N] fp32 are written; run fp8_splitk_reduce_launch behind it.
 hipError_t fp8_skinny_launch(int out_kind, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
                              float* Cs, int M, int N, int K, int S, float* partial, hipStream_t stream);
 

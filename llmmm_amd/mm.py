@@ -130,13 +130,14 @@ def query_config(out_kind, M, N, K):
 
 def _fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, workspace, tile, split_k, stream, b_preshuffled=False):
     kb = K // 128 if K % 128 == 0 else 0
-    c_dtypes = {_lib.OUT_F32: (torch.float32,), _lib.OUT_BF16: (torch.bfloat16,), _lib.OUT_FP8Q: _FP8_DTYPES}[out_kind]
+    c_dtypes = {_lib.OUT_F32: (torch.float32,), _lib.OUT_BF16: (torch.bfloat16,), _lib.OUT_FP8Q: _FP8_DTYPES, _lib.OUT_FP8Q_SWIGLU: _FP8_DTYPES}[out_kind]
+    n_out = N // 2 if out_kind == _lib.OUT_FP8Q_SWIGLU else N  # SwiGLU halves the width
     a_p = _ptr(A, "A", _FP8_DTYPES, M * K)
     as_p = _ptr(As, "A_scale_transposed", (torch.float32,), kb * M)
     b_p = _ptr(Bt, "B_transposed", _FP8_DTYPES, N * K)
     bs_p = _ptr(Bs, "B_scale_transposed", (torch.float32,), ((N + 127) // 128) * kb)
-    c_p = _ptr(C, "C", c_dtypes, M * N)
-    cs_p = _ptr(Cs, "C_scale_transposed", (torch.float32,), ((N + 127) // 128) * M) if out_kind == _lib.OUT_FP8Q else None
+    c_p = _ptr(C, "C", c_dtypes, M * n_out)
+    cs_p = _ptr(Cs, "C_scale_transposed", (torch.float32,), ((n_out + 127) // 128) * M) if out_kind in (_lib.OUT_FP8Q, _lib.OUT_FP8Q_SWIGLU) else None
     ws_p, ws_n = (ctypes.c_void_p(workspace.data_ptr()), workspace.numel() * workspace.element_size()) if workspace is not None else (None, 0)
     cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS)
     check(lib.llmmm_fp8_gemm_ex(out_kind, a_p, as_p, b_p, bs_p, c_p, cs_p, M, N, K, ws_p, ws_n, ctypes.byref(cfg), _stream(stream)))
@@ -166,6 +167,17 @@ def fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(A, A_scale_
     C_scale_transposed float32 [N/128, M]."""
     _fp8_gemm(_lib.OUT_FP8Q, A, A_scale_transposed, B_transposed, B_scale_transposed, C, C_scale_transposed, M, N, K, workspace, tile,
               split_k, stream, b_preshuffled)
+
+
+def fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(A, A_scale_transposed, B_transposed, B_scale_transposed, C,
+                                                                             C_scale_transposed, M, N, K, stream=None, workspace=None,
+                                                                             tile=_lib.TILE_AUTO, split_k=0, b_preshuffled=False):
+    """The gate_up projection of a gated MLP with the activation fused in front of the C quantisation (the fusion
+    the reference plans, README.md:16; no reference kernel).  B_transposed [N,K] holds the gate rows in [0, N/2) and
+    the up rows in [N/2, N); C = e4m3 codes of silu(gate) * up [M, N/2], C_scale_transposed float32 [N/256, M].
+    M <= 128 needs a workspace (``make_workspace(OUT_FP8Q_SWIGLU, ...)``)."""
+    _fp8_gemm(_lib.OUT_FP8Q_SWIGLU, A, A_scale_transposed, B_transposed, B_scale_transposed, C, C_scale_transposed, M, N, K, workspace,
+              tile, split_k, stream, b_preshuffled)
 
 
 # ------------------------------------------------------------------------------------- offline layout helpers

@@ -232,6 +232,25 @@ def requant_c_1x128(C, reciprocal=True, zero_guard=True):
     return Cq, Cs
 
 
+def swiglu(C):
+    """h[m, j] = silu(C[m, j]) * C[m, N/2 + j] in fp32, silu(x) = x / (1 + exp(-x)): the gated-MLP activation
+    between the gate_up and down projections (gate columns first, up columns second).  The reference has no such
+    kernel -- fusing SiLU into the GEMM is on its plan (README.md:16) -- so this definition is the build's own;
+    pinned by tests/test_oracle_swiglu.py (known values, the tanh form in float64, limits, gate/up asymmetry)."""
+    C = _f32(C)
+    half = C.shape[1] // 2
+    assert C.shape[1] == 2 * half
+    g, u = C[:, :half], C[:, half:]
+    with np.errstate(over="ignore"):
+        e = np.exp(-g)  # float32
+    return ((g / (np.float32(1.0) + e)) * u).astype(np.float32)
+
+
+def swiglu_requant(C):
+    """(Cq [M, N/2], Cs [N/256, M]): the fused epilogue's 1x128 quantisation applied to swiglu(C)."""
+    return requant_c_1x128(swiglu(C))
+
+
 # ----------------------------------------------------------------------------- offline layouts
 def operand_swizzle_rows16(r):
     """Chunk XOR of row r (0..15) in the 16-row x 128-byte MFMA operand image of the pre-shuffled

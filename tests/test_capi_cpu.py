@@ -169,3 +169,28 @@ def test_layout_helpers_validation_without_device():
     assert lib.llmmm_fp8_gemm_ex(2, *args, 128, 128, 256, None, 0, ctypes.byref(cfg), None) == _lib.ERR_INVALID_ARGUMENT
     q = _lib.GemmCfg(5, 5, 5)
     assert lib.llmmm_fp8_gemm_query(2, 128, 128, 256, ctypes.byref(q)) == _lib.OK and q.b_layout == _lib.FP8_B_ROWS
+
+
+def test_swiglu_validation_without_device():
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    args = (FAKE, FAKE, FAKE, FAKE, FAKE, FAKE)
+    f = lib.llmmm_fp8_gemm
+    assert f(_lib.OUT_FP8Q_SWIGLU, *args, 256, 384, 256, None, 0, None) == _lib.ERR_NOT_ALIGNED   # N % 256 != 0
+    assert f(_lib.OUT_FP8Q_SWIGLU, FAKE, FAKE, FAKE, FAKE, FAKE, None, 256, 512, 256, None, 0, None) == _lib.ERR_INVALID_ARGUMENT  # Cs missing
+    assert f(_lib.OUT_FP8Q_SWIGLU, *args, 16, 512, 256, None, 0, None) == _lib.ERR_WORKSPACE       # small M always needs a plane
+    assert b"workspace" in lib.llmmm_last_error()
+    assert f(4, *args, 256, 512, 256, None, 0, None) == _lib.ERR_INVALID_ARGUMENT
+    # the workspace query covers the plane the small-M path needs, and an unsplit tile run needs none
+    assert lib.llmmm_fp8_gemm_workspace(_lib.OUT_FP8Q_SWIGLU, 16, 19456, 2560) >= 16 * 19456 * 4
+    assert lib.llmmm_fp8_gemm_workspace(_lib.OUT_FP8Q_SWIGLU, 4096, 4096, 4096) == 0
+    # an unsplit SwiGLU run is given a 256-column tile
+    q = _lib.GemmCfg()
+    assert lib.llmmm_fp8_gemm_query(_lib.OUT_FP8Q_SWIGLU, 2048, 2560, 9728, ctypes.byref(q)) == _lib.OK
+    assert q.split_k > 1 or q.tile in (_lib.TILE_256x256, _lib.TILE_128x256)
+    cfg = _lib.GemmCfg(_lib.TILE_128x128, 1, 0)
+    assert lib.llmmm_fp8_gemm_ex(_lib.OUT_FP8Q_SWIGLU, *args, 256, 512, 256, None, 0, ctypes.byref(cfg), None) == _lib.ERR_WORKSPACE
+    # decode-sized M on a wide N: a 128-column tile through one fp32 plane, and the workspace query says so
+    assert lib.llmmm_fp8_gemm_query(_lib.OUT_FP8Q_SWIGLU, 128, 19456, 2560, ctypes.byref(q)) == _lib.OK
+    if q.tile in (_lib.TILE_128x128, _lib.TILE_256x128):
+        assert lib.llmmm_fp8_gemm_workspace(_lib.OUT_FP8Q_SWIGLU, 128, 19456, 2560) >= 128 * 19456 * 4
