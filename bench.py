@@ -31,7 +31,8 @@ PREHEAT_S = 0.25  # seconds of untimed launches before the warm-up steps of ever
 # these same workloads, each scaled by the counter's reading for a 1 GiB device copy (FETCH_SIZE x 2.0 KiB,
 # WRITE_SIZE x 1.0 KiB per count).  Counters cannot be read from inside this process, so the figures are
 # carried here; the summaries they come from are kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"fp16_gemm_4096": 235.0e6, "fp8_gemm_fused_4096": 119.2e6, "decode_gate_up_m1": 50.0e6}
+MEASURED_TRAFFIC_BYTES = {"fp16_gemm_4096": 235.0e6, "fp8_gemm_fused_4096": 119.2e6, "decode_gate_up_m1": 50.0e6,
+                          "decode_gate_up_m1_pre": 50.0e6}
 
 QWEN3_4B = {"qkv": (6144, 2560), "o": (2560, 4096), "gate_up": (19456, 2560), "down": (2560, 9728)}
 
