@@ -113,8 +113,8 @@ LLMMM_API int llmmm_fp8_gemm(int out_kind, const void* A, const float* As, const
 LLMMM_API int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
                                 int M, int N, int K, void* workspace, size_t workspace_bytes, const llmmm_gemm_cfg* cfg,
                                 void* stream);
-/* Bytes of workspace that any configuration the library may pick for this shape needs
- * (0 when the shape never splits K); an explicit split_k = S needs S * M * N * 4 bytes.  No
+/* Bytes of workspace that the configuration the library picks for this shape and output needs
+ * (0 when it neither splits K nor goes through a plane); an explicit split_k = S needs S * M * N * 4 bytes.  No
  * reference counterpart: split-K is "still to do" there (README.md:22). */
 LLMMM_API size_t llmmm_fp8_gemm_workspace(int out_kind, int M, int N, int K);
 /* The configuration llmmm_fp8_gemm would use for this shape (tune table, then heuristic). */

@@ -235,8 +235,7 @@ size_t llmmm_fp8_gemm_workspace(int out_kind, int M, int N, int K)
   if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
   llmmm_gemm_cfg cfg;
   if (choose_fp8_out(out_kind, M, N, K, &cfg) != LLMMM_OK) return 0;
-  // the weight-streaming kernel: room for any split the tuner may try; tile kernels: the split chosen
-  const int  s       = cfg.tile == LLMMM_TILE_SKINNY ? max_split_for(K) : cfg.split_k;
+  const int  s       = cfg.split_k;  // the split the library would pick (an explicit cfg->split_k = S needs S planes)
   const bool narrow  = cfg.tile == LLMMM_TILE_256x128 || cfg.tile == LLMMM_TILE_128x128;
   const bool a_plane = out_kind == LLMMM_OUT_FP8Q_SWIGLU && (cfg.tile == LLMMM_TILE_SKINNY || narrow);  // SwiGLU outside a 256-column tile
   if (s <= 1 && !a_plane) return 0;

@@ -94,16 +94,14 @@ def test_workspace_sizes_and_config_queries():
         for m in (1, 16):
             tile, split = llmmm_amd.query_config(_lib.OUT_FP8Q, m, n, k)
             assert tile == _lib.TILE_SKINNY and 1 <= split <= min(32, k // 128)
-            assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, m, n, k) >= split * m * n * 4
+            assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, m, n, k) == (0 if split == 1 else split * m * n * 4)
         for m in (128, 2048):
             tile, split = llmmm_amd.query_config(_lib.OUT_FP8Q, m, n, k)
             tiles = (_lib.TILE_256x256, _lib.TILE_128x256, _lib.TILE_256x128, _lib.TILE_128x128)
             assert tile in tiles + ((_lib.TILE_SKINNY,) if m == 128 else ())
             if tile in tiles:
                 assert 1 <= split <= 8
-                assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, m, n, k) == (0 if split == 1 else split * m * n * 4)
-            else:
-                assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, m, n, k) >= split * m * n * 4
+            assert llmmm_amd.workspace_bytes(_lib.OUT_FP8Q, m, n, k) == (0 if split == 1 else split * m * n * 4)
     assert llmmm_amd.query_config(_lib.OUT_FP8Q, 4096, 4096, 4096) == (_lib.TILE_256x256, 1)
     with pytest.raises(RuntimeError, match="M or N or K are not aligned."):
         llmmm_amd.query_config(_lib.OUT_FP8Q, 200, 4096, 4096)
