@@ -140,13 +140,22 @@ struct Fp8Next {
   const uint8_t* Bg;
   const float*   As_slice;   // As + kb_next * M
   const float*   Bs_elem;    // &Bs[nb, kb_next]
+  const char*    sc_ptr;     // deep pipeline only: this lane's scale of the slice being requested (see fp8_scale_load_lds)
 };
+
+// Deep pipeline: the slice scales travel with the stage.  One 4-byte LDS-direct load per wave and slice: lanes
+// 0 .. WM-1 fetch As[kb, row] of the wave's rows, the other lanes all fetch Bs[nb, kb]; lane l's value lands at
+// lds_addr + 4*l, so the wave later reads its row scales at 4*(16*mf + i) and the column-group scale at 128.
+__device__ __forceinline__ void fp8_scale_load_lds(const char* lane_ptr, unsigned lds_addr)
+{
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(lane_ptr), "s"(lds_addr) : "memory");
+}
 
 // One 128-K slice of the wave's WM x 128 sub-tile.  s[mf] = As[kb, row] * Bs[nb, kb].
 // With LOAD, the next stage's loads go out two or more per fragment step during the first four
 // steps (spread, so that no wave sits in the memory pipeline's issue queue while its matrix
 // work waits, and early enough to land within the slice), its scales during the fifth.
-template <int BM, int BN, int WM, bool BNT, bool LOAD>
+template <int BM, int BN, int WM, bool BNT, bool LOAD, bool SCALE_LDS = false>
 __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int a_rd0, int a_rd1, int b_rd0, int b_rd1,
                                                   const float (&s)[WM / 16], f32x4 (&acc)[8][WM / 16], const Fp8Next& nx, unsigned lane_off,
                                                   unsigned b_lane_off, unsigned row_off, unsigned zero, int K, size_t b_hi, int wave, float (&sa_next)[WM / 16],
@@ -172,7 +181,12 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int
       if (nf == 1) fp8_issue_loads<BM, BN, WM, BNT, LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
       if (nf == 2) fp8_issue_loads<BM, BN, WM, BNT, 2 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
       if (nf == 3) fp8_issue_loads<BM, BN, WM, BNT, 3 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
-      if (nf == 4) fp8_issue_scales<MF>(sa_next, sb_next, nx.As_slice, row_off, nx.Bs_elem, zero);
+      if (nf == 4) {
+        if constexpr (SCALE_LDS)
+          fp8_scale_load_lds(nx.sc_ptr, nx.lds_stage + TC::STAGE + wave * 256);
+        else
+          fp8_issue_scales<MF>(sa_next, sb_next, nx.As_slice, row_off, nx.Bs_elem, zero);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -294,7 +308,13 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   typedef Fp8Tile<BM, BN, WM> TC;
   constexpr int  MF   = TC::MF;
   constexpr bool BPRE = (BMODE & 1) != 0, BNT = (BMODE & 2) != 0;
-  __shared__ __attribute__((aligned(1024))) char lds[2 * TC::STAGE];
+  // Weights that are streamed once (a single tile row: decode-sized M) leave the workgroups waiting on memory
+  // latency, not on the matrix pipe, and there is at most one workgroup per CU: the 32-row-wave tiles then run a
+  // deeper pipeline -- as many stages as fit the LDS instead of two, the slice scales travelling with the stage.
+  constexpr bool DEEP    = BNT && WM == 32;
+  constexpr int  STAGE_D = TC::STAGE + TC::NW * 256;                 // operands + 256 bytes of scales per wave
+  constexpr int  NST     = !DEEP ? 2 : (4 * STAGE_D <= 160 * 1024 ? 4 : 3);
+  __shared__ __attribute__((aligned(1024))) char lds[DEEP ? NST * STAGE_D : 2 * TC::STAGE];
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -351,6 +371,57 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const unsigned lds0 = (unsigned)(size_t)(char LLMMM_LDS*)lds;
   char LLMMM_LDS* const s0 = (char LLMMM_LDS*)lds;
 
+  if constexpr (DEEP) {
+    constexpr int PER = TC::A_LOADS + TC::B_LOADS + 1;  // vector-memory loads of a wave per slice
+    static_assert((NST - 2) * PER < 64, "vmcnt is a 6-bit counter");
+    // this lane's scale source: a row scale (stride M floats per slice) or the column-group scale (stride 1)
+    const bool     row_lane = lane < WM;
+    const char*    sc_ptr   = row_lane ? (const char*)(Asl + (m0 + wm * WM + lane)) : (const char*)Bsp;
+    const unsigned sc_step  = row_lane ? (unsigned)M * 4u : 4u;
+    // prologue: slices 0 .. NST-2 (a K range shorter than that repeats its last slice into the spare stages)
+#pragma unroll
+    for (int u = 0; u < NST - 1; ++u) {
+      const int kk = min(u, KBL - 1);
+      fp8_issue_loads<BM, BN, WM, BNT, 0, TC::A_LOADS + TC::B_LOADS>(lds0 + u * STAGE_D, Ag + (size_t)kk * 128, Bg + (size_t)kk * B_KSTEP, lane_off,
+                                                                     b_lane_off, K, b_hi, wave);
+      fp8_scale_load_lds(sc_ptr + (size_t)kk * sc_step, lds0 + u * STAGE_D + TC::STAGE + wave * 256);
+    }
+    const char* sc_next = sc_ptr + (size_t)(NST - 1) * sc_step;
+    unsigned    cur     = 0;  // byte offset of the stage being computed
+    const float LLMMM_LDS* const my_scales = (const float LLMMM_LDS*)(s0 + TC::STAGE + wave * 256);
+#define LLMMM_FP8_DEEP_SLICE(LOAD, WAIT)                                                                                          \
+  {                                                                                                                               \
+    wait_vmcnt<(WAIT)>();                                                                                                         \
+    __syncthreads();                                                                                                              \
+    const float LLMMM_LDS* sc_ = (const float LLMMM_LDS*)((const char LLMMM_LDS*)my_scales + cur);                                \
+    float                  s[MF];                                                                                                 \
+    const float            sb_ = sc_[32];                                                                                         \
+    _Pragma("unroll") for (int mf = 0; mf < MF; ++mf) s[mf] = sc_[mf * 16 + (lane & 15)] * sb_;                                    \
+    Fp8Next nx;                                                                                                                   \
+    nx.lds_stage = lds0 + (cur == 0 ? (NST - 1) * STAGE_D : cur - STAGE_D);                                                       \
+    nx.Ag        = Ag + (size_t)(kc + NST - 1) * 128;                                                                             \
+    nx.Bg        = Bg + (size_t)(kc + NST - 1) * B_KSTEP;                                                                         \
+    nx.As_slice  = nullptr;                                                                                                       \
+    nx.Bs_elem   = nullptr;                                                                                                       \
+    nx.sc_ptr    = sc_next;                                                                                                       \
+    fp8_compute_stage<BM, BN, WM, BNT, LOAD, true>(s0 + cur, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, b_lane_off, row_off, zero, K, b_hi, \
+                                                   wave, sa_next, sb_next);                                                       \
+    cur = cur + STAGE_D == NST * STAGE_D ? 0 : cur + STAGE_D;                                                                     \
+  }
+    int kc = 0;
+    for (; kc + (NST - 1) < KBL; ++kc) {  // slices that still have a slice NST-1 ahead of them to request
+      LLMMM_FP8_DEEP_SLICE(true, (NST - 2) * PER)
+      sc_next += sc_step;
+    }
+    // the last (up to) NST-1 slices request nothing more: the waits count down
+    if (kc < KBL) { LLMMM_FP8_DEEP_SLICE(false, (NST - 2) * PER) ++kc; }
+    if (kc < KBL) { LLMMM_FP8_DEEP_SLICE(false, (NST - 3) * PER) ++kc; }
+    if constexpr (NST == 4)
+      if (kc < KBL) { LLMMM_FP8_DEEP_SLICE(false, 0) ++kc; }
+#undef LLMMM_FP8_DEEP_SLICE
+    wait_vmcnt<0>();  // repeats of the last slice that a short K range left in flight
+  }
+  else {
   fp8_issue_loads<BM, BN, WM, BNT, 0, TC::A_LOADS + TC::B_LOADS>(lds0, Ag, Bg, lane_off, b_lane_off, K, b_hi, wave);
   fp8_issue_scales<MF>(sa_next, sb_next, Asl, row_off, Bsp, zero);
 
@@ -383,6 +454,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   }
   LLMMM_FP8_SLICE(false, s0 + cur, 0u, KBL - 1)
 #undef LLMMM_FP8_SLICE
+  }
 
   // ---- epilogue.  lane (g, i): row m = .. + mf*16 + i, columns n = nf*16 + 4g + r.
   // Written straight from this layout, one store instruction would touch 16 rows with 16..64

@@ -83,6 +83,18 @@ def test_short_k(lib, oracle, K):
     _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, tile=TILES["256x256"]), ref, "K=%d" % K)
 
 
+@pytest.mark.parametrize("K", [128, 256, 384, 512, 640, 1152])
+@pytest.mark.parametrize("tile,M", [("128x128", 128), ("128x256", 128), ("256x128", 256)])
+def test_short_k_single_tile_row(lib, oracle, tile, M, K):
+    """One tile row (M = BM): the 32-row-wave tiles stream the weights through their deep pipeline (3 or 4 stages);
+    1 to 9 slices cover a K range shorter than the pipeline, equal to it, and longer."""
+    N = 512
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=60 + K)
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, tile=TILES[tile]), ref, "tile %s M=%d K=%d" % (tile, M, K))
+    _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, tile=TILES[tile], split_k=2 if K >= 256 else 1), ref, "tile %s M=%d K=%d split" % (tile, M, K))
+
+
 def test_single_slice(lib, oracle):
     Aq, As, Bq, Bs = fp8_inputs(oracle, 128, 128, 128, seed=11)
     _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs), oracle.fp8_gemm(Aq, As, Bq, Bs), "K=128")
