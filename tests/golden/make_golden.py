@@ -48,6 +48,23 @@ def main():
     C5q, C5s = oracle.requant_c_1x128(C5)
     np.savez_compressed(os.path.join(HERE, "fp8_gemm_128x256x256.npz"), aq=Aq, a_scale_t=As, bq_t=Bq, b_scale=Bs, c_f32=C,
                         c_bf16=oracle.f32_to_bf16_bits(C), cq=Cq, c_scale_t=Cs, a5q=A5q, a5_scale_t=A5s, c5_f32=C5, c5q=C5q, c5_scale_t=C5s)
+    # offline layouts: the pre-shuffled image of a 48 x 384 weight block and a 128 x 256 byte transpose
+    bt = rng.integers(0, 256, (48, 384), dtype=np.uint8)
+    t_in = rng.integers(0, 256, (128, 256), dtype=np.uint8)
+    np.savez_compressed(os.path.join(HERE, "layout_48x384.npz"), bt=bt, bp=oracle.preshuffle_b(bt), t_in=t_in,
+                        t_out=oracle.transpose_aligned_128(t_in))
+    # SwiGLU output of a gate_up-like GEMM 128 x 512 x 256 (256 gate + 256 up columns; the gate scales are raised so
+    # that silu leaves its linear range)
+    Xs = rng.normal(0, 1, (128, 256)).astype(np.float32)
+    Xs[:, [3, 131]] *= 20
+    Ws = rng.normal(0, 0.02, (512, 256)).astype(np.float32)
+    Sq, Ss = oracle.quant_fp8(Xs, 1, True)
+    Wq, Wsc = oracle.quant_fp8(Ws, 128, False)
+    Wsc[:2] *= np.float32(40.0)
+    Cg = oracle.fp8_gemm(Sq, Ss, Wq, Wsc, promote=128)
+    Hq, Hs = oracle.swiglu_requant(Cg)
+    np.savez_compressed(os.path.join(HERE, "swiglu_128x512x256.npz"), aq=Sq, a_scale_t=Ss, bq_t=Wq, b_scale=Wsc, c_f32=Cg, h_f32=oracle.swiglu(Cg),
+                        hq=Hq, h_scale_t=Hs)
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

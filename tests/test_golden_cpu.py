@@ -37,3 +37,30 @@ def test_fp8_fixture(oracle):
     A = oracle.dequant_fp8(d["aq"], d["a_scale_t"], 1, True).astype(np.float64)
     W = oracle.dequant_fp8(d["bq_t"], d["b_scale"], 128, False).astype(np.float64)
     assert np.abs(C - A @ W.T).max() <= 1e-5 * np.abs(C).max()
+
+
+def test_layout_fixture(oracle):
+    d = np.load(os.path.join(G, "layout_48x384.npz"))
+    assert np.array_equal(oracle.preshuffle_b(d["bt"]), d["bp"]) and np.array_equal(oracle.unshuffle_b(d["bp"]), d["bt"])
+    assert np.array_equal(d["t_out"], d["t_in"].T)
+    # spot value fixed by the layout's definition: row 17 (= row 1 of row group 1), chunk 5 of slice 2 sits in block
+    # (1, 2) at row 1's line, chunk 5 ^ swz(1) = 5 ^ 0
+    blk = d["bp"].reshape(-1)[(1 * 3 + 2) * 2048:(1 * 3 + 2 + 1) * 2048]
+    assert np.array_equal(blk[1 * 128 + 5 * 16:1 * 128 + 6 * 16], d["bt"][17, 2 * 128 + 5 * 16:2 * 128 + 6 * 16])
+
+
+def test_swiglu_fixture(oracle):
+    d = np.load(os.path.join(G, "swiglu_128x512x256.npz"))
+    C = oracle.fp8_gemm(d["aq"], d["a_scale_t"], d["bq_t"], d["b_scale"], promote=128)
+    assert (C == d["c_f32"]).all()
+    h = oracle.swiglu(C)
+    # exp may differ by an ulp between numpy builds / CPUs: hold the stored activation to 2 ulp, not to the bit
+    assert np.all(np.abs(h - d["h_f32"]) <= 2.4e-7 * np.abs(d["h_f32"]) + 1e-38)
+    assert np.abs(C[:, :256]).max() > 2.0, "the fixture does not leave silu's linear range"
+    hq, hs = oracle.swiglu_requant(C)
+    step = np.abs(oracle.e4m3_code_index(hq) - oracle.e4m3_code_index(d["hq"]))
+    assert (step <= 1).all() and (step == 0).mean() >= 0.9999
+    assert np.all(np.abs(hs - d["h_scale_t"]) <= 1e-6 * np.abs(d["h_scale_t"]))
+    # closed-form cross-check of the stored activation: float64, tanh form
+    g, u = C[:, :256].astype(np.float64), C[:, 256:].astype(np.float64)
+    assert np.all(np.abs(d["h_f32"] - g * 0.5 * (1 + np.tanh(g / 2)) * u) <= 4e-7 * np.abs(g * u) + 1e-37)

@@ -117,3 +117,16 @@ def test_decode_shape_pre_shuffled_against_oracle(lib, oracle):
     torch.cuda.synchronize()
     rq, rs = oracle.requant_c_1x128(oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128))
     assert_fused_close(oracle, Cq.cpu().numpy(), Cs.cpu().numpy(), rq, rs, "gate_up M=16 pre-shuffled")
+
+
+def test_golden_fixture(lib):
+    import os
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "layout_48x384.npz"))
+    bt = torch.from_numpy(d["bt"]).cuda()
+    bp = torch.empty_like(bt)
+    lib.construct_mfma_B_layout(bp, bt, 48, 384)
+    t_in = torch.from_numpy(d["t_in"]).cuda()
+    t_out = torch.empty((256, 128), dtype=torch.uint8, device="cuda")
+    lib.transpose_matrix__aligned_128(t_out, t_in, 128, 256)
+    torch.cuda.synchronize()
+    assert np.array_equal(bp.cpu().numpy(), d["bp"]) and np.array_equal(t_out.cpu().numpy(), d["t_out"])

@@ -126,3 +126,12 @@ def test_full_size_properties(lib):
     assert (Hs > 0).all()
     assert torch.equal(Hq, Hq2) and torch.equal(Hs, Hs2)
     assert torch.equal(Hq[perm], Hq3) and torch.equal(Hs[:, perm], Hs3)
+
+
+def test_golden_fixture(lib, oracle):
+    import os
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "swiglu_128x512x256.npz"))
+    t = _gpu(d["aq"], d["a_scale_t"], d["bq_t"], d["b_scale"])
+    for tile in ("128x256", "128x128", "skinny"):
+        Hq, Hs, C32 = _run(lib, t, 128, 512, 256, TILES[tile], 1)
+        assert_fused_close(oracle, Hq, Hs, d["hq"], d["h_scale_t"], "golden swiglu " + tile)
