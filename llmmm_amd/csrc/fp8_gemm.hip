@@ -558,6 +558,31 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   }
 }
 
+// Sum of S planes at one position, added in plane order 0 .. S-1.  W planes are in flight at a time; positions
+// beyond S repeat the last plane and are not added.
+template <int W>
+__device__ __forceinline__ void reduce_planes_chunk(f32x4& v, const float* src, int s0, int S, size_t plane)
+{
+  f32x4 t[W];
+#pragma unroll
+  for (int u = 0; u < W; ++u) t[u] = __builtin_nontemporal_load((const f32x4*)(src + (size_t)min(s0 + u, S - 1) * plane));
+#pragma unroll
+  for (int u = 0; u < W; ++u)
+    if (s0 + u < S) v += t[u];
+}
+// One memory round trip for up to 16 planes (the split counts in use are 2 .. 10).
+__device__ __forceinline__ f32x4 reduce_planes(const float* src, int S, size_t plane)
+{
+  f32x4 v = {0.f, 0.f, 0.f, 0.f};
+  if (S <= 4)
+    reduce_planes_chunk<4>(v, src, 0, S, plane);
+  else if (S <= 8)
+    reduce_planes_chunk<8>(v, src, 0, S, plane);
+  else
+    for (int s0 = 0; s0 < S; s0 += 16) reduce_planes_chunk<16>(v, src, s0, S, plane);
+  return v;
+}
+
 // Second kernel of a split-K run: C = epilogue(sum over s = 0..S-1, in that order, of plane s).
 // Half a wavefront (32 lanes x 4 columns) owns one row of one 128-column group, which is also
 // one quantisation group of the fused output; a workgroup of 256 threads covers 8 rows per step.
@@ -578,26 +603,10 @@ fp8_splitk_reduce_kernel(const float* __restrict__ planes, int S, void* __restri
   const size_t plane = (size_t)M * N;
   for (int m = mbeg + sub; m < mend; m += 8) {
     const float* src = planes + (size_t)m * N + n;
-    f32x4        v   = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < S; s0 += 4) {  // four planes in flight, added in order
-      f32x4 t[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) t[u] = __builtin_nontemporal_load((const f32x4*)(src + (size_t)min(s0 + u, S - 1) * plane));
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-        if (s0 + u < S) v += t[u];
-    }
+    f32x4        v   = reduce_planes(src, S, plane);
     if constexpr (OUT == OUT_SWIGLU) {
       // v = the gate columns; the up columns of the same outputs lie N/2 further on.  h = silu(gate) * up.
-      f32x4 up = {0.f, 0.f, 0.f, 0.f};
-      for (int s0 = 0; s0 < S; s0 += 4) {
-        f32x4 t[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) t[u] = __builtin_nontemporal_load((const f32x4*)(src + (N >> 1) + (size_t)min(s0 + u, S - 1) * plane));
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-          if (s0 + u < S) up += t[u];
-      }
+      const f32x4 up = reduce_planes(src + (N >> 1), S, plane);
 #pragma unroll
       for (int q = 0; q < 4; ++q) v[q] = silu_mul(v[q], up[q]);
     }
