@@ -1,5 +1,5 @@
-// FP8 (OCP e4m3) blockwise-scaled GEMM for gfx950 with fp32 / bf16 output or the fused
-// per-1x128 re-quantisation of C.
+// FP8 (OCP e4m3) blockwise-scaled GEMM for gfx950 with fp32 / bf16 output, the fused per-1x128
+// re-quantisation of C, or the same re-quantisation of silu(gate) * up (SwiGLU) for a gate_up projection.
 //
 //   C[m,n] = sum_kb ( sum_{k in 128-slice kb} Aq[m,k] * Bq[n,k] ) * As[kb,m] * Bs[n/128,kb]
 //
@@ -18,8 +18,11 @@
 //    row operand and A the column operand, so a lane owns one row m and its scale is a single
 //    register per 16-row fragment;
 //  * one stage = one slice: a BM x 128 B tile of A and a BN x 128 B tile of Bt, both K-major,
-//    land in LDS by LDS-direct loads (two stages in flight) and are read with ds_read_b128
-//    through the SWZ_ROWS16 placement;
+//    land in LDS by LDS-direct loads (two stages in flight; three or four with the slice scales in the
+//    stage when a single tile row streams the weights) and are read with ds_read_b128 through the
+//    SWZ_ROWS16 placement; the weights may also arrive pre-shuffled into that placement (layout.hip);
+//  * split-K: gridDim.y workgroups per tile write fp32 planes, and a second kernel adds them in split
+//    order and runs the epilogue (fixed order: results do not depend on timing);
 //  * fused epilogue (examples/005.fp8.mm.opt.cu:401-462): a wavefront owns 64 rows x one whole
 //    128-column quantisation group, so the row amax needs the lane's 32 values and two
 //    cross-lane steps; scale = amax/448, codes = e4m3(C * (448/amax)), saturating.
