@@ -297,6 +297,22 @@ def main():
                 e.update({"hbm_gbs": x["gbs"], "frac_of_hbm_peak": x["gbs"] / PEAK_HBM_GBS, "weight_copies": x["weight_copies"]})
             shapes.append(e)
             torch.cuda.empty_cache()
+        # RMSNorm fused in front of the activation quantiser, bf16 hidden states of the Qwen3-4B width (HBM-bound: 3 B per element)
+        for m in (16, 2048, 16384):
+            xh = torch.randn((m, 2560), device="cuda", dtype=torch.bfloat16)
+            wn = torch.ones(2560, device="cuda")
+            qh = torch.empty((m, 2560), device="cuda", dtype=torch.uint8)
+            sh = torch.empty((20, m), device="cuda", dtype=torch.float32)
+
+            def norm_step():
+                rc = llmmm_amd._lib.lib.llmmm_rmsnorm_quant_fp8(llmmm_amd._lib.DTYPE_BF16, xh.data_ptr(), wn.data_ptr(), 1e-6, qh.data_ptr(),
+                                                                sh.data_ptr(), m, 2560, torch.cuda.current_stream().cuda_stream)
+                assert rc == 0
+
+            ms_, _ = _events_ms(norm_step, s2, w2, graph=True)
+            nb = m * 2560 * 3.0 + m * 20 * 4.0
+            shapes.append({"name": "rmsnorm_quant_bf16_m%d_k2560" % m, "M": m, "K": 2560, "us": ms_ * 1e3, "hbm_gbs": nb / ms_ * 1e-6,
+                           "frac_of_hbm_peak": nb / ms_ * 1e-6 / PEAK_HBM_GBS})
         line["shapes"] = shapes
 
     if not args.no_cpu:

@@ -39,6 +39,7 @@ extern "C" {
 /* ---- enums ----------------------------------------------------------------------------- */
 #define LLMMM_DTYPE_F16 0  /* half            src/mm/fp16/mm.cu:44 */
 #define LLMMM_DTYPE_BF16 1 /* __nv_bfloat16   src/mm/fp16/mm.cu:45-46 */
+#define LLMMM_DTYPE_F32 2  /* float: input type of the quantisers only */
 
 #define LLMMM_B_ROW_MAJOR 0  /* B[K,N], the reference layout (src/mm/fp16/mm.cuh:103) */
 #define LLMMM_B_TRANSPOSED 1 /* Bt[N,K]; an extension, same arithmetic */
@@ -126,6 +127,15 @@ LLMMM_API int llmmm_fp8_gemm_query(int out_kind, int M, int N, int K, llmmm_gemm
  *                float* scale, int M, int N, cudaStream_t)             examples/005.fp8.mm.cu:547-563.
  * x [M,N] fp32 -> q [M,N] e4m3 + scales (layout per `kind`).  Any M; N % 4 == 0. */
 LLMMM_API int llmmm_quant_fp8(int kind, const float* x, void* q, float* scale, int M, int N, void* stream);
+
+/* RMSNorm fused in front of the activation quantiser -- the "RMSNorm + fp8 dynamic quant" fusion the reference plans
+ * (README.md:16); it has no kernel for it.  x [M,K] (in_dtype: LLMMM_DTYPE_F32, _BF16 or _F16), weight [K] fp32:
+ *   y = x / sqrt(mean_k(x^2) + eps) * weight   (fp32),   then   q, scale = 1x128 quantisation of y as by
+ * llmmm_quant_fp8(LLMMM_QUANT_1x128_T): q [M,K] e4m3, scale [(k/128)*M + m] -- the A / A_scale_transposed pair of
+ * llmmm_fp8_gemm.  K % 128 == 0; x, weight and q 16-byte aligned.  The sum of squares is taken in a fixed order
+ * (documented at the kernel), so results are reproducible bit for bit. */
+LLMMM_API int llmmm_rmsnorm_quant_fp8(int in_dtype, const void* x, const float* weight, float eps, void* q, float* scale, int M, int K,
+                                      void* stream);
 
 /* ---- offline layout helpers --------------------------------------------------------------
  * llmmm_fp8_preshuffle_b takes the role of  construct_m16n8k32_B_layout(dst, src_transposed, N, K,

@@ -16,8 +16,10 @@
 // without split-K here because the reference signature has no workspace -- use llmmm_fp8_gemm()
 // with a workspace for the split-K path.
 #pragma once
+#include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 #include <stdexcept>
+#include <type_traits>
 #include <string>
 
 #include "../../../llmmm.h"
@@ -72,6 +74,18 @@ inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(con
 {
   detail8::throw_on_error(llmmm_fp8_gemm(LLMMM_OUT_FP8Q, A, A_scale_transposed, B_transposed, B_scale_transposed, C, C_scale_transposed, M,
                                          N, K, nullptr, 0, (void*)stream));
+}
+
+// RMSNorm fused in front of the 1x128 activation quantiser (planned by the reference, README.md:16; no reference
+// kernel): q, scale = quantise<1,128,true>(x / sqrt(mean(x^2) + eps) * weight).  T = float, __half/_Float16 or a
+// 2-byte bfloat16 type; weight is fp32.
+template <typename T>
+void rmsnorm_fp8_blockwise_symmetric_quantization(const T* x, const float* weight, float eps, fp8_t* q, float* scale, int M, int K,
+                                                  hipStream_t stream)
+{
+  constexpr int dtype = sizeof(T) == 4 ? LLMMM_DTYPE_F32 : (std::is_same<T, _Float16>::value || std::is_same<T, __half>::value) ? LLMMM_DTYPE_F16 : LLMMM_DTYPE_BF16;
+  static_assert(sizeof(T) == 4 || sizeof(T) == 2, "T must be float, half or bfloat16");
+  detail8::throw_on_error(llmmm_rmsnorm_quant_fp8(dtype, x, weight, eps, q, scale, M, K, (void*)stream));
 }
 
 // The gate_up projection of a gated MLP with silu(gate) * up fused in front of the C quantisation -- the

@@ -19,6 +19,7 @@ from .mm import (  # noqa: F401
     quantize_weight,
     query_config,
     restore_B_layout,
+    rmsnorm_quantize_activation,
     transpose_matrix__aligned_128,
     workspace_bytes,
 )

@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libllmmm.so")
 
 OK, ERR_NOT_ALIGNED, ERR_UNSUPPORTED_TYPE, ERR_INVALID_ARGUMENT, ERR_WORKSPACE, ERR_RUNTIME = range(6)
-DTYPE_F16, DTYPE_BF16 = 0, 1
+DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
 B_ROW_MAJOR, B_TRANSPOSED = 0, 1
 OUT_F32, OUT_BF16, OUT_FP8Q, OUT_FP8Q_SWIGLU = 0, 1, 2, 3
 QUANT_1x128_T, QUANT_128x128, QUANT_1x128, QUANT_128x128_T = 0, 1, 2, 3
@@ -38,6 +38,7 @@ SIGNATURES = {
     "llmmm_fp8_gemm_workspace": (_sz, [_i, _i, _i, _i]),
     "llmmm_fp8_gemm_query": (_i, [_i, _i, _i, _i, _c.POINTER(GemmCfg)]),
     "llmmm_quant_fp8": (_i, [_i, _fp, _vp, _fp, _i, _i, _vp]),
+    "llmmm_rmsnorm_quant_fp8": (_i, [_i, _vp, _fp, _c.c_float, _vp, _fp, _i, _i, _vp]),
     "llmmm_fp8_preshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
     "llmmm_fp8_unshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
     "llmmm_transpose": (_i, [_i, _vp, _vp, _i, _i, _vp]),

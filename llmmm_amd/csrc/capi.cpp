@@ -341,6 +341,20 @@ int llmmm_quant_fp8(int kind, const float* x, void* q, float* scale, int M, int 
   return LLMMM_OK;
 }
 
+int llmmm_rmsnorm_quant_fp8(int in_dtype, const void* x, const float* weight, float eps, void* q, float* scale, int M, int K, void* stream)
+{
+  if (in_dtype != LLMMM_DTYPE_F16 && in_dtype != LLMMM_DTYPE_BF16 && in_dtype != LLMMM_DTYPE_F32) return fail(LLMMM_ERR_UNSUPPORTED_TYPE, "T is not supported.");
+  if (M <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "M and K must be positive (got %d, %d)", M, K);
+  if (K % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+  if (!x || !weight || !q || !scale) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (!(eps >= 0.f)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "eps must be non-negative");
+  if (!aligned16(x) || !aligned16(weight) || !aligned16(q)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+  if ((long)M * K >= (1L << 31)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
+  const hipError_t e = llmmm::rmsnorm_quant_launch(in_dtype, x, weight, eps, q, scale, M, K, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "rmsnorm + quantiser launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
 static int preshuffle(int inverse, const void* src, void* dst, int N, int K, void* stream)
 {
   if (N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "N and K must be positive (got %d, %d)", N, K);

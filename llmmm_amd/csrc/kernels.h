@@ -37,6 +37,10 @@ hipError_t transpose_launch(int elem_size, const void* src, void* dst, int M, in
 
 hipError_t quant_fp8_launch(int quant_m, int transpose, const float* x, void* q, float* scale, int M, int N, hipStream_t stream);
 
+// RMSNorm + 1x128 quantisation with transposed scales; x [M,K] of in_dtype (LLMMM_DTYPE_*), w [K] fp32, K % 128 == 0.
+hipError_t rmsnorm_quant_launch(int in_dtype, const void* x, const float* w, float eps, void* q, float* scale, int M, int K,
+                                hipStream_t stream);
+
 hipError_t fill_u32_launch(uint32_t* p, uint32_t value, size_t n, hipStream_t stream);
 
 }  // namespace llmmm

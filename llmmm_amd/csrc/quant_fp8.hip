@@ -116,6 +116,139 @@ __global__ void __launch_bounds__(256) quant_128x128_kernel(const float* __restr
   }
 }
 
+// RMSNorm fused in front of the 1 x 128 activation quantiser (the "RMSNorm + fp8 dynamic quant" fusion the reference
+// plans, README.md:16; no reference kernel):
+//   y[m,k] = (x[m,k] * r) * w[k],  r = 1 / sqrt(sum_k x[m,k]^2 / K + eps),  then q, s = quant_1x128(y), scales transposed.
+// One wavefront per row.  The row is cut into chunks of four elements; lane l owns chunks l, l+64, ...: a first pass
+// accumulates the squares (one fused multiply-add per element, chunks in ascending order, then the xor butterfly
+// 32, 16, .. 1 over the lanes -- this fixed order is what the CPU oracle restates, so the results are bit-exact), a
+// second pass normalises and quantises: a 128-column group is the 32 consecutive chunks of half a wavefront, so its
+// amax needs five cross-lane steps.  HBM traffic: x once, q once.
+template <typename IN_T>
+__device__ __forceinline__ f32x4 load_row4(const IN_T* p);
+template <>
+__device__ __forceinline__ f32x4 load_row4<float>(const float* p)
+{
+  return *(const f32x4*)p;
+}
+template <>
+__device__ __forceinline__ f32x4 load_row4<__bf16>(const __bf16* p)
+{
+  typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+  const bf16x4   v = *(const bf16x4*)p;
+  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+template <>
+__device__ __forceinline__ f32x4 load_row4<_Float16>(const _Float16* p)
+{
+  const f16x4 v = *(const f16x4*)p;
+  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+
+// One chunk (4 elements) per lane of row m: normalise, take the amax of the 128-column group (the 32 chunks of this
+// half of the wavefront), quantise, store codes and the group's scale.
+__device__ __forceinline__ void rmsnorm_quant_chunk(f32x4 v, float r, const float* __restrict__ w, uint8_t* __restrict__ q,
+                                                    float* __restrict__ scale, int m, int M, int K, int c, int chunks, int lane)
+{
+  const bool live = c < chunks;
+  f32x4      y    = {0.f, 0.f, 0.f, 0.f};
+  if (live) {
+    const f32x4 wv = *(const f32x4*)(w + 4 * c);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) y[e] = (v[e] * r) * wv[e];
+  }
+  float a = amax4(0.f, y);
+  a       = wave_xor_max(a, 1);
+  a       = wave_xor_max(a, 2);
+  a       = wave_xor_max(a, 4);
+  a       = wave_xor_max(a, 8);
+  a       = wave_xor_max(a, 16);
+  const float s  = a / 448.f;
+  uint32_t    cd = 0;
+  if (s != 0.f) cd = q_pack_e4m3x4(y[0] / s, y[1] / s, y[2] / s, y[3] / s);
+  if (live) {
+    *(uint32_t*)(q + (size_t)m * K + 4 * c) = cd;
+    if ((lane & 31) == 0) scale[(size_t)(c >> 5) * M + m] = s;
+  }
+}
+
+// NJ > 0: the row has at most 64 * NJ chunks and stays in registers between the two passes (all its loads in flight
+// at once, the row read once).  NJ == 0: any K, the row is read twice (the second time from the L2).
+template <typename IN_T, int NJ>
+__global__ void __launch_bounds__(256) rmsnorm_quant_1x128_kernel(const IN_T* __restrict__ x, const float* __restrict__ w, float eps,
+                                                                  uint8_t* __restrict__ q, float* __restrict__ scale, int M, int K)
+{
+  const int lane = threadIdx.x & 63;
+  const int m    = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (m >= M) return;  // whole wavefronts leave: no barrier below
+  const IN_T* xr     = x + (size_t)m * K;
+  const int   chunks = K >> 2;
+  float       acc    = 0.f;
+  f32x4       held[NJ > 0 ? NJ : 1];
+  if constexpr (NJ > 0) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int c = lane + 64 * j;
+      held[j]     = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (c < chunks) held[j] = load_row4<IN_T>(xr + 4 * c);
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+      if (lane + 64 * j < chunks) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_fmaf(held[j][e], held[j][e], acc);
+      }
+  }
+  else {
+    for (int c = lane; c < chunks; c += 64) {
+      const f32x4 v = load_row4<IN_T>(xr + 4 * c);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc = __builtin_fmaf(v[e], v[e], acc);
+    }
+  }
+#pragma unroll
+  for (int step = 32; step >= 1; step >>= 1) acc = acc + __shfl_xor(acc, step, 64);
+  const float ms = acc / (float)K;
+  const float r  = 1.0f / __builtin_sqrtf(ms + eps);
+  // second pass: lanes beyond the row's end still take part in the cross-lane maxima (with zeros)
+  if constexpr (NJ > 0) {
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+      if (64 * j < chunks) rmsnorm_quant_chunk(held[j], r, w, q, scale, m, M, K, 64 * j + lane, chunks, lane);
+  }
+  else {
+    for (int c0 = 0; c0 < chunks; c0 += 64) {
+      const int c = c0 + lane;
+      f32x4     v = {0.f, 0.f, 0.f, 0.f};
+      if (c < chunks) v = load_row4<IN_T>(xr + 4 * c);
+      rmsnorm_quant_chunk(v, r, w, q, scale, m, M, K, c, chunks, lane);
+    }
+  }
+}
+
+hipError_t rmsnorm_quant_launch(int in_dtype, const void* x, const float* w, float eps, void* q, float* scale, int M, int K,
+                                hipStream_t stream)
+{
+  const dim3 grid((M + 3) / 4), block(256);
+#define LLMMM_NORM_GO(T)                                                                                                                     \
+  {                                                                                                                                          \
+    if (K <= 64 * 4 * 10)                                                                                                                    \
+      hipLaunchKernelGGL((rmsnorm_quant_1x128_kernel<T, 10>), grid, block, 0, stream, (const T*)x, w, eps, (uint8_t*)q, scale, M, K);         \
+    else if (K <= 64 * 4 * 16)                                                                                                               \
+      hipLaunchKernelGGL((rmsnorm_quant_1x128_kernel<T, 16>), grid, block, 0, stream, (const T*)x, w, eps, (uint8_t*)q, scale, M, K);         \
+    else                                                                                                                                     \
+      hipLaunchKernelGGL((rmsnorm_quant_1x128_kernel<T, 0>), grid, block, 0, stream, (const T*)x, w, eps, (uint8_t*)q, scale, M, K);          \
+  }
+  switch (in_dtype) {
+    case LLMMM_DTYPE_F16: LLMMM_NORM_GO(_Float16) break;
+    case LLMMM_DTYPE_BF16: LLMMM_NORM_GO(__bf16) break;
+    case LLMMM_DTYPE_F32: LLMMM_NORM_GO(float) break;
+    default: return hipErrorInvalidValue;
+  }
+#undef LLMMM_NORM_GO
+  return hipGetLastError();
+}
+
 __global__ void fill_u32_kernel(uint32_t* p, uint32_t value, size_t n)
 {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

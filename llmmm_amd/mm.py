@@ -109,6 +109,21 @@ def quantize_weight(wt, stream=None):
     return q, s
 
 
+def rmsnorm_quantize_activation(x, weight, eps, stream=None):
+    """RMSNorm fused in front of the activation quantiser (the fusion the reference plans, README.md:16):
+    x [M,K] float32 / bfloat16 / float16, weight [K] float32 -> (codes uint8 [M,K], scales float32 [K/128, M]) of
+    ``x / sqrt(mean(x^2) + eps) * weight``, ready to be the A operand of the FP8 GEMM."""
+    M, K = x.shape
+    code = {torch.float32: _lib.DTYPE_F32, torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16}.get(x.dtype)
+    if code is None:
+        raise RuntimeError("T is not supported.")
+    q = torch.empty((M, K), dtype=torch.uint8, device=x.device)
+    s = torch.empty(((K + 127) // 128, M), dtype=torch.float32, device=x.device)
+    check(lib.llmmm_rmsnorm_quant_fp8(code, _ptr(x, "x"), _ptr(weight, "weight", (torch.float32,), K), ctypes.c_float(eps), _ptr(q, "q"),
+                                      _ptr(s, "scale"), M, K, _stream(stream)))
+    return q, s
+
+
 # ------------------------------------------------------------------------------------- FP8 GEMM
 def workspace_bytes(out_kind, M, N, K):
     return int(lib.llmmm_fp8_gemm_workspace(out_kind, M, N, K))

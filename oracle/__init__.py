@@ -25,8 +25,7 @@ def build(force=False):
 
 
 def _load():
-    if not os.path.exists(_LIB_PATH):
-        build()
+    build()  # no-op unless the library is missing or older than oracle.c
     lib = ctypes.CDLL(_LIB_PATH)
     c = ctypes
     f32p, u8p, u16p = c.POINTER(c.c_float), c.POINTER(c.c_uint8), c.POINTER(c.c_uint16)
@@ -46,6 +45,7 @@ def _load():
         "oracle_dequant_fp8": (None, [u8p, f32p, f32p, c.c_int, c.c_int, c.c_int, c.c_int]),
         "oracle_fp8_gemm": (c.c_int, [u8p, f32p, u8p, f32p, f32p, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int]),
         "oracle_requant_c_1x128": (None, [f32p, u8p, f32p, c.c_int, c.c_int, c.c_int, c.c_int]),
+        "oracle_rmsnorm": (None, [f32p, f32p, c.c_float, f32p, c.c_int, c.c_int]),
         "oracle_e4m3_encode_n": (None, [f32p, u8p, c.c_size_t]),
         "oracle_e4m3_decode_n": (None, [u8p, f32p, c.c_size_t]),
         "oracle_f32_to_f16_n": (None, [f32p, u16p, c.c_size_t]),
@@ -249,6 +249,22 @@ def swiglu(C):
 def swiglu_requant(C):
     """(Cq [M, N/2], Cs [N/256, M]): the fused epilogue's 1x128 quantisation applied to swiglu(C)."""
     return requant_c_1x128(swiglu(C))
+
+
+def rmsnorm(x, w, eps):
+    """y = x / sqrt(mean(x^2) + eps) * w in fp32, rows of x [M,K] (K % 4 == 0), w [K].  No reference kernel
+    (README.md:16 plans the fusion); the summation order is that of a 64-lane wavefront, see oracle.c."""
+    x, w = _f32(x), _f32(w)
+    M, K = x.shape
+    assert K % 4 == 0 and w.shape == (K,)
+    y = np.empty((M, K), np.float32)
+    _lib.oracle_rmsnorm(_p(x, ctypes.c_float), _p(w, ctypes.c_float), ctypes.c_float(eps), _p(y, ctypes.c_float), M, K)
+    return y
+
+
+def rmsnorm_quant(x, w, eps):
+    """RMSNorm followed by the activation quantiser (1x128, transposed scales): (q [M,K], s [ceil(K/128), M])."""
+    return quant_fp8(rmsnorm(x, w, eps), 1, True)
 
 
 # ----------------------------------------------------------------------------- offline layouts

@@ -30,6 +30,12 @@
  *                            examples/005.fp8.mm.cu:759-774 (division form)
  *                                                            pinned: idempotence, B = I => Cq == Aq
  *
+ *   oracle_rmsnorm           no reference kernel (fusing RMSNorm into the quantiser is on the reference's
+ *                            plan, README.md:16): y = x / sqrt(mean(x^2) + eps) * w in fp32, the sum of squares
+ *                            taken in the order of a 64-lane wavefront (see the function)
+ *                                                            pinned: float64 evaluation, exact invariance under
+ *                                                            power-of-two scaling (eps = 0), unit mean square
+ *
  * Compile with -ffp-contract=off: every fused multiply-add below is written explicitly.
  */
 #include <math.h>
@@ -441,4 +447,32 @@ ORACLE_API void oracle_f32_to_bf16_n(const float* x, uint16_t* h, size_t n)
 ORACLE_API void oracle_bf16_to_f32_n(const uint16_t* h, float* x, size_t n)
 {
   for (size_t i = 0; i < n; ++i) x[i] = oracle_bf16_to_f32(h[i]);
+}
+
+/* RMSNorm in fp32: y[m,k] = (x[m,k] * r) * w[k], r = 1 / sqrt(sum_k x[m,k]^2 / K + eps).
+ * No reference kernel (README.md:16 plans the fusion); the arithmetic order is this build's definition, chosen so
+ * that a 64-lane wavefront reproduces it bit for bit: the row is cut into chunks of 4 consecutive elements, lane l
+ * accumulates chunks l, l+64, l+128, ... in ascending order with one fused multiply-add per element
+ * (acc = fma(x, x, acc), elements of a chunk in ascending order), and the 64 partial sums are combined by a
+ * butterfly: p[l] += p[l ^ 32], then ^16, ^8, ^4, ^2, ^1.  Division by K, the square root and the reciprocal are
+ * correctly rounded IEEE operations.  K % 4 == 0. */
+ORACLE_API void oracle_rmsnorm(const float* x, const float* w, float eps, float* y, int M, int K)
+{
+#pragma omp parallel for schedule(static)
+  for (int m = 0; m < M; ++m) {
+    const float* xr = x + (size_t)m * K;
+    float        p[64];
+    for (int l = 0; l < 64; ++l) p[l] = 0.f;
+    const int chunks = K / 4;
+    for (int c = 0; c < chunks; ++c)
+      for (int e = 0; e < 4; ++e) p[c & 63] = fmaf(xr[4 * c + e], xr[4 * c + e], p[c & 63]);
+    for (int step = 32; step >= 1; step >>= 1) {
+      float t[64];
+      for (int l = 0; l < 64; ++l) t[l] = p[l] + p[l ^ step];
+      for (int l = 0; l < 64; ++l) p[l] = t[l];
+    }
+    const float ms = p[0] / (float)K;
+    const float r  = 1.0f / sqrtf(ms + eps);
+    for (int k = 0; k < K; ++k) y[(size_t)m * K + k] = (xr[k] * r) * w[k];
+  }
 }

@@ -192,3 +192,17 @@ def test_swiglu_validation_without_device():
     assert lib.llmmm_fp8_gemm_query(_lib.OUT_FP8Q_SWIGLU, 128, 19456, 2560, ctypes.byref(q)) == _lib.OK
     if q.tile in (_lib.TILE_128x128, _lib.TILE_256x128):
         assert lib.llmmm_fp8_gemm_workspace(_lib.OUT_FP8Q_SWIGLU, 128, 19456, 2560) >= 128 * 19456 * 4
+
+
+def test_rmsnorm_quant_validation_without_device():
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    f = lib.llmmm_rmsnorm_quant_fp8
+    eps = ctypes.c_float(1e-6)
+    assert f(_lib.DTYPE_F32, FAKE, FAKE, eps, FAKE, FAKE, 4, 100, None) == _lib.ERR_NOT_ALIGNED
+    assert f(7, FAKE, FAKE, eps, FAKE, FAKE, 4, 128, None) == _lib.ERR_UNSUPPORTED_TYPE
+    assert f(_lib.DTYPE_BF16, None, FAKE, eps, FAKE, FAKE, 4, 128, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(_lib.DTYPE_BF16, FAKE, FAKE, ctypes.c_float(-1.0), FAKE, FAKE, 4, 128, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(_lib.DTYPE_BF16, FAKE, FAKE, ctypes.c_float(float("nan")), FAKE, FAKE, 4, 128, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(_lib.DTYPE_F16, FAKE, FAKE, eps, FAKE, FAKE, 0, 128, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(_lib.DTYPE_F16, ctypes.c_void_p(0x1008), FAKE, eps, FAKE, FAKE, 4, 128, None) == _lib.ERR_INVALID_ARGUMENT
