@@ -212,9 +212,36 @@ __global__ void __launch_bounds__(256) rmsnorm_quant_1x128_kernel(const IN_T* __
   const float r  = 1.0f / __builtin_sqrtf(ms + eps);
   // second pass: lanes beyond the row's end still take part in the cross-lane maxima (with zeros)
   if constexpr (NJ > 0) {
+    // phase by phase over all the chunks of the lane, so that the NJ independent cross-lane reductions overlap
+    // instead of queueing behind each other: normalise, five lockstep max steps, then quantise and store
+    float amax[NJ];
 #pragma unroll
-    for (int j = 0; j < NJ; ++j)
-      if (64 * j < chunks) rmsnorm_quant_chunk(held[j], r, w, q, scale, m, M, K, 64 * j + lane, chunks, lane);
+    for (int j = 0; j < NJ; ++j) {
+      const int c = 64 * j + lane;
+      f32x4     y = {0.f, 0.f, 0.f, 0.f};
+      if (c < chunks) {
+        const f32x4 wv = *(const f32x4*)(w + 4 * c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = (held[j][e] * r) * wv[e];
+      }
+      held[j] = y;
+      amax[j] = amax4(0.f, y);
+    }
+#pragma unroll
+    for (int step = 1; step <= 16; step <<= 1)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) amax[j] = wave_xor_max(amax[j], step);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      const int   c  = 64 * j + lane;
+      const float sc = amax[j] / 448.f;
+      uint32_t    cd = 0;
+      if (sc != 0.f) cd = q_pack_e4m3x4(held[j][0] / sc, held[j][1] / sc, held[j][2] / sc, held[j][3] / sc);
+      if (c < chunks) {
+        *(uint32_t*)(q + (size_t)m * K + 4 * c) = cd;
+        if ((lane & 31) == 0) scale[(size_t)(c >> 5) * M + m] = sc;
+      }
+    }
   }
   else {
     for (int c0 = 0; c0 < chunks; c0 += 64) {
