@@ -169,6 +169,49 @@ def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0, preshuffled=False):
             "split_k": split, "weight_copies": copies}
 
 
+def bench_mlp_chain(M, steps, warmup, hidden=2560, inter=9728, rotate_bytes=768 << 20):
+    """Qwen3-4B MLP block at decode-sized M: hidden state bf16 [M, hidden] -> RMSNorm+quant -> gate_up (N = 2*inter)
+    with SwiGLU output -> down (bf16 out).  Algorithmic bytes: both weight matrices once."""
+    import llmmm_amd
+    from llmmm_amd import _lib
+    g = torch.Generator(device="cuda").manual_seed(11)
+    per_copy = 3 * inter * hidden
+    copies = max(2, int(np.ceil(rotate_bytes / float(per_copy))))
+    weights = []
+    for _ in range(copies):
+        Wgu = torch.randn((2 * inter, hidden), generator=g, device="cuda") * 0.02
+        Wd = torch.randn((hidden, inter), generator=g, device="cuda") * 0.02
+        gq, gs = llmmm_amd.quantize_weight(Wgu)
+        dq, ds = llmmm_amd.quantize_weight(Wd)
+        weights.append((llmmm_amd.preshuffle_weight(gq), gs, llmmm_amd.preshuffle_weight(dq), ds))
+        del Wgu, Wd, gq, dq
+    x = torch.randn((M, hidden), generator=g, device="cuda").to(torch.bfloat16)
+    wn = torch.ones(hidden, device="cuda")
+    Aq = torch.empty((M, hidden), dtype=torch.uint8, device="cuda")
+    As = torch.empty((hidden // 128, M), dtype=torch.float32, device="cuda")
+    Hq = torch.empty((M, inter), dtype=torch.uint8, device="cuda")
+    Hs = torch.empty((inter // 128, M), dtype=torch.float32, device="cuda")
+    Y = torch.empty((M, hidden), dtype=torch.bfloat16, device="cuda")
+    ws1 = llmmm_amd.make_workspace(_lib.OUT_FP8Q_SWIGLU, M, 2 * inter, hidden)
+    ws2 = llmmm_amd.make_workspace(_lib.OUT_BF16, M, hidden, inter)
+    state = {"i": 0}
+
+    def step():
+        gq, gs, dq, ds = weights[state["i"] % copies]
+        state["i"] += 1
+        rc = _lib.lib.llmmm_rmsnorm_quant_fp8(_lib.DTYPE_BF16, x.data_ptr(), wn.data_ptr(), 1e-6, Aq.data_ptr(), As.data_ptr(), M, hidden,
+                                              torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(Aq, As, gq, gs, Hq, Hs, M, 2 * inter, hidden, workspace=ws1,
+                                                                                           b_preshuffled=True)
+        llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(Hq, Hs, dq, ds, Y, M, hidden, inter, workspace=ws2, b_preshuffled=True)
+
+    ms, _ = _events_ms(step, steps, warmup, graph=True)
+    return {"name": "qwen3_4b_mlp_block_m%d" % M, "M": M, "hidden": hidden, "intermediate": inter, "us": ms * 1e3,
+            "hbm_gbs": per_copy / ms * 1e-6, "frac_of_hbm_peak": per_copy / ms * 1e-6 / PEAK_HBM_GBS, "weight_copies": copies,
+            "launches": "rmsnorm+quant, gate_up+swiglu (+reduce), down (+reduce)"}
+
+
 def cpu_baseline_fp16(M, N, K, rows):
     """Oracle Kahan GEMM on the first `rows` rows of the headline workload, all host threads."""
     import oracle
@@ -313,6 +356,11 @@ def main():
             nb = m * 2560 * 3.0 + m * 20 * 4.0
             shapes.append({"name": "rmsnorm_quant_bf16_m%d_k2560" % m, "M": m, "K": 2560, "us": ms_ * 1e3, "hbm_gbs": nb / ms_ * 1e-6,
                            "frac_of_hbm_peak": nb / ms_ * 1e-6 / PEAK_HBM_GBS})
+        # One decoder MLP block as three launches: RMSNorm+quant -> gate_up GEMM with fused SwiGLU output -> down GEMM
+        # (bf16 output), weights pre-shuffled and rotated over distinct copies so that they stream from HBM.
+        for m in (1, 16):
+            shapes.append(bench_mlp_chain(m, s2, w2))
+            torch.cuda.empty_cache()
         line["shapes"] = shapes
 
     if not args.no_cpu:

@@ -119,11 +119,17 @@ __global__ void __launch_bounds__(256) quant_128x128_kernel(const float* __restr
 // RMSNorm fused in front of the 1 x 128 activation quantiser (the "RMSNorm + fp8 dynamic quant" fusion the reference
 // plans, README.md:16; no reference kernel):
 //   y[m,k] = (x[m,k] * r) * w[k],  r = 1 / sqrt(sum_k x[m,k]^2 / K + eps),  then q, s = quant_1x128(y), scales transposed.
-// One wavefront per row.  The row is cut into chunks of four elements; lane l owns chunks l, l+64, ...: a first pass
-// accumulates the squares (one fused multiply-add per element, chunks in ascending order, then the xor butterfly
-// 32, 16, .. 1 over the lanes -- this fixed order is what the CPU oracle restates, so the results are bit-exact), a
-// second pass normalises and quantises: a 128-column group is the 32 consecutive chunks of half a wavefront, so its
-// amax needs five cross-lane steps.  HBM traffic: x once, q once.
+// The sum of squares has one fixed order, which the CPU oracle restates, so that results are bit-exact and do not
+// depend on which of the two kernels below runs: the row is cut into chunks of four elements; chunk c belongs to
+// virtual lane c % 256, which accumulates its chunks in ascending order with one fused multiply-add per element;
+// the 256 partial sums are combined per group of 64 by an xor butterfly (32, 16, .. 1) and the four group sums as
+// (G0 + G1) + (G2 + G3).  A second pass normalises and quantises: a 128-column group is 32 consecutive chunks =
+// half a wavefront in either kernel, so its amax needs five cross-lane steps.  HBM traffic: x once, q once.
+//   * rmsnorm_quant_row_kernel:   one 256-thread workgroup per row (a thread is a virtual lane), the row held in
+//     registers: K <= 10240.  Measured at K = 2560 against a wavefront per row: 3.2 instead of 8.2 us at M = 16 (a
+//     single wavefront works through the row's 40 divisions per lane on its own), 6.9 instead of 9.4 us at M = 2048.
+//   * rmsnorm_quant_1x128_kernel: one wavefront per row (a lane plays four virtual lanes), the row read twice:
+//     longer rows.
 template <typename IN_T>
 __device__ __forceinline__ f32x4 load_row4(const IN_T* p);
 template <>
@@ -172,83 +178,101 @@ __device__ __forceinline__ void rmsnorm_quant_chunk(f32x4 v, float r, const floa
   }
 }
 
-// NJ > 0: the row has at most 64 * NJ chunks and stays in registers between the two passes (all its loads in flight
-// at once, the row read once).  NJ == 0: any K, the row is read twice (the second time from the L2).
-template <typename IN_T, int NJ>
+// One wavefront per row, any K: the row is read twice (the second time from the L2).  A lane plays the four
+// virtual lanes lane, lane + 64, lane + 128, lane + 192.
+template <typename IN_T>
 __global__ void __launch_bounds__(256) rmsnorm_quant_1x128_kernel(const IN_T* __restrict__ x, const float* __restrict__ w, float eps,
                                                                   uint8_t* __restrict__ q, float* __restrict__ scale, int M, int K)
 {
   const int lane = threadIdx.x & 63;
   const int m    = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (m >= M) return;  // whole wavefronts leave: no barrier below
+  const IN_T* xr      = x + (size_t)m * K;
+  const int   chunks  = K >> 2;
+  float       part[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int c0 = 0; c0 < chunks; c0 += 256) {
+#pragma unroll
+    for (int gidx = 0; gidx < 4; ++gidx) {
+      const int c = c0 + 64 * gidx + lane;
+      if (c < chunks) {
+        const f32x4 v = load_row4<IN_T>(xr + 4 * c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) part[gidx] = __builtin_fmaf(v[e], v[e], part[gidx]);
+      }
+    }
+  }
+#pragma unroll
+  for (int step = 32; step >= 1; step >>= 1)
+#pragma unroll
+    for (int gidx = 0; gidx < 4; ++gidx) part[gidx] = part[gidx] + __shfl_xor(part[gidx], step, 64);
+  const float acc = (part[0] + part[1]) + (part[2] + part[3]);
+  const float ms  = acc / (float)K;
+  const float r   = 1.0f / __builtin_sqrtf(ms + eps);
+  // second pass: lanes beyond the row's end still take part in the cross-lane maxima (with zeros)
+  for (int c0 = 0; c0 < chunks; c0 += 64) {
+    const int c = c0 + lane;
+    f32x4     v = {0.f, 0.f, 0.f, 0.f};
+    if (c < chunks) v = load_row4<IN_T>(xr + 4 * c);
+    rmsnorm_quant_chunk(v, r, w, q, scale, m, M, K, c, chunks, lane);
+  }
+}
+
+// One workgroup of 256 threads per row: thread t is virtual lane t and owns chunks t, t + 256, ...  NI = chunks per
+// thread held in registers (K <= 1024 * NI).
+template <typename IN_T, int NI>
+__global__ void __launch_bounds__(256) rmsnorm_quant_row_kernel(const IN_T* __restrict__ x, const float* __restrict__ w, float eps,
+                                                                uint8_t* __restrict__ q, float* __restrict__ scale, int M, int K)
+{
+  __shared__ float group_sum[4];
+  const int   t      = threadIdx.x;
+  const int   m      = blockIdx.x;
   const IN_T* xr     = x + (size_t)m * K;
   const int   chunks = K >> 2;
-  float       acc    = 0.f;
-  f32x4       held[NJ > 0 ? NJ : 1];
-  if constexpr (NJ > 0) {
+  f32x4       held[NI], wv[NI];
+  float       acc = 0.f;
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int c = lane + 64 * j;
-      held[j]     = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (c < chunks) held[j] = load_row4<IN_T>(xr + 4 * c);
-    }
-#pragma unroll
-    for (int j = 0; j < NJ; ++j)
-      if (lane + 64 * j < chunks) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc = __builtin_fmaf(held[j][e], held[j][e], acc);
-      }
-  }
-  else {
-    for (int c = lane; c < chunks; c += 64) {
-      const f32x4 v = load_row4<IN_T>(xr + 4 * c);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) acc = __builtin_fmaf(v[e], v[e], acc);
+  for (int i = 0; i < NI; ++i) {
+    const int c = t + 256 * i;
+    held[i]     = f32x4{0.f, 0.f, 0.f, 0.f};
+    wv[i]       = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (c < chunks) {
+      held[i] = load_row4<IN_T>(xr + 4 * c);
+      wv[i]   = *(const f32x4*)(w + 4 * c);
     }
   }
+#pragma unroll
+  for (int i = 0; i < NI; ++i)
+    if (t + 256 * i < chunks) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc = __builtin_fmaf(held[i][e], held[i][e], acc);
+    }
 #pragma unroll
   for (int step = 32; step >= 1; step >>= 1) acc = acc + __shfl_xor(acc, step, 64);
-  const float ms = acc / (float)K;
-  const float r  = 1.0f / __builtin_sqrtf(ms + eps);
-  // second pass: lanes beyond the row's end still take part in the cross-lane maxima (with zeros)
-  if constexpr (NJ > 0) {
-    // phase by phase over all the chunks of the lane, so that the NJ independent cross-lane reductions overlap
-    // instead of queueing behind each other: normalise, five lockstep max steps, then quantise and store
-    float amax[NJ];
+  if ((t & 63) == 0) group_sum[t >> 6] = acc;
+  __syncthreads();
+  const float total = (group_sum[0] + group_sum[1]) + (group_sum[2] + group_sum[3]);
+  const float ms    = total / (float)K;
+  const float r     = 1.0f / __builtin_sqrtf(ms + eps);
+  float       amax[NI];
 #pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int c = 64 * j + lane;
-      f32x4     y = {0.f, 0.f, 0.f, 0.f};
-      if (c < chunks) {
-        const f32x4 wv = *(const f32x4*)(w + 4 * c);
+  for (int i = 0; i < NI; ++i) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) y[e] = (held[j][e] * r) * wv[e];
-      }
-      held[j] = y;
-      amax[j] = amax4(0.f, y);
-    }
-#pragma unroll
-    for (int step = 1; step <= 16; step <<= 1)
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) amax[j] = wave_xor_max(amax[j], step);
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      const int   c  = 64 * j + lane;
-      const float sc = amax[j] / 448.f;
-      uint32_t    cd = 0;
-      if (sc != 0.f) cd = q_pack_e4m3x4(held[j][0] / sc, held[j][1] / sc, held[j][2] / sc, held[j][3] / sc);
-      if (c < chunks) {
-        *(uint32_t*)(q + (size_t)m * K + 4 * c) = cd;
-        if ((lane & 31) == 0) scale[(size_t)(c >> 5) * M + m] = sc;
-      }
-    }
+    for (int e = 0; e < 4; ++e) held[i][e] = (held[i][e] * r) * wv[i][e];  // zeros beyond the row's end
+    amax[i] = amax4(0.f, held[i]);
   }
-  else {
-    for (int c0 = 0; c0 < chunks; c0 += 64) {
-      const int c = c0 + lane;
-      f32x4     v = {0.f, 0.f, 0.f, 0.f};
-      if (c < chunks) v = load_row4<IN_T>(xr + 4 * c);
-      rmsnorm_quant_chunk(v, r, w, q, scale, m, M, K, c, chunks, lane);
+#pragma unroll
+  for (int step = 1; step <= 16; step <<= 1)
+#pragma unroll
+    for (int i = 0; i < NI; ++i) amax[i] = wave_xor_max(amax[i], step);
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int   c  = t + 256 * i;
+    const float sc = amax[i] / 448.f;
+    uint32_t    cd = 0;
+    if (sc != 0.f) cd = q_pack_e4m3x4(held[i][0] / sc, held[i][1] / sc, held[i][2] / sc, held[i][3] / sc);
+    if (c < chunks) {
+      *(uint32_t*)(q + (size_t)m * K + 4 * c) = cd;
+      if ((t & 31) == 0) scale[(size_t)(c >> 5) * M + m] = sc;
     }
   }
 }
@@ -257,14 +281,14 @@ hipError_t rmsnorm_quant_launch(int in_dtype, const void* x, const float* w, flo
                                 hipStream_t stream)
 {
   const dim3 grid((M + 3) / 4), block(256);
-#define LLMMM_NORM_GO(T)                                                                                                                     \
-  {                                                                                                                                          \
-    if (K <= 64 * 4 * 10)                                                                                                                    \
-      hipLaunchKernelGGL((rmsnorm_quant_1x128_kernel<T, 10>), grid, block, 0, stream, (const T*)x, w, eps, (uint8_t*)q, scale, M, K);         \
-    else if (K <= 64 * 4 * 16)                                                                                                               \
-      hipLaunchKernelGGL((rmsnorm_quant_1x128_kernel<T, 16>), grid, block, 0, stream, (const T*)x, w, eps, (uint8_t*)q, scale, M, K);         \
-    else                                                                                                                                     \
-      hipLaunchKernelGGL((rmsnorm_quant_1x128_kernel<T, 0>), grid, block, 0, stream, (const T*)x, w, eps, (uint8_t*)q, scale, M, K);          \
+#define LLMMM_NORM_GO(T)                                                                                                               \
+  {                                                                                                                                    \
+    if (K <= 1024 * 3)                                                                                                                 \
+      hipLaunchKernelGGL((rmsnorm_quant_row_kernel<T, 3>), dim3(M), block, 0, stream, (const T*)x, w, eps, (uint8_t*)q, scale, M, K);   \
+    else if (K <= 1024 * 10)                                                                                                           \
+      hipLaunchKernelGGL((rmsnorm_quant_row_kernel<T, 10>), dim3(M), block, 0, stream, (const T*)x, w, eps, (uint8_t*)q, scale, M, K);  \
+    else                                                                                                                               \
+      hipLaunchKernelGGL((rmsnorm_quant_1x128_kernel<T>), grid, block, 0, stream, (const T*)x, w, eps, (uint8_t*)q, scale, M, K);       \
   }
   switch (in_dtype) {
     case LLMMM_DTYPE_F16: LLMMM_NORM_GO(_Float16) break;

@@ -253,7 +253,7 @@ def swiglu_requant(C):
 
 def rmsnorm(x, w, eps):
     """y = x / sqrt(mean(x^2) + eps) * w in fp32, rows of x [M,K] (K % 4 == 0), w [K].  No reference kernel
-    (README.md:16 plans the fusion); the summation order is that of a 64-lane wavefront, see oracle.c."""
+    (README.md:16 plans the fusion); the summation order is that of 256 GPU lanes, see oracle.c."""
     x, w = _f32(x), _f32(w)
     M, K = x.shape
     assert K % 4 == 0 and w.shape == (K,)

@@ -32,7 +32,7 @@
  *
  *   oracle_rmsnorm           no reference kernel (fusing RMSNorm into the quantiser is on the reference's
  *                            plan, README.md:16): y = x / sqrt(mean(x^2) + eps) * w in fp32, the sum of squares
- *                            taken in the order of a 64-lane wavefront (see the function)
+ *                            taken in the order of 256 GPU lanes (see the function)
  *                                                            pinned: float64 evaluation, exact invariance under
  *                                                            power-of-two scaling (eps = 0), unit mean square
  *
@@ -451,28 +451,35 @@ ORACLE_API void oracle_bf16_to_f32_n(const uint16_t* h, float* x, size_t n)
 
 /* RMSNorm in fp32: y[m,k] = (x[m,k] * r) * w[k], r = 1 / sqrt(sum_k x[m,k]^2 / K + eps).
  * No reference kernel (README.md:16 plans the fusion); the arithmetic order is this build's definition, chosen so
- * that a 64-lane wavefront reproduces it bit for bit: the row is cut into chunks of 4 consecutive elements, lane l
- * accumulates chunks l, l+64, l+128, ... in ascending order with one fused multiply-add per element
- * (acc = fma(x, x, acc), elements of a chunk in ascending order), and the 64 partial sums are combined by a
- * butterfly: p[l] += p[l ^ 32], then ^16, ^8, ^4, ^2, ^1.  Division by K, the square root and the reciprocal are
- * correctly rounded IEEE operations.  K % 4 == 0. */
+ * that GPU wavefronts reproduce it bit for bit: the row is cut into chunks of 4 consecutive elements; chunk c belongs
+ * to virtual lane c % 256, which accumulates its chunks in ascending order with one fused multiply-add per element
+ * (acc = fma(x, x, acc), elements of a chunk in ascending order); each group of 64 virtual lanes combines its partial
+ * sums by a butterfly (p[l] += p[l ^ 32], then ^16, ^8, ^4, ^2, ^1), and the four group sums are added as
+ * (G0 + G1) + (G2 + G3).  Division by K, the square root and the reciprocal are correctly rounded IEEE operations.
+ * K % 4 == 0. */
 ORACLE_API void oracle_rmsnorm(const float* x, const float* w, float eps, float* y, int M, int K)
 {
 #pragma omp parallel for schedule(static)
   for (int m = 0; m < M; ++m) {
     const float* xr = x + (size_t)m * K;
-    float        p[64];
-    for (int l = 0; l < 64; ++l) p[l] = 0.f;
+    float        p[256];
+    for (int l = 0; l < 256; ++l) p[l] = 0.f;
     const int chunks = K / 4;
     for (int c = 0; c < chunks; ++c)
-      for (int e = 0; e < 4; ++e) p[c & 63] = fmaf(xr[4 * c + e], xr[4 * c + e], p[c & 63]);
-    for (int step = 32; step >= 1; step >>= 1) {
-      float t[64];
-      for (int l = 0; l < 64; ++l) t[l] = p[l] + p[l ^ step];
-      for (int l = 0; l < 64; ++l) p[l] = t[l];
+      for (int e = 0; e < 4; ++e) p[c & 255] = fmaf(xr[4 * c + e], xr[4 * c + e], p[c & 255]);
+    float G[4];
+    for (int g = 0; g < 4; ++g) {
+      float* pg = p + 64 * g;
+      for (int step = 32; step >= 1; step >>= 1) {
+        float t[64];
+        for (int l = 0; l < 64; ++l) t[l] = pg[l] + pg[l ^ step];
+        for (int l = 0; l < 64; ++l) pg[l] = t[l];
+      }
+      G[g] = pg[0];
     }
-    const float ms = p[0] / (float)K;
-    const float r  = 1.0f / sqrtf(ms + eps);
+    const float total = (G[0] + G[1]) + (G[2] + G[3]);
+    const float ms    = total / (float)K;
+    const float r     = 1.0f / sqrtf(ms + eps);
     for (int k = 0; k < K; ++k) y[(size_t)m * K + k] = (xr[k] * r) * w[k];
   }
 }

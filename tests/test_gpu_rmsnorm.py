@@ -8,7 +8,10 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("M,K", [(1, 2560), (16, 2560), (5, 128), (77, 4096), (2048, 2560), (33, 9728), (3, 384)])
+# both kernels (a workgroup per row with 3 or 10 chunks per thread for K <= 10240, a wavefront per row above) must
+# give the oracle's bits
+@pytest.mark.parametrize("M,K", [(1, 2560), (16, 2560), (5, 128), (77, 4096), (2048, 2560), (33, 9728), (3, 384), (520, 4096), (600, 9728),
+                                 (513, 128), (12, 10240 + 128), (70, 16384)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_bit_exact_against_oracle(lib, oracle, M, K, dtype):
     rng = np.random.default_rng(M * 7 + K)

@@ -38,11 +38,12 @@ def test_power_of_two_scaling_is_exact_without_eps(oracle):
 
 
 def test_documented_summation_order(oracle):
-    """The sum of squares in the documented order (64 interleaved partial sums of fused multiply-adds, then the
-    xor butterfly), restated with Python floats rounded to fp32 after every operation."""
+    """The sum of squares in the documented order (256 interleaved partial sums of fused multiply-adds, an xor
+    butterfly inside each group of 64, then (G0 + G1) + (G2 + G3)), restated with exact rationals rounded to fp32
+    after every operation."""
     from fractions import Fraction
     rng = np.random.default_rng(4)
-    K = 1024
+    K = 2560
     x = rng.standard_normal((1, K)).astype(np.float32)
 
     def f32(v):
@@ -51,14 +52,19 @@ def test_documented_summation_order(oracle):
     def fma(a, b, c):  # exactly rounded a*b+c
         return np.float32(float(Fraction(float(a)) * Fraction(float(b)) + Fraction(float(c))))
 
-    p = [np.float32(0)] * 64
+    p = [np.float32(0)] * 256
     for c in range(K // 4):
         for e in range(4):
             v = x[0, 4 * c + e]
-            p[c % 64] = fma(v, v, p[c % 64])
-    for step in (32, 16, 8, 4, 2, 1):
-        p = [f32(p[l] + p[l ^ step]) for l in range(64)]
-    ms = f32(p[0] / np.float32(K))
+            p[c % 256] = fma(v, v, p[c % 256])
+    G = []
+    for g in range(4):
+        pg = p[64 * g:64 * g + 64]
+        for step in (32, 16, 8, 4, 2, 1):
+            pg = [f32(pg[l] + pg[l ^ step]) for l in range(64)]
+        G.append(pg[0])
+    total = f32(f32(G[0] + G[1]) + f32(G[2] + G[3]))
+    ms = f32(total / np.float32(K))
     r = f32(np.float32(1.0) / np.sqrt(f32(ms + np.float32(1e-6))))
     w = np.ones(K, np.float32)
     want = (x[0] * r) * w
