@@ -302,6 +302,7 @@ __device__ __forceinline__ void swiglu_finish(const f32x4 (&acc)[8][MF], const f
 
 // BMODE bit 0 (BPRE): Bt is the pre-shuffled image of the weights (layout.hip) instead of row-major [N, K].
 // BMODE bit 1 (BNT): the weight loads carry the non-temporal hint (one tile row: every weight byte is read once).
+// BMODE bit 2 (DEEP, 32-row-wave tiles only): the launch has at most one workgroup per CU, which then runs a deeper pipeline.
 template <int BM, int BN, int WM, int OUT, int BMODE>
 __global__ void __launch_bounds__((BM / WM) * (BN / 128) * 64)
 fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
@@ -311,10 +312,12 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   typedef Fp8Tile<BM, BN, WM> TC;
   constexpr int  MF   = TC::MF;
   constexpr bool BPRE = (BMODE & 1) != 0, BNT = (BMODE & 2) != 0;
-  // Weights that are streamed once (a single tile row: decode-sized M) leave the workgroups waiting on memory
-  // latency, not on the matrix pipe, and there is at most one workgroup per CU: the 32-row-wave tiles then run a
-  // deeper pipeline -- as many stages as fit the LDS instead of two, the slice scales travelling with the stage.
-  constexpr bool DEEP    = BNT && WM == 32;
+  // A launch with at most one workgroup per CU (few tiles: decode-sized or mid-sized M) leaves the workgroups
+  // waiting on memory latency, not on the matrix pipe, and the LDS a second workgroup would have used lies idle:
+  // the 32-row-wave tiles then run a deeper pipeline -- as many stages as fit the LDS instead of two, the slice
+  // scales travelling with the stage.  (With two workgroups per CU the two-stage form is faster: 29 vs 38 us on
+  // 2048 x 2560 x 4096 in 128 x 128 tiles.)
+  constexpr bool DEEP    = (BMODE & 4) != 0 && WM == 32;
   constexpr int  STAGE_D = TC::STAGE + TC::NW * 256;                 // operands + 256 bytes of scales per wave
   constexpr int  NST     = !DEEP ? 2 : (4 * STAGE_D <= 160 * 1024 ? 4 : 3);
   __shared__ __attribute__((aligned(1024))) char lds[DEEP ? NST * STAGE_D : 2 * TC::STAGE];
@@ -654,10 +657,15 @@ static hipError_t launch_reduce(const float* planes, int S, void* C, float* Cs, 
 template <int BM, int BN, int WM, int OUT>
 static auto pick_kernel(int bmode) -> decltype(&fp8_gemm_kernel<BM, BN, WM, OUT, 0>)
 {
+  if constexpr (WM != 32) bmode &= 3;  // only the 32-row-wave tiles have a deep form
   switch (bmode) {
     case 1: return fp8_gemm_kernel<BM, BN, WM, OUT, 1>;
     case 2: return fp8_gemm_kernel<BM, BN, WM, OUT, 2>;
     case 3: return fp8_gemm_kernel<BM, BN, WM, OUT, 3>;
+    case 4: return fp8_gemm_kernel<BM, BN, WM, OUT, WM == 32 ? 4 : 0>;
+    case 5: return fp8_gemm_kernel<BM, BN, WM, OUT, WM == 32 ? 5 : 1>;
+    case 6: return fp8_gemm_kernel<BM, BN, WM, OUT, WM == 32 ? 6 : 2>;
+    case 7: return fp8_gemm_kernel<BM, BN, WM, OUT, WM == 32 ? 7 : 3>;
     default: return fp8_gemm_kernel<BM, BN, WM, OUT, 0>;
   }
 }
@@ -668,7 +676,9 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
 {
   typedef Fp8Tile<BM, BN, WM> TC;
   const int tiles_m = M / BM, tiles_n = N / BN;
-  const int bmode   = (bpre ? 1 : 0) | (tiles_m == 1 ? 2 : 0);
+  // one tile row: the weights are read once (streamed, deep); at most one workgroup per CU: deep
+  const bool one_per_cu = (long)tiles_m * tiles_n * (S < 1 ? 1 : S) <= 256;
+  const int  bmode      = (bpre ? 1 : 0) | (tiles_m == 1 ? 2 | 4 : 0) | (one_per_cu ? 4 : 0);
   if (S <= 1 && planes == nullptr) {
     if constexpr (OUT == OUT_SWIGLU && BN != 256) {
       return hipErrorInvalidValue;  // unsplit SwiGLU needs a 256-wide tile (the host picks one)

@@ -95,6 +95,16 @@ def test_short_k_single_tile_row(lib, oracle, tile, M, K):
     _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, tile=TILES[tile], split_k=2 if K >= 256 else 1), ref, "tile %s M=%d K=%d split" % (tile, M, K))
 
 
+@pytest.mark.parametrize("tile", ["128x256", "256x128", "128x128"])
+def test_small_tiles_with_more_workgroups_than_cus(lib, oracle, tile):
+    """More than 256 workgroups: the 32-row-wave tiles run their two-stage form (two workgroups per CU) instead of
+    the deep pipeline that the smaller test shapes get."""
+    M, N, K = 2048, 4352, 384
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=77)
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, tile=TILES[tile]), ref, "tile %s, 272+ workgroups" % tile)
+
+
 def test_single_slice(lib, oracle):
     Aq, As, Bq, Bs = fp8_inputs(oracle, 128, 128, 128, seed=11)
     _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs), oracle.fp8_gemm(Aq, As, Bq, Bs), "K=128")
