@@ -62,6 +62,7 @@ extern "C" {
 #define LLMMM_TILE_128x256 1
 #define LLMMM_TILE_256x128 2
 #define LLMMM_TILE_128x128 3
+#define LLMMM_TILE_64x128 4 /* FP16/BF16 GEMM only: small problems */
 #define LLMMM_TILE_SKINNY 8 /* M <= 128 weight-streaming kernel */
 
 /* Weight layout of the FP8 GEMM's B operand (llmmm_gemm_cfg.b_layout). */

@@ -20,7 +20,7 @@ B_ROW_MAJOR, B_TRANSPOSED = 0, 1
 OUT_F32, OUT_BF16, OUT_FP8Q, OUT_FP8Q_SWIGLU = 0, 1, 2, 3
 QUANT_1x128_T, QUANT_128x128, QUANT_1x128, QUANT_128x128_T = 0, 1, 2, 3
 FP8_B_ROWS, FP8_B_PRESHUFFLED = 0, 1
-TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_SKINNY = -1, 0, 1, 2, 3, 8
+TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_64x128, TILE_SKINNY = -1, 0, 1, 2, 3, 4, 8
 
 
 class GemmCfg(ctypes.Structure):

@@ -42,7 +42,7 @@ struct Mfma32<__bf16> {
   static __device__ __forceinline__ f32x4 run(vec x, vec y, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, c, 0, 0, 0); }
 };
 
-// WM = rows of a wave's sub-tile (64 or 32); its columns are always 128.
+// WM = rows of a wave's sub-tile (64, 32 or 16); its columns are always 128.
 template <typename T, int BM, int BN, int WM, bool B_NK>
 struct Fp16Tile {
   static constexpr int MF      = WM / 16;  // 16-row fragments per wave
@@ -370,6 +370,7 @@ static hipError_t dispatch_fp16(int tile, const void* A, const void* B, void* C,
     case LLMMM_TILE_128x256: return launch_fp16<T, 128, 256, 32, B_NK>(A, B, C, M, N, K, stream);
     case LLMMM_TILE_256x128: return launch_fp16<T, 256, 128, 32, B_NK>(A, B, C, M, N, K, stream);
     case LLMMM_TILE_128x128: return launch_fp16<T, 128, 128, 32, B_NK>(A, B, C, M, N, K, stream);
+    case LLMMM_TILE_64x128: return launch_fp16<T, 64, 128, 16, B_NK>(A, B, C, M, N, K, stream);  // four 16-row waves: small problems
     default: return hipErrorInvalidValue;
   }
 }

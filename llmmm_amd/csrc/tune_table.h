@@ -49,7 +49,7 @@ static const TileTune kTileTune[] = {
 // FP16/BF16 MFMA tile kernels.
 static const TileTune kFp16TileTune[] = {
   {4096, 4096, 4096, 0, 1},
-  {1024, 1024, 1024, 3, 1},
+  {1024, 1024, 1024, 4, 1},
 };
 
 }  // namespace llmmm

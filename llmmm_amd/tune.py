@@ -128,7 +128,7 @@ def main():
                 tile_rows.append((M, N, K, tile, split))
             torch.cuda.empty_cache()
     skinny_rows.sort(key=lambda r: (r[1], r[2], r[0]))
-    fp16_rows = [(4096, 4096, 4096, _lib.TILE_256x256, 1), (1024, 1024, 1024, _lib.TILE_128x128, 1)]
+    fp16_rows = [(4096, 4096, 4096, _lib.TILE_256x256, 1), (1024, 1024, 1024, _lib.TILE_64x128, 1)]
     text = render_table(skinny_rows, tile_rows, fp16_rows)
     print(text)
     if args.write:

@@ -206,3 +206,11 @@ def test_rmsnorm_quant_validation_without_device():
     assert f(_lib.DTYPE_BF16, FAKE, FAKE, ctypes.c_float(float("nan")), FAKE, FAKE, 4, 128, None) == _lib.ERR_INVALID_ARGUMENT
     assert f(_lib.DTYPE_F16, FAKE, FAKE, eps, FAKE, FAKE, 0, 128, None) == _lib.ERR_INVALID_ARGUMENT
     assert f(_lib.DTYPE_F16, ctypes.c_void_p(0x1008), FAKE, eps, FAKE, FAKE, 4, 128, None) == _lib.ERR_INVALID_ARGUMENT
+
+
+def test_the_64x128_tile_is_fp16_only():
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    args = (FAKE, FAKE, FAKE, FAKE, FAKE, FAKE)
+    cfg = _lib.GemmCfg(_lib.TILE_64x128, 1, 0)
+    assert lib.llmmm_fp8_gemm_ex(2, *args, 256, 256, 256, None, 0, ctypes.byref(cfg), None) == _lib.ERR_INVALID_ARGUMENT

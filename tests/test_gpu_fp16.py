@@ -10,7 +10,7 @@ from helpers import assert_fp16_close, fp16_inputs_normal, fp16_inputs_uniform
 
 pytestmark = pytest.mark.gpu
 G = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-TILES = {"auto": -1, "256x256": 0, "128x256": 1, "256x128": 2, "128x128": 3}
+TILES = {"auto": -1, "256x256": 0, "128x256": 1, "256x128": 2, "128x128": 3, "64x128": 4}
 
 
 def _gpu(a):
@@ -32,7 +32,7 @@ def test_cfg1_1024_both_layouts_bit_identical(lib, oracle):
     assert (c_rm.view(np.uint16) == c_bt.view(np.uint16)).all(), "the two B layouts must give identical bits"
 
 
-@pytest.mark.parametrize("tile", ["256x256", "128x256", "256x128", "128x128"])
+@pytest.mark.parametrize("tile", ["256x256", "128x256", "256x128", "128x128", "64x128"])
 @pytest.mark.parametrize("bt", [False, True])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_every_tile_and_dtype(lib, oracle, tile, bt, dtype):
@@ -55,8 +55,9 @@ def test_k_tails_and_short_k(lib, oracle, K):
     B = rng.uniform(-1, 1, (K, 256)).astype(np.float16)
     ref = oracle.kahan_gemm(A.astype(np.float32), B.astype(np.float32))
     for bt in (False, True):
-        C = lib.fp16_gemm(_gpu(A), _gpu(B.T if bt else B), b_transposed=bt)
-        assert_fp16_close(C.cpu().numpy(), ref, "K=%d bt=%s" % (K, bt))
+        for tile in ("auto", "128x128", "64x128"):  # auto picks the 64 x 128 tile for a problem this small
+            C = lib.fp16_gemm(_gpu(A), _gpu(B.T if bt else B), b_transposed=bt, tile=TILES[tile])
+            assert_fp16_close(C.cpu().numpy(), ref, "K=%d bt=%s tile=%s" % (K, bt, tile))
 
 
 def test_golden_fixture(lib, oracle):
