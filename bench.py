@@ -12,7 +12,7 @@ fp32 accumulation, fp16 output, one kernel, no split-K); ``value`` is its TFLOP/
     region;
   * ``cpu_baseline``: the CPU oracle (a port of the reference's Kahan GEMM, test/kahan.cu:16-26)
     timed on this host's cores on a bounded sample of the same workload;
-  * ``shapes``: TFLOP/s (and GB/s for M <= 16) of the other BASELINE shapes, measured the same way.
+  * ``shapes``: TFLOP/s (and GB/s for M <= 16) of the other benchmark shapes, measured the same way.
 """
 import argparse
 import json
@@ -267,7 +267,7 @@ def main():
         roof = {"bound": "mfma", "achieved": r["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": r["tflops"] / peak, "traffic": None,
                 "kernel": "fp16_gemm_kernel<%s,256,256,row-major B>" % dtype}
         value, unit = r["tflops"], "TFLOP/s"
-        cfg = {"workload": "FP16 GEMM M=N=K=4096 (BASELINE configs[1]), A~N(0,1) B~N(0,0.02) seed 2, fp32 accumulate, %s out, "
+        cfg = {"workload": "FP16 GEMM M=N=K=4096 A~N(0,1) B~N(0,0.02) seed 2, fp32 accumulate, %s out, "
                            "single kernel, no split-K" % dtype, "M": M, "N": N, "K": K}
     elif w in ("fp8_gemm_fused_4096", "fp8_gemm_bf16_4096"):
         out = "fp8q" if "fused" in w else "bf16"

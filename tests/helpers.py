@@ -1,4 +1,4 @@
-"""Shared helpers of the test-suite: seeded inputs of the BASELINE configs and tolerance checks."""
+"""Shared helpers of the test-suite: seeded inputs of the benchmark configurations and tolerance checks."""
 import numpy as np
 
 

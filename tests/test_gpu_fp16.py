@@ -18,7 +18,7 @@ def _gpu(a):
 
 
 def test_cfg1_1024_both_layouts_bit_identical(lib, oracle):
-    # BASELINE configs[0]: M=N=K=1024, U(-1,1) seed 1, B row-major and transposed
+    # the small benchmark configuration: M=N=K=1024, U(-1,1) seed 1, B row-major and transposed
     A, B = fp16_inputs_uniform(1024, 1024, 1024, seed=1)
     ref = oracle.kahan_gemm(A.astype(np.float32), B.astype(np.float32))
     tA, tB = _gpu(A), _gpu(B)
@@ -96,7 +96,7 @@ def test_output_is_fully_overwritten_and_deterministic(lib):
 
 
 def test_cfg2_4096_slab_against_kahan_and_linearity(lib, oracle):
-    # BASELINE configs[1] at full size: A ~ N(0,1), B ~ N(0,0.02), seed 2.  The Kahan oracle checks a
+    # the headline configuration at full size: A ~ N(0,1), B ~ N(0,0.02), seed 2.  The Kahan oracle checks a
     # 256-row slab of the full product; a size-independent property covers the rest:
     # the rows of C only depend on the matching rows of A (row independence) -> compare with the GEMM of a
     # permuted A.

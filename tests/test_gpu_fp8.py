@@ -186,7 +186,7 @@ def test_split_k_is_deterministic_and_reusable(lib, oracle):
 @pytest.mark.parametrize("name,N,K", [("qkv", 6144, 2560), ("o", 2560, 4096), ("gate_up", 19456, 2560), ("down", 2560, 9728)])
 @pytest.mark.parametrize("M", [1, 16])
 def test_cfg5_decode_shapes(lib, oracle, name, N, K, M):
-    # BASELINE configs[4] at M in {1, 16}: full shapes, oracle on the whole (small-M) product
+    # the Qwen3-4B projection shapes at M in {1, 16}: full shapes, oracle on the whole (small-M) product
     Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=hash(name) % 1000)
     ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
     _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs), ref, "%s M=%d" % (name, M))

@@ -46,7 +46,7 @@ def test_transpose_equals_numpy(lib, oracle, M, N, dtype):
 
 
 def test_transpose_round_trip_full_size(lib):
-    """BASELINE-sized case through a size-independent property: transposing twice is the identity."""
+    """Full-size case through a size-independent property: transposing twice is the identity."""
     M, N = 4096, 19456
     x = torch.randint(0, 256, (M, N), dtype=torch.uint8, device="cuda")
     y = torch.empty((N, M), dtype=torch.uint8, device="cuda")

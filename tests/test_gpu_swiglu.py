@@ -82,7 +82,7 @@ def test_unsplit_and_split_paths_use_the_same_epilogue_arithmetic(lib, oracle):
 
 @pytest.mark.parametrize("M", [16, 128, 256])
 def test_qwen3_gate_up_auto_config(lib, oracle, M):
-    """BASELINE's gate_up shape (N = 19456 = 2 x 9728, K = 2560), library-chosen configuration, against the oracle."""
+    """The Qwen3-4B gate_up shape (N = 19456 = 2 x 9728, K = 2560), library-chosen configuration, against the oracle."""
     N, K = 19456, 2560
     Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=23)
     Bs = Bs.copy()
