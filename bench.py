@@ -212,6 +212,38 @@ def bench_mlp_chain(M, steps, warmup, hidden=2560, inter=9728, rotate_bytes=768 
             "launches": "rmsnorm+quant, gate_up+swiglu (+reduce), down (+reduce)"}
 
 
+def measured_peaks():
+    """What this GPU sustains, next to the nominal peaks: register-only MFMA loops (the counterpart of the reference's
+    test_fp8_peak_work, examples/005.fp8.test.cu:19-71) on zero and on random operands, and a streaming read."""
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    sink = torch.zeros(4, device="cuda")
+    out = {}
+    g = torch.Generator(device="cuda").manual_seed(5)
+    pats = {
+        "f16": (_lib.DTYPE_F16, torch.randn(16384, generator=g, device="cuda").to(torch.float16).view(torch.uint8)),
+        "bf16": (_lib.DTYPE_BF16, torch.randn(16384, generator=g, device="cuda").to(torch.bfloat16).view(torch.uint8)),
+        "fp8": (_lib.PROBE_FP8, (torch.randint(0, 0x78, (32768,), generator=g, device="cuda", dtype=torch.uint8)
+                                 | (torch.randint(0, 2, (32768,), generator=g, device="cuda", dtype=torch.uint8) << 7))),
+    }
+    wgs, iters = 1024, 2000
+    for name, (kind, rnd) in pats.items():
+        for label, ops in (("zero", torch.zeros(32768, dtype=torch.uint8, device="cuda")), ("random", rnd)):
+            def step():
+                assert lib.llmmm_probe_mfma(kind, ops.data_ptr(), sink.data_ptr(), wgs, iters, torch.cuda.current_stream().cuda_stream) == 0
+            ms, _ = _events_ms(step, 10, 2, graph=False)
+            out["mfma_%s_%s_operands_tflops" % (name, label)] = lib.llmmm_probe_mfma_flops(kind, wgs, iters) / ms * 1e-9
+    buf = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 255)
+
+    def read_step():
+        assert lib.llmmm_probe_hbm_read(buf.data_ptr(), buf.numel(), sink.data_ptr(), 2048, torch.cuda.current_stream().cuda_stream) == 0
+    ms, _ = _events_ms(read_step, 20, 3, graph=False)
+    out["hbm_read_1gib_gbs"] = buf.numel() / ms * 1e-6
+    out["note"] = ("register-only v_mfma loops, 1024 workgroups x 8 waves (16x16x32 f16/bf16, 16x16x128 fp8); zero operands run at the "
+                   "full clock, random operands at the power-limited one; hbm_read: 1 GiB read once, nothing written")
+    return out
+
+
 def cpu_baseline_fp16(M, N, K, rows):
     """Oracle Kahan GEMM on the first `rows` rows of the headline workload, all host threads."""
     import oracle
@@ -237,6 +269,7 @@ def main():
                          "decode_<qkv|o|gate_up|down>_m<M>[_pre] (_pre: weights pre-shuffled offline) | copy_1g (counter calibration only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table")
+    ap.add_argument("--no-peaks", action="store_true", help="skip the measured-peak probes")
     ap.add_argument("--cpu-rows", type=int, default=4096)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -363,6 +396,13 @@ def main():
             torch.cuda.empty_cache()
         line["shapes"] = shapes
 
+    if not args.no_peaks:
+        # the same kernel against what this very part sustains: random-operand MFMA rate / streaming read rate
+        mp = measured_peaks()
+        line["measured_peaks"] = mp
+        key = {"f16": "mfma_f16_random_operands_tflops", "bf16": "mfma_bf16_random_operands_tflops", "fp8": "mfma_fp8_random_operands_tflops"}[dtype]
+        roof["peak_measured"] = mp["hbm_read_1gib_gbs"] if roof["bound"] == "hbm" else mp[key]
+        roof["frac_of_measured"] = roof["achieved"] / roof["peak_measured"]
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_fp16(4096, 4096, 4096, args.cpu_rows)
     else:

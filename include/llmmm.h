@@ -157,6 +157,20 @@ LLMMM_API int llmmm_fp8_preshuffle_b(const void* Bt, void* Bp, int N, int K, voi
 LLMMM_API int llmmm_fp8_unshuffle_b(const void* Bp, void* Bt, int N, int K, void* stream);
 LLMMM_API int llmmm_transpose(int elem_size, const void* src, void* dst, int M, int N, void* stream);
 
+/* ---- peak-rate probes ---------------------------------------------------------------------
+ * What this very GPU sustains, next to the nominal peaks: the counterpart of the reference's register-only MMA
+ * loop test_fp8_peak_work(stream) (examples/005.fp8.test.cu:19-71).
+ * llmmm_probe_mfma enqueues `workgroups` x 8 wavefronts that issue v_mfma back to back from registers for `iters`
+ * iterations; kind: LLMMM_DTYPE_F16 / LLMMM_DTYPE_BF16 (16x16x32) or LLMMM_PROBE_FP8 (e4m3, 16x16x128).  `operands`
+ * = 32 KB of device memory whose bits become the operand fragments (the sustained rate depends on them: zeros run at
+ * full clock, random data draws more power); `sink` = one float of device memory, never written in practice.
+ * llmmm_probe_mfma_flops gives the FLOP of such a launch, so rate = flops / measured time.
+ * llmmm_probe_hbm_read reads `bytes` (a multiple of 16) once with `workgroups` x 512 threads and writes nothing. */
+#define LLMMM_PROBE_FP8 2
+LLMMM_API int    llmmm_probe_mfma(int kind, const void* operands, float* sink, int workgroups, int iters, void* stream);
+LLMMM_API double llmmm_probe_mfma_flops(int kind, int workgroups, int iters);
+LLMMM_API int    llmmm_probe_hbm_read(const void* src, size_t bytes, float* sink, int workgroups, void* stream);
+
 /* ---- misc ------------------------------------------------------------------------------- */
 LLMMM_API const char* llmmm_error_string(int code); /* the reference's exception texts for codes 1 and 2 */
 LLMMM_API const char* llmmm_last_error(void);       /* thread-local detail of the last failure */

@@ -20,6 +20,7 @@ B_ROW_MAJOR, B_TRANSPOSED = 0, 1
 OUT_F32, OUT_BF16, OUT_FP8Q, OUT_FP8Q_SWIGLU = 0, 1, 2, 3
 QUANT_1x128_T, QUANT_128x128, QUANT_1x128, QUANT_128x128_T = 0, 1, 2, 3
 FP8_B_ROWS, FP8_B_PRESHUFFLED = 0, 1
+PROBE_FP8 = 2
 TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_64x128, TILE_SKINNY = -1, 0, 1, 2, 3, 4, 8
 
 
@@ -42,6 +43,9 @@ SIGNATURES = {
     "llmmm_fp8_preshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
     "llmmm_fp8_unshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
     "llmmm_transpose": (_i, [_i, _vp, _vp, _i, _i, _vp]),
+    "llmmm_probe_mfma": (_i, [_i, _vp, _fp, _i, _i, _vp]),
+    "llmmm_probe_mfma_flops": (_c.c_double, [_i, _i, _i]),
+    "llmmm_probe_hbm_read": (_i, [_vp, _sz, _fp, _i, _vp]),
     "llmmm_error_string": (_c.c_char_p, [_i]),
     "llmmm_last_error": (_c.c_char_p, []),
     "llmmm_version": (_i, []),

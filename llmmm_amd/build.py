@@ -28,6 +28,7 @@ SOURCES = {
     "fp8_skinny.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "quant_fp8.hip": [],
     "layout.hip": [],
+    "probe.hip": [],
     "capi.cpp": ["-x", "hip"],
 }
 

@@ -361,6 +361,33 @@ int llmmm_rmsnorm_quant_fp8(int in_dtype, const void* x, const float* weight, fl
   return LLMMM_OK;
 }
 
+int llmmm_probe_mfma(int kind, const void* operands, float* sink, int workgroups, int iters, void* stream)
+{
+  if (kind < 0 || kind > LLMMM_PROBE_FP8) return fail(LLMMM_ERR_UNSUPPORTED_TYPE, "T is not supported.");
+  if (!operands || !sink) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (!aligned16(operands) || (reinterpret_cast<uintptr_t>(operands) & 31u)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "operands must be 32-byte aligned");
+  if (workgroups <= 0 || workgroups > 65536 || iters <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workgroups must be 1..65536 and iters positive");
+  const hipError_t e = llmmm::probe_mfma_launch(kind, operands, sink, workgroups, iters, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "probe launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
+double llmmm_probe_mfma_flops(int kind, int workgroups, int iters)
+{
+  if (kind < 0 || kind > LLMMM_PROBE_FP8 || workgroups <= 0 || iters <= 0) return 0.0;
+  return llmmm::probe_mfma_flops(kind, workgroups, iters);
+}
+
+int llmmm_probe_hbm_read(const void* src, size_t bytes, float* sink, int workgroups, void* stream)
+{
+  if (!src || !sink) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (!aligned16(src) || bytes == 0 || bytes % 16) return fail(LLMMM_ERR_INVALID_ARGUMENT, "src must be 16-byte aligned and bytes a positive multiple of 16");
+  if (workgroups <= 0 || workgroups > 65536) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workgroups must be 1..65536");
+  const hipError_t e = llmmm::probe_stream_read_launch(src, bytes, sink, workgroups, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "probe launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
 static int preshuffle(int inverse, const void* src, void* dst, int N, int K, void* stream)
 {
   if (N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "N and K must be positive (got %d, %d)", N, K);

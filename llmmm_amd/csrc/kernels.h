@@ -41,6 +41,11 @@ hipError_t quant_fp8_launch(int quant_m, int transpose, const float* x, void* q,
 hipError_t rmsnorm_quant_launch(int in_dtype, const void* x, const float* w, float eps, void* q, float* scale, int M, int K,
                                 hipStream_t stream);
 
+// Peak-rate probes (probe.hip).  kind: 0 = f16, 1 = bf16 (16x16x32), 2 = fp8 e4m3 (16x16x128); operands: 32 KB of operand bits.
+hipError_t probe_mfma_launch(int kind, const void* operands, float* sink, int workgroups, int iters, hipStream_t stream);
+double     probe_mfma_flops(int kind, int workgroups, int iters);
+hipError_t probe_stream_read_launch(const void* src, size_t bytes, float* sink, int workgroups, hipStream_t stream);
+
 hipError_t fill_u32_launch(uint32_t* p, uint32_t value, size_t n, hipStream_t stream);
 
 }  // namespace llmmm

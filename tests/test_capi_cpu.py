@@ -214,3 +214,20 @@ def test_the_64x128_tile_is_fp16_only():
     args = (FAKE, FAKE, FAKE, FAKE, FAKE, FAKE)
     cfg = _lib.GemmCfg(_lib.TILE_64x128, 1, 0)
     assert lib.llmmm_fp8_gemm_ex(2, *args, 256, 256, 256, None, 0, ctypes.byref(cfg), None) == _lib.ERR_INVALID_ARGUMENT
+
+
+def test_probe_validation_without_device():
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    a32 = ctypes.c_void_p(0x2000)
+    assert lib.llmmm_probe_mfma(5, a32, FAKE, 256, 10, None) == _lib.ERR_UNSUPPORTED_TYPE
+    assert lib.llmmm_probe_mfma(0, None, FAKE, 256, 10, None) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.llmmm_probe_mfma(0, ctypes.c_void_p(0x2010), FAKE, 256, 10, None) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.llmmm_probe_mfma(0, a32, FAKE, 0, 10, None) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.llmmm_probe_mfma(0, a32, FAKE, 256, 0, None) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.llmmm_probe_hbm_read(a32, 100, FAKE, 256, None) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.llmmm_probe_hbm_read(None, 1024, FAKE, 256, None) == _lib.ERR_INVALID_ARGUMENT
+    # FLOP of a launch: workgroups x 8 waves x iters x (16 MFMAs x 16384 | 8 MFMAs x 65536)
+    assert lib.llmmm_probe_mfma_flops(0, 256, 10) == 256 * 8 * 10 * 16 * 16384.0
+    assert lib.llmmm_probe_mfma_flops(_lib.PROBE_FP8, 256, 10) == 256 * 8 * 10 * 8 * 65536.0
+    assert lib.llmmm_probe_mfma_flops(9, 256, 10) == 0.0
