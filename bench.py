@@ -266,7 +266,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="fp16_gemm_4096",
                     help="fp16_gemm_4096 (headline) | fp8_gemm_fused_4096 | fp8_gemm_bf16_4096 | bf16_gemm_4096 | "
-                         "decode_<qkv|o|gate_up|down>_m<M>[_pre] (_pre: weights pre-shuffled offline) | copy_1g (counter calibration only)")
+                         "decode_<qkv|o|gate_up|down>_m<M>[_pre] (_pre: weights pre-shuffled offline) | prefill_<qkv|o|gate_up|down>_m<M> | "
+                         "prefill_gate_up_swiglu_m<M> | copy_1g (counter calibration only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measured-peak probes")
@@ -326,6 +327,21 @@ def main():
         value, unit = r["gbs"], "GB/s"
         cfg = {"workload": "Qwen3-4B %s projection, FP8 blockwise GEMM + fused C quant, M=%d N=%d K=%d, %s weights rotated over %d "
                            "copies" % (name, M, N, K, "pre-shuffled" if pre else "row-major", r["weight_copies"]), "M": M, "N": N, "K": K}
+    elif w.startswith("prefill_"):
+        import re
+        mo = re.fullmatch(r"prefill_(qkv|o|gate_up|down)(_swiglu)?_m(\d+)", w)
+        if not mo or (mo.group(2) and mo.group(1) != "gate_up"):
+            print("unknown workload", w, file=sys.stderr)
+            sys.exit(2)
+        name, M = mo.group(1), int(mo.group(3))
+        N, K = QWEN3_4B[name]
+        out = "swiglu" if mo.group(2) else "fp8q"
+        r = bench_fp8(M, N, K, out, args.steps, args.warmup)
+        dtype, peak = "fp8", PEAK_TFLOPS["fp8"]
+        roof = {"bound": "mfma", "achieved": r["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": r["tflops"] / peak, "traffic": None,
+                "kernel": "fp8_gemm_kernel tile %d split_k %d, output %s" % (r["tile"], r["split_k"], out)}
+        value, unit = r["tflops"], "TFLOP/s"
+        cfg = {"workload": "Qwen3-4B %s projection at M=%d (N=%d K=%d), FP8 blockwise GEMM, output %s" % (name, M, N, K, out), "M": M, "N": N, "K": K}
     else:
         print("unknown workload", w, file=sys.stderr)
         sys.exit(2)
