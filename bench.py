@@ -412,6 +412,18 @@ def main():
             torch.cuda.empty_cache()
         line["shapes"] = shapes
 
+    if not args.no_shapes:
+        # Side-by-side comparison only (never part of the product or of `value`): the vendor library behind torch.matmul
+        # (hipBLASLt) on the same FP16 inputs, timed the same way.
+        comp = {}
+        for (m, n, k) in ((4096, 4096, 4096), (1024, 1024, 1024)):
+            A, B = fp16_inputs(m, n, k)
+            C = torch.empty((m, n), dtype=torch.float16, device="cuda")
+            ms_, _ = _events_ms(lambda: torch.matmul(A, B, out=C), max(10, args.steps // 2), max(3, args.warmup // 2), graph=True)
+            comp["torch_matmul_fp16_%d_tflops" % m] = 2.0 * m * n * k / ms_ * 1e-9
+            comp["torch_matmul_fp16_%d_us" % m] = ms_ * 1e3
+        comp["note"] = "hipBLASLt via torch.matmul, same inputs and timing method; reported for comparison only"
+        line["comparison"] = comp
     if not args.no_peaks:
         # the same kernel against what this very part sustains: random-operand MFMA rate / streaming read rate
         mp = measured_peaks()
