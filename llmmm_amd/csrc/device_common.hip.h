@@ -123,9 +123,33 @@ __device__ __forceinline__ void tile_coords(int wg, int tiles_m, int tiles_n, in
   tn                    = in / gm;
 }
 
+// The value lane (l ^ mask) holds, for mask = 1, 2, 4, 8, 16 or 32 (a compile-time constant at every call site once
+// inlined).  No LDS address computation and, for 1, 2 and 32, no trip through the LDS crossbar at all:
+//   1, 2     DPP quad permutes (a VALU move),
+//   4 .. 16  ds_swizzle in bit-mask mode (xor inside each group of 32 lanes),
+//   32       v_permlane32_swap exchanges the upper 32 lanes of its first register with the lower 32 lanes of its second:
+//            from (v, v) it returns r[0] = the lower half of v in both halves, r[1] = the upper half in both halves.
+__device__ __forceinline__ float wave_xor_get(float v, int mask)
+{
+  const int iv = __builtin_bit_cast(int, v);
+  switch (mask) {
+    case 1: return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(iv, 0xB1, 0xf, 0xf, true));  // quad_perm [1,0,3,2]
+    case 2: return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(iv, 0x4E, 0xf, 0xf, true));  // quad_perm [2,3,0,1]
+    case 4: return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(iv, (4 << 10) | 0x1f));
+    case 8: return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(iv, (8 << 10) | 0x1f));
+    case 16: return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(iv, (16 << 10) | 0x1f));
+    case 32: {
+      const auto r = __builtin_amdgcn_permlane32_swap((unsigned)iv, (unsigned)iv, false, false);
+      // lanes 0..31 want the upper half (r[1]), lanes 32..63 the lower half (r[0])
+      return __builtin_bit_cast(float, (__lane_id() < 32) ? r[1] : r[0]);
+    }
+    default: return __shfl_xor(v, mask, 64);
+  }
+}
+
 __device__ __forceinline__ float wave_xor_max(float v, int mask)
 {
-  return fmaxf(v, __shfl_xor(v, mask, 64));
+  return fmaxf(v, wave_xor_get(v, mask));
 }
 
 }  // namespace llmmm

@@ -204,7 +204,7 @@ __global__ void __launch_bounds__(256) rmsnorm_quant_1x128_kernel(const IN_T* __
 #pragma unroll
   for (int step = 32; step >= 1; step >>= 1)
 #pragma unroll
-    for (int gidx = 0; gidx < 4; ++gidx) part[gidx] = part[gidx] + __shfl_xor(part[gidx], step, 64);
+    for (int gidx = 0; gidx < 4; ++gidx) part[gidx] = part[gidx] + wave_xor_get(part[gidx], step);
   const float acc = (part[0] + part[1]) + (part[2] + part[3]);
   const float ms  = acc / (float)K;
   const float r   = 1.0f / __builtin_sqrtf(ms + eps);
@@ -247,7 +247,7 @@ __global__ void __launch_bounds__(256) rmsnorm_quant_row_kernel(const IN_T* __re
       for (int e = 0; e < 4; ++e) acc = __builtin_fmaf(held[i][e], held[i][e], acc);
     }
 #pragma unroll
-  for (int step = 32; step >= 1; step >>= 1) acc = acc + __shfl_xor(acc, step, 64);
+  for (int step = 32; step >= 1; step >>= 1) acc = acc + wave_xor_get(acc, step);
   if ((t & 63) == 0) group_sum[t >> 6] = acc;
   __syncthreads();
   const float total = (group_sum[0] + group_sum[1]) + (group_sum[2] + group_sum[3]);
