@@ -212,6 +212,44 @@ def bench_mlp_chain(M, steps, warmup, hidden=2560, inter=9728, rotate_bytes=768 
             "launches": "rmsnorm+quant, gate_up+swiglu (+reduce), down (+reduce)"}
 
 
+def bench_proj_add_norm(name, M, steps, warmup, rotate_bytes=768 << 20):
+    """A projection back to the hidden size (o or down of Qwen3-4B) with the decoder block's epilogue: residual add, the next
+    RMSNorm and the 1x128 quantisation.  Timed fused (one entry point: GEMM into fp32 planes + one epilogue kernel) and as
+    separate launches (GEMM with bf16 output, torch add, rmsnorm+quant)."""
+    import llmmm_amd
+    N, K = QWEN3_4B[name]
+    copies = max(2, int(np.ceil(rotate_bytes / float(N * K)))) if M <= 128 else 1
+    Aq, As, weights = fp8_inputs(M, N, K, copies=copies)
+    weights = [(llmmm_amd.preshuffle_weight(bq), bs) for bq, bs in weights]
+    g = torch.Generator(device="cuda").manual_seed(5)
+    res = torch.randn((M, N), generator=g, device="cuda").to(torch.bfloat16)
+    hid = torch.empty_like(res)
+    Y = torch.empty_like(res)
+    wn = torch.ones(N, device="cuda")
+    ws = torch.empty(int(llmmm_amd._lib.lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K)), dtype=torch.uint8, device="cuda")
+    ws2 = llmmm_amd.make_workspace(llmmm_amd._lib.OUT_BF16, M, N, K)
+    state = {"i": 0}
+
+    def fused():
+        bq, bs = weights[state["i"] % copies]
+        state["i"] += 1
+        llmmm_amd.fp8_gemm_add_rmsnorm_quant(Aq, As, bq, bs, res, hid, wn, 1e-6, M, N, K, workspace=ws, b_preshuffled=True)
+
+    def separate():
+        bq, bs = weights[state["i"] % copies]
+        state["i"] += 1
+        llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(Aq, As, bq, bs, Y, M, N, K, workspace=ws2, b_preshuffled=True)
+        torch.add(Y, res, out=hid)
+        llmmm_amd.rmsnorm_quantize_activation(hid, wn, 1e-6)
+
+    ms_f, _ = _events_ms(fused, steps, warmup, graph=True)
+    ms_s, _ = _events_ms(separate, steps, warmup, graph=True)
+    nbytes = fp8_bytes(M, N, K, "fp8q") + 4.0 * M * N  # + residual in, hidden out (bf16 each)
+    return {"name": "qwen3_4b_%s_add_rmsnorm_quant_m%d" % (name, M), "M": M, "N": N, "K": K, "us": ms_f * 1e3, "us_separate_launches": ms_s * 1e3,
+            "hbm_gbs": nbytes / ms_f * 1e-6, "frac_of_hbm_peak": nbytes / ms_f * 1e-6 / PEAK_HBM_GBS, "tflops": 2.0 * M * N * K / ms_f * 1e-9,
+            "weight_copies": copies}
+
+
 def measured_peaks():
     """What this GPU sustains, next to the nominal peaks: register-only MFMA loops (the counterpart of the reference's
     test_fp8_peak_work, examples/005.fp8.test.cu:19-71) on zero and on random operands, and a streaming read."""
@@ -410,6 +448,11 @@ def main():
         for m in (1, 16):
             shapes.append(bench_mlp_chain(m, s2, w2))
             torch.cuda.empty_cache()
+        # o / down projection + residual add + next RMSNorm + quantisation in one entry point, beside the same work as separate launches
+        for name in ("o", "down"):
+            for m in (1, 16, 128, 2048):
+                shapes.append(bench_proj_add_norm(name, m, s2 * 2 if m <= 16 else s2, w2))
+                torch.cuda.empty_cache()
         line["shapes"] = shapes
 
     if not args.no_shapes:

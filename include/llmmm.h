@@ -138,6 +138,23 @@ LLMMM_API int llmmm_quant_fp8(int kind, const float* x, void* q, float* scale, i
 LLMMM_API int llmmm_rmsnorm_quant_fp8(int in_dtype, const void* x, const float* weight, float eps, void* q, float* scale, int M, int K,
                                       void* stream);
 
+/* Decoder-block epilogue fused behind a projection back to the hidden size (O, down) -- the "RMSNorm + fp8 dynamic
+ * quant fused into MM" of the reference's plan (README.md:16); no reference kernel.  With C32 = the fp32 result of the
+ * blockwise GEMM of llmmm_fp8_gemm (same operands, same layouts):
+ *   h          = C32 + residual                          (fp32; residual [M,N] of hidden_dtype)
+ *   hidden_out = hidden_dtype(h)                         (the new residual stream; may be the same buffer as residual)
+ *   q, q_scale = llmmm_rmsnorm_quant_fp8(hidden_out, norm_weight, eps)   -- bit for bit what the separate call gives
+ * so the next projection's A operand leaves this call, and neither the GEMM's result nor the normalised activations
+ * make a round trip of their own.  The GEMM always goes through fp32 planes in `workspace`
+ * (llmmm_fp8_gemm_add_rmsnorm_quant_workspace bytes; at least M * N * 4), which the fused kernel sums in split order.
+ * hidden_dtype: LLMMM_DTYPE_F32 / _BF16 / _F16.  N % 128 == 0, N <= 10240, K % 128 == 0, M as for llmmm_fp8_gemm.
+ * cfg may be NULL (library's choice of kernel and split). */
+LLMMM_API int    llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As, const void* Bt, const float* Bs, int hidden_dtype,
+                                                  const void* residual, void* hidden_out, const float* norm_weight, float eps, void* q,
+                                                  float* q_scale, int M, int N, int K, void* workspace, size_t workspace_bytes,
+                                                  const llmmm_gemm_cfg* cfg, void* stream);
+LLMMM_API size_t llmmm_fp8_gemm_add_rmsnorm_quant_workspace(int M, int N, int K);
+
 /* ---- offline layout helpers --------------------------------------------------------------
  * llmmm_fp8_preshuffle_b takes the role of  construct_m16n8k32_B_layout(dst, src_transposed, N, K,
  * stream)  (src/base/base.h:13, src/base/base.cu:222-271): a one-off permutation of the weights

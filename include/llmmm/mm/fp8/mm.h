@@ -102,4 +102,20 @@ inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output
                                          C_scale_transposed, M, N, K, nullptr, 0, (void*)stream));
 }
 
+// A projection back to the hidden size (O, down) with the decoder block's epilogue behind it -- residual add, the next
+// RMSNorm and the 1x128 quantisation (planned by the reference, README.md:16; no reference kernel):
+//   hidden_out = T(A @ B + residual);  q, q_scale = quantise<1,128,true>(rmsnorm(hidden_out) * norm_weight)
+// hidden_out may be the residual buffer.  workspace: llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K) bytes.
+template <typename T>
+void fp8_gemm_blockwise_quant_A_1x128__B_128x128__add_rmsnorm__output_fp8(const fp8_t* A, const float* A_scale_transposed, const fp8_t* B_transposed,
+                                                                          const float* B_scale_transposed, const T* residual, T* hidden_out,
+                                                                          const float* norm_weight, float eps, fp8_t* q, float* q_scale, int M, int N,
+                                                                          int K, void* workspace, size_t workspace_bytes, hipStream_t stream)
+{
+  constexpr int dtype = sizeof(T) == 4 ? LLMMM_DTYPE_F32 : (std::is_same<T, _Float16>::value || std::is_same<T, __half>::value) ? LLMMM_DTYPE_F16 : LLMMM_DTYPE_BF16;
+  static_assert(sizeof(T) == 4 || sizeof(T) == 2, "T must be float, half or bfloat16");
+  detail8::throw_on_error(llmmm_fp8_gemm_add_rmsnorm_quant(A, A_scale_transposed, B_transposed, B_scale_transposed, dtype, residual, hidden_out, norm_weight,
+                                                           eps, q, q_scale, M, N, K, workspace, workspace_bytes, nullptr, (void*)stream));
+}
+
 }  // namespace LLMMM

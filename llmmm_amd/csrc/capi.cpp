@@ -388,6 +388,69 @@ int llmmm_probe_hbm_read(const void* src, size_t bytes, float* sink, int workgro
   return LLMMM_OK;
 }
 
+size_t llmmm_fp8_gemm_add_rmsnorm_quant_workspace(int M, int N, int K)
+{
+  if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
+  llmmm_gemm_cfg cfg;
+  if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
+  return (size_t)(cfg.split_k < 1 ? 1 : cfg.split_k) * M * N * sizeof(float);
+}
+
+int llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As, const void* Bt, const float* Bs, int hidden_dtype, const void* residual,
+                                     void* hidden_out, const float* norm_weight, float eps, void* q, float* q_scale, int M, int N, int K,
+                                     void* workspace, size_t workspace_bytes, const llmmm_gemm_cfg* user, void* stream)
+{
+  if (hidden_dtype != LLMMM_DTYPE_F16 && hidden_dtype != LLMMM_DTYPE_BF16 && hidden_dtype != LLMMM_DTYPE_F32)
+    return fail(LLMMM_ERR_UNSUPPORTED_TYPE, "T is not supported.");
+  llmmm_gemm_cfg cfg;
+  const int      rc = choose_fp8(M, N, K, &cfg);
+  if (rc) return rc;
+  if (N > 10240) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the fused norm handles rows of at most 10240 columns (got %d)", N);
+  if (!A || !As || !Bt || !Bs || !residual || !hidden_out || !norm_weight || !q || !q_scale) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (!(eps >= 0.f)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "eps must be non-negative");
+  if (!aligned16(A) || !aligned16(Bt) || !aligned16(residual) || !aligned16(hidden_out) || !aligned16(norm_weight) || !aligned16(q))
+    return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+  if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
+    return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
+  if (user) {
+    if (user->tile != LLMMM_TILE_AUTO) cfg.tile = user->tile;
+    if (user->split_k > 0) cfg.split_k = user->split_k;
+    if (user->b_layout != LLMMM_FP8_B_ROWS && user->b_layout != LLMMM_FP8_B_PRESHUFFLED)
+      return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown B layout %d", user->b_layout);
+    cfg.b_layout = user->b_layout;
+  }
+  const size_t plane = (size_t)M * N * sizeof(float);
+  if (!workspace || workspace_bytes < plane) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, one fp32 plane needs %zu", workspace ? workspace_bytes : (size_t)0, plane);
+  if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+  int bm = 0, bn = 0;
+  const bool skinny = cfg.tile == LLMMM_TILE_SKINNY;
+  if (skinny) {
+    if (M > SKINNY_MAX_M) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the weight-streaming kernel handles M <= %d", SKINNY_MAX_M);
+  }
+  else {
+    if (!tile_dims(cfg.tile, bm, bn) || cfg.tile == LLMMM_TILE_64x128) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown tile id %d", cfg.tile);
+    if (M % bm || N % bn) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+    if (user && user->tile != LLMMM_TILE_AUTO && user->split_k <= 0) cfg.split_k = heuristic_tile_split(cfg.tile, M, N, K);
+  }
+  int split = cfg.split_k < 1 ? 1 : cfg.split_k;
+  const int cap = skinny ? max_split_for(K) : (K / 128 < MAX_SPLIT_K ? K / 128 : MAX_SPLIT_K);
+  if (split > cap) split = cap;
+  if ((size_t)split * plane > workspace_bytes) {
+    if (user && user->split_k > 0) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace_bytes, split, (size_t)split * plane);
+    split = (int)(workspace_bytes / plane);  // >= 1: checked above
+  }
+  float*     planes = (float*)workspace;
+  hipError_t e;
+  if (skinny)
+    e = llmmm::fp8_skinny_launch(LLMMM_OUT_F32, cfg.b_layout, A, As, Bt, Bs, nullptr, nullptr, M, N, K, split, planes, (hipStream_t)stream);
+  else
+    e = llmmm::fp8_gemm_launch(LLMMM_OUT_F32, cfg.tile, cfg.b_layout, A, As, Bt, Bs, nullptr, nullptr, M, N, K, split, planes, (hipStream_t)stream);
+  if (e == hipSuccess)
+    e = llmmm::planes_add_rmsnorm_quant_launch(hidden_dtype, planes, split, residual, hidden_out, norm_weight, eps, q, q_scale, M, N, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "fp8 gemm + add + rmsnorm launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
 static int preshuffle(int inverse, const void* src, void* dst, int N, int K, void* stream)
 {
   if (N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "N and K must be positive (got %d, %d)", N, K);

@@ -697,7 +697,7 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
   hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, S), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs,
                      (void*)planes, (float*)nullptr, M, N, K, tiles_m, tiles_n);
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
+  if (e != hipSuccess || C == nullptr) return e;  // C == nullptr: the caller consumes the planes itself
   return launch_reduce<OUT>(planes, S, C, Cs, M, N, stream);
 }
 

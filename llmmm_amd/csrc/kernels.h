@@ -16,7 +16,8 @@ hipError_t fp16_gemm_launch(int dtype, int b_layout, int tile, const void* A, co
 // out_kind: 0 = fp32, 1 = bf16, 2 = e4m3 codes + per-1x128 scales, 3 = SwiGLU (silu(C[:, :N/2]) * C[:, N/2:]) as codes + scales.  S > 1 splits K over S
 // workgroups per tile (S <= K/128): `planes` then holds S * M * N floats of partial sums, added
 // in split order by a second kernel that also runs the epilogue.  planes != nullptr with S == 1 takes the
-// same two-kernel route through one plane (the SwiGLU output from a 128-column tile).
+// same two-kernel route through one plane (the SwiGLU output from a 128-column tile).  C == nullptr (with planes): only
+// the planes are written, no reduce kernel is launched.
 // b_layout: LLMMM_FP8_B_ROWS (Bt[N,K] row-major) or LLMMM_FP8_B_PRESHUFFLED (the image fp8_preshuffle_launch writes).
 hipError_t fp8_gemm_launch(int out_kind, int tile, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs,
                            void* C, float* Cs, int M, int N, int K, int S, float* planes, hipStream_t stream);
@@ -45,6 +46,11 @@ hipError_t rmsnorm_quant_launch(int in_dtype, const void* x, const float* w, flo
 hipError_t probe_mfma_launch(int kind, const void* operands, float* sink, int workgroups, int iters, hipStream_t stream);
 double     probe_mfma_flops(int kind, int workgroups, int iters);
 hipError_t probe_stream_read_launch(const void* src, size_t bytes, float* sink, int workgroups, hipStream_t stream);
+
+// hidden = T(sum of S planes [S][M][N] + residual); q, scale = quant_1x128_T(RMSNorm(hidden) * w).  N % 128 == 0, N <= 10240;
+// residual and hidden may be the same buffer.
+hipError_t planes_add_rmsnorm_quant_launch(int hidden_dtype, const float* planes, int S, const void* residual, void* hidden, const float* w,
+                                           float eps, void* q, float* scale, int M, int N, hipStream_t stream);
 
 hipError_t fill_u32_launch(uint32_t* p, uint32_t value, size_t n, hipStream_t stream);
 

@@ -277,6 +277,149 @@ __global__ void __launch_bounds__(256) rmsnorm_quant_row_kernel(const IN_T* __re
   }
 }
 
+// The decoder-block epilogue behind a projection back to the hidden size (O, down), in one kernel behind the GEMM's
+// fp32 planes:  h = (plane 0 + plane 1 + ... in split order) + residual,  hidden = T(h) (the new residual stream),
+// y = RMSNorm(float(hidden)) * weight,  q, s = quant_1x128(y) -- the A operand of the next projection.  It takes the
+// place of the split-K reduce kernel and of the separate RMSNorm + quantiser launch; the norm sees the rounded hidden
+// state, exactly what a separate kernel reading `hidden` would see, and follows the same fixed summation order
+// (rmsnorm_quant_row_kernel), so its codes and scales are those of the unfused sequence, bit for bit.
+// One 256-thread workgroup per row; N <= 1024 * NI columns.
+template <typename T>
+__device__ __forceinline__ void store_row4(T* p, f32x4 v);
+template <>
+__device__ __forceinline__ void store_row4<float>(float* p, f32x4 v)
+{
+  *(f32x4*)p = v;
+}
+template <>
+__device__ __forceinline__ void store_row4<__bf16>(__bf16* p, f32x4 v)
+{
+  typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+  *(bf16x4*)p = bf16x4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+}
+template <>
+__device__ __forceinline__ void store_row4<_Float16>(_Float16* p, f32x4 v)
+{
+  *(f16x4*)p = f16x4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+}
+
+template <typename T, int NI>
+__global__ void __launch_bounds__(256) planes_add_rmsnorm_quant_kernel(const float* __restrict__ planes, int S, const T* residual, T* hidden,
+                                                                       const float* __restrict__ w, float eps, uint8_t* __restrict__ q,
+                                                                       float* __restrict__ scale, int M, int N)
+{
+  __shared__ float group_sum[4];
+  const int    t      = threadIdx.x;
+  const int    m      = blockIdx.x;
+  const int    chunks = N >> 2;
+  const size_t plane  = (size_t)M * N;
+  f32x4        held[NI], wv[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    held[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    wv[i]   = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  // Everything that does not depend on the planes is requested first; then the planes, W of them in flight per chunk,
+  // summed in split order (0 + p0 + p1 + ...: the order of the split-K reduce kernel).  Threads past the end of the
+  // row load its last chunk and drop it.
+  f32x4 rv[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int c = min(t + 256 * i, chunks - 1);
+    rv[i]       = load_row4<T>(residual + (size_t)m * N + 4 * c);
+    wv[i]       = *(const f32x4*)(w + 4 * c);
+  }
+  constexpr int W = NI <= 3 ? 8 : 2;
+  for (int s0 = 0; s0 < S; s0 += W) {
+    f32x4 p[W][NI];
+#pragma unroll
+    for (int u = 0; u < W; ++u)
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int c = min(t + 256 * i, chunks - 1);
+        p[u][i]     = __builtin_nontemporal_load((const f32x4*)(planes + (size_t)min(s0 + u, S - 1) * plane + (size_t)m * N + 4 * c));
+      }
+#pragma unroll
+    for (int u = 0; u < W; ++u)
+      if (s0 + u < S) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) held[i] += p[u][i];
+      }
+  }
+  float acc = 0.f;
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int c = t + 256 * i;
+    if (c < chunks) {
+      const f32x4 h = held[i] + rv[i];
+      store_row4<T>(hidden + (size_t)m * N + 4 * c, h);
+      // the norm reads the hidden state as stored (rounded to T)
+      if constexpr (sizeof(T) == 4)
+        held[i] = h;
+      else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) held[i][e] = (float)(T)h[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc = __builtin_fmaf(held[i][e], held[i][e], acc);
+    }
+    else
+      held[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+#pragma unroll
+  for (int step = 32; step >= 1; step >>= 1) acc = acc + wave_xor_get(acc, step);
+  if ((t & 63) == 0) group_sum[t >> 6] = acc;
+  __syncthreads();
+  const float total = (group_sum[0] + group_sum[1]) + (group_sum[2] + group_sum[3]);
+  const float ms    = total / (float)N;
+  const float r     = 1.0f / __builtin_sqrtf(ms + eps);
+  float       amax[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) held[i][e] = (held[i][e] * r) * wv[i][e];
+    amax[i] = amax4(0.f, held[i]);
+  }
+#pragma unroll
+  for (int step = 1; step <= 16; step <<= 1)
+#pragma unroll
+    for (int i = 0; i < NI; ++i) amax[i] = wave_xor_max(amax[i], step);
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int   c  = t + 256 * i;
+    const float sc = amax[i] / 448.f;
+    uint32_t    cd = 0;
+    if (sc != 0.f) cd = q_pack_e4m3x4(held[i][0] / sc, held[i][1] / sc, held[i][2] / sc, held[i][3] / sc);
+    if (c < chunks) {
+      *(uint32_t*)(q + (size_t)m * N + 4 * c) = cd;
+      if ((t & 31) == 0) scale[(size_t)(c >> 5) * M + m] = sc;
+    }
+  }
+}
+
+hipError_t planes_add_rmsnorm_quant_launch(int hidden_dtype, const float* planes, int S, const void* residual, void* hidden, const float* w,
+                                           float eps, void* q, float* scale, int M, int N, hipStream_t stream)
+{
+#define LLMMM_GO(T)                                                                                                                        \
+  {                                                                                                                                        \
+    if (N <= 1024 * 3)                                                                                                                     \
+      hipLaunchKernelGGL((planes_add_rmsnorm_quant_kernel<T, 3>), dim3(M), dim3(256), 0, stream, planes, S, (const T*)residual, (T*)hidden, \
+                         w, eps, (uint8_t*)q, scale, M, N);                                                                                \
+    else                                                                                                                                   \
+      hipLaunchKernelGGL((planes_add_rmsnorm_quant_kernel<T, 10>), dim3(M), dim3(256), 0, stream, planes, S, (const T*)residual,           \
+                         (T*)hidden, w, eps, (uint8_t*)q, scale, M, N);                                                                    \
+  }
+  if (N > 1024 * 10) return hipErrorInvalidValue;
+  switch (hidden_dtype) {
+    case LLMMM_DTYPE_F16: LLMMM_GO(_Float16) break;
+    case LLMMM_DTYPE_BF16: LLMMM_GO(__bf16) break;
+    case LLMMM_DTYPE_F32: LLMMM_GO(float) break;
+    default: return hipErrorInvalidValue;
+  }
+#undef LLMMM_GO
+  return hipGetLastError();
+}
+
 hipError_t rmsnorm_quant_launch(int in_dtype, const void* x, const float* w, float eps, void* q, float* scale, int M, int K,
                                 hipStream_t stream)
 {

@@ -195,6 +195,31 @@ def fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(A, 
               tile, split_k, stream, b_preshuffled)
 
 
+def fp8_gemm_add_rmsnorm_quant(A, A_scale_transposed, B_transposed, B_scale_transposed, residual, hidden_out, norm_weight, eps, M, N, K,
+                               stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0, b_preshuffled=False):
+    """A projection back to the hidden size (O, down) with the decoder block's epilogue behind it (the fusion the reference
+    plans, README.md:16): ``hidden_out = residual + A @ B`` (stored in the residual's dtype; may be the same tensor), then
+    RMSNorm(hidden_out) * norm_weight quantised 1x128 with transposed scales.  Returns (codes uint8 [M,N], scales float32
+    [N/128, M]): the A operand of the next projection, bit-identical to ``rmsnorm_quantize_activation(hidden_out, ...)``."""
+    code = {torch.float32: _lib.DTYPE_F32, torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16}.get(residual.dtype)
+    if code is None or hidden_out.dtype != residual.dtype:
+        raise RuntimeError("T is not supported.")
+    kb = K // 128 if K % 128 == 0 else 0
+    if workspace is None:
+        n = int(lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K))
+        workspace = torch.empty(max(n, 16), dtype=torch.uint8, device=residual.device)
+    q = torch.empty((M, N), dtype=torch.uint8, device=residual.device)
+    s = torch.empty(((N + 127) // 128, M), dtype=torch.float32, device=residual.device)
+    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS)
+    check(lib.llmmm_fp8_gemm_add_rmsnorm_quant(
+        _ptr(A, "A", _FP8_DTYPES, M * K), _ptr(A_scale_transposed, "A_scale_transposed", (torch.float32,), kb * M),
+        _ptr(B_transposed, "B_transposed", _FP8_DTYPES, N * K), _ptr(B_scale_transposed, "B_scale_transposed", (torch.float32,), ((N + 127) // 128) * kb),
+        code, _ptr(residual, "residual", numel=M * N), _ptr(hidden_out, "hidden_out", numel=M * N), _ptr(norm_weight, "norm_weight", (torch.float32,), N),
+        ctypes.c_float(eps), _ptr(q, "q"), _ptr(s, "q_scale"), M, N, K, ctypes.c_void_p(workspace.data_ptr()),
+        workspace.numel() * workspace.element_size(), ctypes.byref(cfg), _stream(stream)))
+    return q, s
+
+
 # ------------------------------------------------------------------------------------- offline layout helpers
 def construct_mfma_B_layout(dst, src_transposed, N, K, stream=None):
     """The role of ``LLMMM::construct_m16n8k32_B_layout(dst, src_transposed, N, K, stream)``
