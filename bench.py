@@ -250,6 +250,43 @@ def bench_proj_add_norm(name, M, steps, warmup, rotate_bytes=768 << 20):
             "weight_copies": copies}
 
 
+def bench_qkv_rope(M, steps, warmup, rotate_bytes=768 << 20):
+    """The Qwen3-4B QKV projection (32 query, 8 key/value heads of 128) with per-head RMSNorm and RoPE fused behind it, bf16
+    output, beside the plain bf16-output GEMM of the same shape (which still needs a norm + rope kernel after it)."""
+    import llmmm_amd
+    N, K = QWEN3_4B["qkv"]
+    n_q, n_kv = 32, 8
+    copies = max(2, int(np.ceil(rotate_bytes / float(N * K)))) if M <= 128 else 1
+    Aq, As, weights = fp8_inputs(M, N, K, copies=copies)
+    weights = [(llmmm_amd.preshuffle_weight(bq), bs) for bq, bs in weights]
+    w = torch.ones(128, device="cuda")
+    inv = 1e6 ** (-torch.arange(64, device="cuda", dtype=torch.float64) / 64)
+    ang = torch.arange(4096, device="cuda", dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang).float().contiguous(), torch.sin(ang).float().contiguous()
+    pos = torch.arange(M, device="cuda", dtype=torch.int32)
+    ws = torch.empty(max(16, int(llmmm_amd._lib.lib.llmmm_fp8_gemm_qkv_rope_workspace(M, N, K))), dtype=torch.uint8, device="cuda")
+    ws2 = llmmm_amd.make_workspace(llmmm_amd._lib.OUT_BF16, M, N, K)
+    Y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    state = {"i": 0}
+
+    def fused():
+        bq, bs = weights[state["i"] % copies]
+        state["i"] += 1
+        llmmm_amd.fp8_gemm_qkv_rope(Aq, As, bq, bs, w, w, 1e-6, cos, sin, pos, n_q, n_kv, M, N, K, workspace=ws, b_preshuffled=True)
+
+    def plain():
+        bq, bs = weights[state["i"] % copies]
+        state["i"] += 1
+        llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(Aq, As, bq, bs, Y, M, N, K, workspace=ws2, b_preshuffled=True)
+
+    ms_f, _ = _events_ms(fused, steps, warmup, graph=True)
+    ms_p, _ = _events_ms(plain, steps, warmup, graph=True)
+    nbytes = fp8_bytes(M, N, K, "bf16")
+    return {"name": "qwen3_4b_qkv_norm_rope_m%d" % M, "M": M, "N": N, "K": K, "us": ms_f * 1e3, "us_plain_bf16_gemm": ms_p * 1e3,
+            "hbm_gbs": nbytes / ms_f * 1e-6, "frac_of_hbm_peak": nbytes / ms_f * 1e-6 / PEAK_HBM_GBS, "tflops": 2.0 * M * N * K / ms_f * 1e-9,
+            "weight_copies": copies}
+
+
 def measured_peaks():
     """What this GPU sustains, next to the nominal peaks: register-only MFMA loops (the counterpart of the reference's
     test_fp8_peak_work, examples/005.fp8.test.cu:19-71) on zero and on random operands, and a streaming read."""
@@ -453,6 +490,10 @@ def main():
             for m in (1, 16, 128, 2048):
                 shapes.append(bench_proj_add_norm(name, m, s2 * 2 if m <= 16 else s2, w2))
                 torch.cuda.empty_cache()
+        # QKV projection + per-head RMSNorm + RoPE in one entry point, beside the plain bf16-output GEMM
+        for m in (1, 16, 128, 2048):
+            shapes.append(bench_qkv_rope(m, s2 * 2 if m <= 16 else s2, w2))
+            torch.cuda.empty_cache()
         line["shapes"] = shapes
 
     if not args.no_shapes:

@@ -155,6 +155,30 @@ LLMMM_API int    llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As
                                                   const llmmm_gemm_cfg* cfg, void* stream);
 LLMMM_API size_t llmmm_fp8_gemm_add_rmsnorm_quant_workspace(int M, int N, int K);
 
+/* The QKV projection with what stands between it and attention fused behind it -- per-head RMSNorm (the q_norm / k_norm
+ * of Qwen3) and rotary position embedding; "RMSNorm, RoPE fused into MM" is on the reference's plan (README.md:16), no
+ * reference kernel.  Heads are 128 columns wide: columns [0, n_q_heads*128) are query heads, the next n_kv_heads*128 key
+ * heads, the last n_kv_heads*128 value heads; N = (n_q_heads + 2 n_kv_heads) * 128.  With C32 the fp32 GEMM result:
+ *   query / key head x (128 values of row m):
+ *     x <- x / sqrt(mean(x^2) + eps) * w          w = q_norm_weight / k_norm_weight [128]; skipped when that pointer is NULL
+ *     p  = clamp(positions[m], 0, table_rows-1)   positions [M] int32; cos_table / sin_table [table_rows, 64] fp32
+ *     y[i]    = x[i]    * cos[p,i] - x[i+64] * sin[p,i]        (rotate-half pairing, i < 64)
+ *     y[i+64] = x[i+64] * cos[p,i] + x[i]    * sin[p,i]
+ *   value heads: y = x.
+ * out_kind LLMMM_OUT_BF16: out [M,N] bf16.  LLMMM_OUT_FP8Q: out [M,N] e4m3 and out_scale [N/128, M] -- one scale per row
+ * and head (the 1x128 rule of the fused C quantisation), for an FP8 attention.
+ * Small M (the weight-streaming kernel) and split-K runs go through fp32 planes in `workspace`
+ * (llmmm_fp8_gemm_qkv_rope_workspace bytes), where the second kernel takes the place of the split-K reduce kernel, so norm
+ * and rope cost no launch of their own; an unsplit tile kernel applies them to its accumulators and needs no workspace
+ * (the query function then returns 0).  Both routes perform the same operations in the same order: the results agree
+ * bit for bit with each other for equal fp32 sums. */
+LLMMM_API int    llmmm_fp8_gemm_qkv_rope(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* out,
+                                         float* out_scale, const float* q_norm_weight, const float* k_norm_weight, float eps,
+                                         const float* cos_table, const float* sin_table, int table_rows, const int* positions,
+                                         int n_q_heads, int n_kv_heads, int M, int N, int K, void* workspace, size_t workspace_bytes,
+                                         const llmmm_gemm_cfg* cfg, void* stream);
+LLMMM_API size_t llmmm_fp8_gemm_qkv_rope_workspace(int M, int N, int K);
+
 /* ---- offline layout helpers --------------------------------------------------------------
  * llmmm_fp8_preshuffle_b takes the role of  construct_m16n8k32_B_layout(dst, src_transposed, N, K,
  * stream)  (src/base/base.h:13, src/base/base.cu:222-271): a one-off permutation of the weights

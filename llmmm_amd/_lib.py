@@ -43,6 +43,9 @@ SIGNATURES = {
     "llmmm_fp8_gemm_add_rmsnorm_quant": (_i, [_vp, _fp, _vp, _fp, _i, _vp, _vp, _fp, _c.c_float, _vp, _fp, _i, _i, _i, _vp, _sz,
                                               _c.POINTER(GemmCfg), _vp]),
     "llmmm_fp8_gemm_add_rmsnorm_quant_workspace": (_sz, [_i, _i, _i]),
+    "llmmm_fp8_gemm_qkv_rope": (_i, [_i, _vp, _fp, _vp, _fp, _vp, _fp, _fp, _fp, _c.c_float, _fp, _fp, _i, _vp, _i, _i, _i, _i, _i, _vp, _sz,
+                                     _c.POINTER(GemmCfg), _vp]),
+    "llmmm_fp8_gemm_qkv_rope_workspace": (_sz, [_i, _i, _i]),
     "llmmm_fp8_preshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
     "llmmm_fp8_unshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
     "llmmm_transpose": (_i, [_i, _vp, _vp, _i, _i, _vp]),

@@ -396,20 +396,22 @@ size_t llmmm_fp8_gemm_add_rmsnorm_quant_workspace(int M, int N, int K)
   return (size_t)(cfg.split_k < 1 ? 1 : cfg.split_k) * M * N * sizeof(float);
 }
 
-int llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As, const void* Bt, const float* Bs, int hidden_dtype, const void* residual,
-                                     void* hidden_out, const float* norm_weight, float eps, void* q, float* q_scale, int M, int N, int K,
-                                     void* workspace, size_t workspace_bytes, const llmmm_gemm_cfg* user, void* stream)
+// Kernel and split for the entry points whose epilogue lives in a second kernel behind fp32 planes, chosen and
+// validated as llmmm_fp8_gemm_ex does.  split == 0 on return: a tile kernel without split, which `allow_direct`
+// callers run with the epilogue inside the kernel (no planes, no workspace); otherwise split >= 1 planes are needed
+// and the workspace has been checked to hold them.
+struct PlaneCfg {
+  int  tile = 0, split = 0, b_layout = 0;
+  bool skinny = false;
+};
+static int resolve_plane_cfg(const void* A, const float* As, const void* Bt, const float* Bs, int M, int N, int K, void* workspace,
+                             size_t workspace_bytes, const llmmm_gemm_cfg* user, bool allow_direct, PlaneCfg* out)
 {
-  if (hidden_dtype != LLMMM_DTYPE_F16 && hidden_dtype != LLMMM_DTYPE_BF16 && hidden_dtype != LLMMM_DTYPE_F32)
-    return fail(LLMMM_ERR_UNSUPPORTED_TYPE, "T is not supported.");
   llmmm_gemm_cfg cfg;
   const int      rc = choose_fp8(M, N, K, &cfg);
   if (rc) return rc;
-  if (N > 10240) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the fused norm handles rows of at most 10240 columns (got %d)", N);
-  if (!A || !As || !Bt || !Bs || !residual || !hidden_out || !norm_weight || !q || !q_scale) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
-  if (!(eps >= 0.f)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "eps must be non-negative");
-  if (!aligned16(A) || !aligned16(Bt) || !aligned16(residual) || !aligned16(hidden_out) || !aligned16(norm_weight) || !aligned16(q))
-    return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+  if (!A || !As || !Bt || !Bs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (!aligned16(A) || !aligned16(Bt)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
   if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
   if (user) {
@@ -419,9 +421,6 @@ int llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As, const void*
       return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown B layout %d", user->b_layout);
     cfg.b_layout = user->b_layout;
   }
-  const size_t plane = (size_t)M * N * sizeof(float);
-  if (!workspace || workspace_bytes < plane) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, one fp32 plane needs %zu", workspace ? workspace_bytes : (size_t)0, plane);
-  if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
   int bm = 0, bn = 0;
   const bool skinny = cfg.tile == LLMMM_TILE_SKINNY;
   if (skinny) {
@@ -433,21 +432,105 @@ int llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As, const void*
     if (user && user->tile != LLMMM_TILE_AUTO && user->split_k <= 0) cfg.split_k = heuristic_tile_split(cfg.tile, M, N, K);
   }
   int split = cfg.split_k < 1 ? 1 : cfg.split_k;
-  const int cap = skinny ? max_split_for(K) : (K / 128 < MAX_SPLIT_K ? K / 128 : MAX_SPLIT_K);
-  if (split > cap) split = cap;
-  if ((size_t)split * plane > workspace_bytes) {
-    if (user && user->split_k > 0) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace_bytes, split, (size_t)split * plane);
-    split = (int)(workspace_bytes / plane);  // >= 1: checked above
+  if (split > max_split_for(K)) split = max_split_for(K);
+  const size_t plane    = (size_t)M * N * sizeof(float);
+  const bool   explicit_split = user && user->split_k > 0;
+  out->tile = cfg.tile, out->b_layout = cfg.b_layout, out->skinny = skinny;
+  if (allow_direct && !skinny && (split == 1 || (!explicit_split && (!workspace || workspace_bytes < 2 * plane)))) {
+    out->split = 0;  // also when a split the library chose itself finds no room for two planes
+    return LLMMM_OK;
   }
+  if (!workspace || workspace_bytes < plane) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, one fp32 plane needs %zu", workspace ? workspace_bytes : (size_t)0, plane);
+  if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+  if ((size_t)split * plane > workspace_bytes) {
+    if (explicit_split) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace_bytes, split, (size_t)split * plane);
+    split = (int)(workspace_bytes / plane);  // a split the library chose itself shrinks to the workspace (>= 1: checked above)
+  }
+  out->split = split;
+  return LLMMM_OK;
+}
+
+static int launch_into_planes(const PlaneCfg& pc, const void* A, const float* As, const void* Bt, const float* Bs, int M, int N, int K,
+                              void* workspace, void* stream)
+{
   float*     planes = (float*)workspace;
   hipError_t e;
-  if (skinny)
-    e = llmmm::fp8_skinny_launch(LLMMM_OUT_F32, cfg.b_layout, A, As, Bt, Bs, nullptr, nullptr, M, N, K, split, planes, (hipStream_t)stream);
+  if (pc.skinny)
+    e = llmmm::fp8_skinny_launch(LLMMM_OUT_F32, pc.b_layout, A, As, Bt, Bs, nullptr, nullptr, M, N, K, pc.split, planes, (hipStream_t)stream);
   else
-    e = llmmm::fp8_gemm_launch(LLMMM_OUT_F32, cfg.tile, cfg.b_layout, A, As, Bt, Bs, nullptr, nullptr, M, N, K, split, planes, (hipStream_t)stream);
-  if (e == hipSuccess)
-    e = llmmm::planes_add_rmsnorm_quant_launch(hidden_dtype, planes, split, residual, hidden_out, norm_weight, eps, q, q_scale, M, N, (hipStream_t)stream);
-  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "fp8 gemm + add + rmsnorm launch: %s", hipGetErrorString(e));
+    e = llmmm::fp8_gemm_launch(LLMMM_OUT_F32, pc.tile, pc.b_layout, A, As, Bt, Bs, nullptr, nullptr, M, N, K, pc.split, planes, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "fp8 gemm launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
+int llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As, const void* Bt, const float* Bs, int hidden_dtype, const void* residual,
+                                     void* hidden_out, const float* norm_weight, float eps, void* q, float* q_scale, int M, int N, int K,
+                                     void* workspace, size_t workspace_bytes, const llmmm_gemm_cfg* user, void* stream)
+{
+  if (hidden_dtype != LLMMM_DTYPE_F16 && hidden_dtype != LLMMM_DTYPE_BF16 && hidden_dtype != LLMMM_DTYPE_F32)
+    return fail(LLMMM_ERR_UNSUPPORTED_TYPE, "T is not supported.");
+  llmmm_gemm_cfg probe;
+  const int      rc0 = choose_fp8(M, N, K, &probe);  // shape checks first, with the reference's texts
+  if (rc0) return rc0;
+  if (N > 10240) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the fused norm handles rows of at most 10240 columns (got %d)", N);
+  if (!residual || !hidden_out || !norm_weight || !q || !q_scale) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (!(eps >= 0.f)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "eps must be non-negative");
+  if (!aligned16(residual) || !aligned16(hidden_out) || !aligned16(norm_weight) || !aligned16(q))
+    return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+  PlaneCfg pc;
+  int      rc = resolve_plane_cfg(A, As, Bt, Bs, M, N, K, workspace, workspace_bytes, user, false, &pc);
+  if (rc) return rc;
+  rc = launch_into_planes(pc, A, As, Bt, Bs, M, N, K, workspace, stream);
+  if (rc) return rc;
+  const hipError_t e = llmmm::planes_add_rmsnorm_quant_launch(hidden_dtype, (const float*)workspace, pc.split, residual, hidden_out, norm_weight, eps, q,
+                                                              q_scale, M, N, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "add + rmsnorm + quantiser launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
+size_t llmmm_fp8_gemm_qkv_rope_workspace(int M, int N, int K)
+{
+  if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
+  llmmm_gemm_cfg cfg;
+  if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
+  if (cfg.tile != LLMMM_TILE_SKINNY && cfg.split_k <= 1) return 0;  // epilogue inside the tile kernel
+  return (size_t)(cfg.split_k < 1 ? 1 : cfg.split_k) * M * N * sizeof(float);
+}
+
+int llmmm_fp8_gemm_qkv_rope(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* out, float* out_scale,
+                            const float* q_norm_weight, const float* k_norm_weight, float eps, const float* cos_table, const float* sin_table,
+                            int table_rows, const int* positions, int n_q_heads, int n_kv_heads, int M, int N, int K, void* workspace,
+                            size_t workspace_bytes, const llmmm_gemm_cfg* user, void* stream)
+{
+  if (out_kind != LLMMM_OUT_BF16 && out_kind != LLMMM_OUT_FP8Q) return fail(LLMMM_ERR_INVALID_ARGUMENT, "output kind %d: bf16 or fp8 (1x128) only", out_kind);
+  llmmm_gemm_cfg probe;
+  const int      rc0 = choose_fp8(M, N, K, &probe);
+  if (rc0) return rc0;
+  if (n_q_heads < 1 || n_kv_heads < 1 || (long)(n_q_heads + 2L * n_kv_heads) * 128 != N)
+    return fail(LLMMM_ERR_INVALID_ARGUMENT, "N = %d is not (n_q_heads + 2 n_kv_heads) * 128 with %d query and %d key/value heads", N, n_q_heads, n_kv_heads);
+  if (!out || !cos_table || !sin_table || !positions) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (out_kind == LLMMM_OUT_FP8Q && !out_scale) return fail(LLMMM_ERR_INVALID_ARGUMENT, "out_scale is required for fp8 output");
+  if (table_rows < 1) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the cos / sin tables need at least one row");
+  if (!(eps >= 0.f)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "eps must be non-negative");
+  if (!aligned16(out) || !aligned16(cos_table) || !aligned16(sin_table) || (q_norm_weight && !aligned16(q_norm_weight)) ||
+      (k_norm_weight && !aligned16(k_norm_weight)) || (reinterpret_cast<uintptr_t>(positions) & 3u))
+    return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned (positions: 4-byte)");
+  PlaneCfg pc;
+  int      rc = resolve_plane_cfg(A, As, Bt, Bs, M, N, K, workspace, workspace_bytes, user, true, &pc);
+  if (rc) return rc;
+  if (pc.split == 0) {  // a tile kernel without split: norm and rope run on the accumulators, no planes
+    llmmm::Fp8HeadOp op;
+    op.qw = q_norm_weight, op.kw = k_norm_weight, op.cos_t = cos_table, op.sin_t = sin_table, op.pos = positions;
+    op.eps = eps, op.table_rows = table_rows, op.n_q = n_q_heads, op.n_kv = n_kv_heads;
+    const hipError_t e = llmmm::fp8_gemm_qk_rope_launch(out_kind, pc.tile, pc.b_layout, A, As, Bt, Bs, out, out_scale, M, N, K, op, (hipStream_t)stream);
+    if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "fp8 gemm + qk-norm + rope launch: %s", hipGetErrorString(e));
+    return LLMMM_OK;
+  }
+  rc = launch_into_planes(pc, A, As, Bt, Bs, M, N, K, workspace, stream);
+  if (rc) return rc;
+  const hipError_t e = llmmm::fp8_planes_qk_norm_rope_launch(out_kind, (const float*)workspace, pc.split, out, out_scale, q_norm_weight, k_norm_weight, eps,
+                                                             cos_table, sin_table, table_rows, positions, n_q_heads, n_kv_heads, M, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "qk-norm + rope launch: %s", hipGetErrorString(e));
   return LLMMM_OK;
 }
 

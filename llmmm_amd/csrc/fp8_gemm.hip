@@ -32,7 +32,9 @@
 
 namespace llmmm {
 
-enum { OUT_F32 = 0, OUT_BF16 = 1, OUT_FP8Q = 2, OUT_SWIGLU = 3 };
+enum { OUT_F32 = 0, OUT_BF16 = 1, OUT_FP8Q = 2, OUT_SWIGLU = 3,
+       // internal: the bf16 / e4m3 epilogues behind the per-head RMSNorm + RoPE of a QKV projection (Fp8HeadOp)
+       OUT_ROPE_BF16 = 4, OUT_ROPE_FP8Q = 5 };
 
 __device__ __forceinline__ f32x4 mfma_fp8_k128(i32x8 x, i32x8 y)
 {
@@ -300,6 +302,62 @@ __device__ __forceinline__ void swiglu_finish(const f32x4 (&acc)[8][MF], const f
   }
 }
 
+// Per-head RMSNorm + rotary embedding on the accumulators of one wave, which hold WM rows x one whole head (128
+// columns): lane (g, li) owns row mf*16 + li, columns nf*16 + 4g + q.  Same arithmetic, in the same order, as
+// fp8_planes_qk_norm_rope_kernel: the 4-column chunk c = nf*4 + g is that kernel's lane c, so the butterfly over chunk
+// bits 4, 3, 2 runs over nf inside the lane (all eight results are equal, one is computed) and bits 1, 0 over g across
+// lanes (xor 32, xor 16); column i < 64 and its partner i + 64 are fragments nf and nf + 4 of the same lane.
+template <int MF>
+__device__ __forceinline__ void qk_norm_rope_fragments(f32x4 (&acc)[8][MF], const Fp8HeadOp& op, int head, int row0, int lane)
+{
+  if (head >= op.n_q + op.n_kv) return;  // value head (wave-uniform)
+  const int    g = lane >> 4, li = lane & 15;
+  const float* nw = head < op.n_q ? op.qw : op.kw;
+  if (nw != nullptr) {
+    float r[MF];
+#pragma unroll
+    for (int mf = 0; mf < MF; ++mf) {
+      float p[8];
+#pragma unroll
+      for (int nf = 0; nf < 8; ++nf) {
+        float a = 0.f;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) a = __builtin_fmaf(acc[nf][mf][q], acc[nf][mf][q], a);
+        p[nf] = a;
+      }
+      float t = ((p[0] + p[4]) + (p[2] + p[6])) + ((p[1] + p[5]) + (p[3] + p[7]));
+      t       = t + wave_xor_get(t, 32);
+      t       = t + wave_xor_get(t, 16);
+      r[mf]   = 1.0f / __builtin_sqrtf(t / 128.0f + op.eps);
+    }
+#pragma unroll
+    for (int nf = 0; nf < 8; ++nf) {
+      const f32x4 w = *(const f32x4*)(nw + nf * 16 + 4 * g);
+#pragma unroll
+      for (int mf = 0; mf < MF; ++mf)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[nf][mf][q] = (acc[nf][mf][q] * r[mf]) * w[q];
+    }
+  }
+#pragma unroll
+  for (int mf = 0; mf < MF; ++mf) {
+    const int    p  = min(max(op.pos[row0 + mf * 16 + li], 0), op.table_rows - 1);
+    const float* cp = op.cos_t + (size_t)p * 64 + 4 * g;
+    const float* sp = op.sin_t + (size_t)p * 64 + 4 * g;
+#pragma unroll
+    for (int nf = 0; nf < 4; ++nf) {
+      const f32x4 cs = *(const f32x4*)(cp + nf * 16), sn = *(const f32x4*)(sp + nf * 16);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float lo = acc[nf][mf][q], hi = acc[nf + 4][mf][q];
+        const float t1 = hi * sn[q], t2 = lo * sn[q];
+        acc[nf][mf][q]     = __builtin_fmaf(lo, cs[q], -t1);
+        acc[nf + 4][mf][q] = __builtin_fmaf(hi, cs[q], t2);
+      }
+    }
+  }
+}
+
 // BMODE bit 0 (BPRE): Bt is the pre-shuffled image of the weights (layout.hip) instead of row-major [N, K].
 // BMODE bit 1 (BNT): the weight loads carry the non-temporal hint (one tile row: every weight byte is read once).
 // BMODE bit 2 (DEEP, 32-row-wave tiles only): the launch has at most one workgroup per CU, which then runs a deeper pipeline.
@@ -307,7 +365,7 @@ template <int BM, int BN, int WM, int OUT, int BMODE>
 __global__ void __launch_bounds__((BM / WM) * (BN / 128) * 64)
 fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
                 const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int tiles_m,
-                int tiles_n)
+                int tiles_n, Fp8HeadOp op)
 {
   typedef Fp8Tile<BM, BN, WM> TC;
   constexpr int  MF   = TC::MF;
@@ -473,6 +531,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const int             row0 = m0 + wm * WM;
   const int             col0 = n0 + wn * 128;
   const int             li   = lane & 15;
+  if constexpr (OUT == OUT_ROPE_BF16 || OUT == OUT_ROPE_FP8Q) qk_norm_rope_fragments<MF>(acc, op, col0 >> 7, row0, lane);
   if constexpr (OUT == OUT_F32) {
     float* C = (float*)Cv + (size_t)sp * M * N;
 #pragma unroll
@@ -487,7 +546,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
       }
     }
   }
-  else if constexpr (OUT == OUT_BF16) {
+  else if constexpr (OUT == OUT_BF16 || OUT == OUT_ROPE_BF16) {
     __bf16* C = (__bf16*)Cv;
     typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
@@ -642,6 +701,81 @@ fp8_splitk_reduce_kernel(const float* __restrict__ planes, int S, void* __restri
   }
 }
 
+// The second kernel behind a QKV projection: ordered plane sum, then per-head RMSNorm and rotary embedding of the
+// query and key heads (heads of 128 columns: n_q query, n_kv key, n_kv value heads), then the bf16 or e4m3 + 1x128
+// epilogue of the reduce kernel -- a head is exactly one quantisation group.  Half a wavefront owns one row of one
+// head, lane l the columns 4l .. 4l+3:
+//   norm  (weight pointer of the head's kind not null): acc = fma(x, x, acc) over the lane's four columns, xor
+//         butterfly 16, 8, 4, 2, 1, r = 1 / sqrt(total / 128 + eps), x = (x * r) * w
+//   rope  rotate-half: column i pairs with column i + 64, which lane l ^ 16 holds at the same register index;
+//         lo' = fma(lo, cos, -(hi * sin)), hi' = fma(hi, cos, lo * sin), angle row clamp(pos[m], 0, table_rows - 1)
+template <int OUT>
+__global__ void __launch_bounds__(256)
+fp8_planes_qk_norm_rope_kernel(const float* __restrict__ planes, int S, void* __restrict__ Cv, float* __restrict__ Cs,
+                               const float* __restrict__ qw, const float* __restrict__ kw, float eps, const float* __restrict__ cos_t,
+                               const float* __restrict__ sin_t, int table_rows, const int* __restrict__ pos, int n_q, int n_kv, int M, int N,
+                               int rows_per_wg)
+{
+  static_assert(OUT == OUT_BF16 || OUT == OUT_FP8Q, "bf16 or e4m3 output");
+  const int    tid    = threadIdx.x;
+  const int    sub    = tid >> 5;
+  const int    l32    = tid & 31;
+  const int    head   = blockIdx.x;
+  const int    n      = head * 128 + l32 * 4;
+  const int    mbeg   = blockIdx.y * rows_per_wg;
+  const int    mend   = min(M, mbeg + rows_per_wg);
+  const size_t plane  = (size_t)M * N;
+  const bool   rotate = head < n_q + n_kv;
+  const float* nw     = head < n_q ? qw : (rotate ? kw : nullptr);
+  f32x4        w4     = {1.f, 1.f, 1.f, 1.f};
+  if (nw != nullptr) w4 = *(const f32x4*)(nw + l32 * 4);
+  const int  ti = (l32 & 15) * 4;  // first of the lane's four angle indices
+  const bool lo = l32 < 16;
+  for (int m = mbeg + sub; m < mend; m += 8) {
+    f32x4 cs = {1.f, 1.f, 1.f, 1.f}, sn = {0.f, 0.f, 0.f, 0.f};
+    if (rotate) {
+      const int p = min(max(pos[m], 0), table_rows - 1);
+      cs          = *(const f32x4*)(cos_t + (size_t)p * 64 + ti);
+      sn          = *(const f32x4*)(sin_t + (size_t)p * 64 + ti);
+    }
+    f32x4 v = reduce_planes(planes + (size_t)m * N + n, S, plane);
+    if (nw != nullptr) {
+      float acc = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc = __builtin_fmaf(v[q], v[q], acc);
+#pragma unroll
+      for (int step = 16; step >= 1; step >>= 1) acc = acc + wave_xor_get(acc, step);
+      const float r = 1.0f / __builtin_sqrtf(acc / 128.0f + eps);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = (v[q] * r) * w4[q];
+    }
+    if (rotate) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float other = wave_xor_get(v[q], 16);
+        const float t     = other * sn[q];
+        v[q]              = __builtin_fmaf(v[q], cs[q], lo ? -t : t);
+      }
+    }
+    if constexpr (OUT == OUT_BF16) {
+      typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+      bf16x4         o;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) o[q] = (__bf16)v[q];
+      *(bf16x4*)((__bf16*)Cv + (size_t)m * N + n) = o;
+    }
+    else {
+      float a = fmaxf(fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1])), fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
+#pragma unroll
+      for (int step = 1; step <= 16; step <<= 1) a = wave_xor_max(a, step);
+      const float scale = a / 448.f;
+      const float inv   = a > 0.f ? 448.f / a : 0.f;
+      *(uint32_t*)((uint8_t*)Cv + (size_t)m * N + n) = pack_e4m3x4(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+      if (l32 == 0) Cs[(size_t)head * M + m] = scale;
+    }
+  }
+}
+
 // --------------------------------------------------------------------------------------------- host
 template <int OUT>
 static hipError_t launch_reduce(const float* planes, int S, void* C, float* Cs, int M, int N, hipStream_t stream)
@@ -672,7 +806,7 @@ static auto pick_kernel(int bmode) -> decltype(&fp8_gemm_kernel<BM, BN, WM, OUT,
 
 template <int BM, int BN, int WM, int OUT>
 static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N,
-                             int K, int S, float* planes, bool bpre, hipStream_t stream)
+                             int K, int S, float* planes, bool bpre, const Fp8HeadOp& op, hipStream_t stream)
 {
   typedef Fp8Tile<BM, BN, WM> TC;
   const int tiles_m = M / BM, tiles_n = N / BN;
@@ -686,31 +820,38 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
     else {
       const auto kernel = pick_kernel<BM, BN, WM, OUT>(bmode);
       hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs,
-                         M, N, K, tiles_m, tiles_n);
+                         M, N, K, tiles_m, tiles_n, op);
       return hipGetLastError();
     }
   }
   // split-K (or planes != nullptr with S = 1: an epilogue that only the second kernel has): S partial planes from
   // the fp32 instantiation, then the ordered sum + epilogue
-  if (S < 1) S = 1;
-  const auto kernel = pick_kernel<BM, BN, WM, OUT_F32>(bmode);
-  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, S), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs,
-                     (void*)planes, (float*)nullptr, M, N, K, tiles_m, tiles_n);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess || C == nullptr) return e;  // C == nullptr: the caller consumes the planes itself
-  return launch_reduce<OUT>(planes, S, C, Cs, M, N, stream);
+  if constexpr (OUT == OUT_ROPE_BF16 || OUT == OUT_ROPE_FP8Q) {
+    return hipErrorInvalidValue;  // the head op has a second kernel of its own behind planes (fp8_planes_qk_norm_rope_launch)
+  }
+  else {
+    if (S < 1) S = 1;
+    const auto kernel = pick_kernel<BM, BN, WM, OUT_F32>(bmode);
+    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, S), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs,
+                       (void*)planes, (float*)nullptr, M, N, K, tiles_m, tiles_n, op);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || C == nullptr) return e;  // C == nullptr: the caller consumes the planes itself
+    return launch_reduce<OUT>(planes, S, C, Cs, M, N, stream);
+  }
 }
 
 template <int OUT>
 static hipError_t dispatch_fp8(int tile, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
-                               int M, int N, int K, int S, float* planes, bool bpre, hipStream_t stream)
+                               int M, int N, int K, int S, float* planes, bool bpre, const Fp8HeadOp& op, hipStream_t stream)
 {
   // the 256 x 256 tile uses eight 64-row waves; the smaller tiles 32-row waves (twice the waves per SIMD)
   switch (tile) {
-    case LLMMM_TILE_256x256: return launch_fp8<256, 256, 64, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
-    case LLMMM_TILE_128x256: return launch_fp8<128, 256, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
-    case LLMMM_TILE_256x128: return launch_fp8<256, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
-    case LLMMM_TILE_128x128: return launch_fp8<128, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
+    // (with the head op the 256 x 256 tile -- 128 accumulator registers per lane -- spills a dozen registers, all of them
+    // inside the epilogue, after the last MFMA: once per launch and lane, not per slice)
+    case LLMMM_TILE_256x256: return launch_fp8<256, 256, 64, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, op, stream);
+    case LLMMM_TILE_128x256: return launch_fp8<128, 256, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, op, stream);
+    case LLMMM_TILE_256x128: return launch_fp8<256, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, op, stream);
+    case LLMMM_TILE_128x128: return launch_fp8<128, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, op, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -720,10 +861,22 @@ hipError_t fp8_gemm_launch(int out_kind, int tile, int b_layout, const void* A, 
 {
   const bool bpre = b_layout == LLMMM_FP8_B_PRESHUFFLED;
   switch (out_kind) {
-    case OUT_F32: return dispatch_fp8<OUT_F32>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
-    case OUT_BF16: return dispatch_fp8<OUT_BF16>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
-    case OUT_FP8Q: return dispatch_fp8<OUT_FP8Q>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
-    case OUT_SWIGLU: return dispatch_fp8<OUT_SWIGLU>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, stream);
+    case OUT_F32: return dispatch_fp8<OUT_F32>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, Fp8HeadOp{}, stream);
+    case OUT_BF16: return dispatch_fp8<OUT_BF16>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, Fp8HeadOp{}, stream);
+    case OUT_FP8Q: return dispatch_fp8<OUT_FP8Q>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, Fp8HeadOp{}, stream);
+    case OUT_SWIGLU: return dispatch_fp8<OUT_SWIGLU>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, Fp8HeadOp{}, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t fp8_gemm_qk_rope_launch(int out_kind, int tile, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
+                                   float* Cs, int M, int N, int K, const Fp8HeadOp& op, hipStream_t stream)
+{
+  const bool bpre = b_layout == LLMMM_FP8_B_PRESHUFFLED;
+  if (N != (op.n_q + 2 * op.n_kv) * 128) return hipErrorInvalidValue;
+  switch (out_kind) {
+    case OUT_BF16: return dispatch_fp8<OUT_ROPE_BF16>(tile, A, As, Bt, Bs, C, Cs, M, N, K, 1, nullptr, bpre, op, stream);
+    case OUT_FP8Q: return dispatch_fp8<OUT_ROPE_FP8Q>(tile, A, As, Bt, Bs, C, Cs, M, N, K, 1, nullptr, bpre, op, stream);
     default: return hipErrorInvalidValue;
   }
 }
@@ -737,6 +890,25 @@ hipError_t fp8_splitk_reduce_launch(int out_kind, const float* planes, int S, vo
     case OUT_SWIGLU: return launch_reduce<OUT_SWIGLU>(planes, S, C, Cs, M, N, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+hipError_t fp8_planes_qk_norm_rope_launch(int out_kind, const float* planes, int S, void* C, float* Cs, const float* qw, const float* kw, float eps,
+                                          const float* cos_t, const float* sin_t, int table_rows, const int* pos, int n_q, int n_kv, int M,
+                                          hipStream_t stream)
+{
+  const int heads = n_q + 2 * n_kv, N = heads * 128;
+  int       rows_per_wg = 8;
+  while (rows_per_wg < 64 && (long)heads * ((M + 2 * rows_per_wg - 1) / (2 * rows_per_wg)) >= 2048) rows_per_wg *= 2;
+  const dim3 grid(heads, (M + rows_per_wg - 1) / rows_per_wg);
+  if (out_kind == OUT_BF16)
+    hipLaunchKernelGGL((fp8_planes_qk_norm_rope_kernel<OUT_BF16>), grid, dim3(256), 0, stream, planes, S, C, Cs, qw, kw, eps, cos_t, sin_t,
+                       table_rows, pos, n_q, n_kv, M, N, rows_per_wg);
+  else if (out_kind == OUT_FP8Q)
+    hipLaunchKernelGGL((fp8_planes_qk_norm_rope_kernel<OUT_FP8Q>), grid, dim3(256), 0, stream, planes, S, C, Cs, qw, kw, eps, cos_t, sin_t,
+                       table_rows, pos, n_q, n_kv, M, N, rows_per_wg);
+  else
+    return hipErrorInvalidValue;
+  return hipGetLastError();
 }
 
 }  // namespace llmmm

@@ -23,6 +23,27 @@ hipError_t fp8_gemm_launch(int out_kind, int tile, int b_layout, const void* A, 
                            void* C, float* Cs, int M, int N, int K, int S, float* planes, hipStream_t stream);
 
 // C = epilogue(planes[0] + planes[1] + ... + planes[S-1]) (that order), planes of M * N floats each.
+// Per-head RMSNorm + rotary embedding behind a QKV projection (heads of 128 columns: n_q query, n_kv key, n_kv value).
+struct Fp8HeadOp {
+  const float* qw         = nullptr;  // norm weights [128] of the query / key heads, nullptr: no norm
+  const float* kw         = nullptr;
+  const float* cos_t      = nullptr;  // [table_rows, 64]
+  const float* sin_t      = nullptr;
+  const int*   pos        = nullptr;  // [M] row of the tables, clamped
+  float        eps        = 0.f;
+  int          table_rows = 0;
+  int          n_q        = 0;
+  int          n_kv       = 0;
+};
+// A tile kernel (no split) with the head op in its epilogue; out_kind LLMMM_OUT_BF16 or LLMMM_OUT_FP8Q.
+hipError_t fp8_gemm_qk_rope_launch(int out_kind, int tile, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
+                                   float* Cs, int M, int N, int K, const Fp8HeadOp& op, hipStream_t stream);
+// Behind a QKV projection whose kernel wrote S fp32 planes: ordered plane sum, per-head RMSNorm (qw / kw [128] or
+// nullptr) and rotate-half RoPE (cos / sin tables [table_rows, 64], positions [M]) of the n_q query and n_kv key heads
+// of 128 columns, value heads untouched; out_kind LLMMM_OUT_BF16 or LLMMM_OUT_FP8Q (1x128 = per-head scales).
+hipError_t fp8_planes_qk_norm_rope_launch(int out_kind, const float* planes, int S, void* C, float* Cs, const float* qw, const float* kw, float eps,
+                                          const float* cos_t, const float* sin_t, int table_rows, const int* pos, int n_q, int n_kv, int M,
+                                          hipStream_t stream);
 hipError_t fp8_splitk_reduce_launch(int out_kind, const float* planes, int S, void* C, float* Cs, int M, int N, hipStream_t stream);
 
 // M <= 128 (row groups of 64); S splits of K.  partial == nullptr (S must be 1): complete result in C / Cs.

@@ -220,6 +220,33 @@ def fp8_gemm_add_rmsnorm_quant(A, A_scale_transposed, B_transposed, B_scale_tran
     return q, s
 
 
+def fp8_gemm_qkv_rope(A, A_scale_transposed, B_transposed, B_scale_transposed, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, positions,
+                      n_q_heads, n_kv_heads, M, N, K, out_fp8=False, stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0,
+                      b_preshuffled=False):
+    """The QKV projection with per-head RMSNorm (weights [128] or None) and rotate-half RoPE of the query and key heads fused
+    behind it (planned by the reference, README.md:16).  Heads are 128 wide; cos_table / sin_table [rows, 64] float32,
+    positions [M] int32.  Returns the bf16 tensor [M,N], or (codes uint8 [M,N], scales float32 [N/128, M]) with out_fp8."""
+    dev = A.device
+    kb = K // 128 if K % 128 == 0 else 0
+    if workspace is None:
+        n = int(lib.llmmm_fp8_gemm_qkv_rope_workspace(M, N, K))
+        workspace = torch.empty(max(n, 16), dtype=torch.uint8, device=dev)
+    out = torch.empty((M, N), dtype=torch.uint8 if out_fp8 else torch.bfloat16, device=dev)
+    sc = torch.empty(((N + 127) // 128, M), dtype=torch.float32, device=dev) if out_fp8 else None
+    rows = cos_table.shape[0]
+    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS)
+    check(lib.llmmm_fp8_gemm_qkv_rope(
+        _lib.OUT_FP8Q if out_fp8 else _lib.OUT_BF16, _ptr(A, "A", _FP8_DTYPES, M * K), _ptr(A_scale_transposed, "A_scale_transposed", (torch.float32,), kb * M),
+        _ptr(B_transposed, "B_transposed", _FP8_DTYPES, N * K), _ptr(B_scale_transposed, "B_scale_transposed", (torch.float32,), ((N + 127) // 128) * kb),
+        _ptr(out, "out"), _ptr(sc, "out_scale") if out_fp8 else None,
+        _ptr(q_norm_weight, "q_norm_weight", (torch.float32,), 128) if q_norm_weight is not None else None,
+        _ptr(k_norm_weight, "k_norm_weight", (torch.float32,), 128) if k_norm_weight is not None else None, ctypes.c_float(eps),
+        _ptr(cos_table, "cos_table", (torch.float32,), rows * 64), _ptr(sin_table, "sin_table", (torch.float32,), rows * 64), rows,
+        _ptr(positions, "positions", (torch.int32,), M), n_q_heads, n_kv_heads, M, N, K, ctypes.c_void_p(workspace.data_ptr()),
+        workspace.numel() * workspace.element_size(), ctypes.byref(cfg), _stream(stream)))
+    return (out, sc) if out_fp8 else out
+
+
 # ------------------------------------------------------------------------------------- offline layout helpers
 def construct_mfma_B_layout(dst, src_transposed, N, K, stream=None):
     """The role of ``LLMMM::construct_m16n8k32_B_layout(dst, src_transposed, N, K, stream)``

@@ -46,6 +46,7 @@ def _load():
         "oracle_fp8_gemm": (c.c_int, [u8p, f32p, u8p, f32p, f32p, c.c_int, c.c_int, c.c_int, c.c_int, c.c_int]),
         "oracle_requant_c_1x128": (None, [f32p, u8p, f32p, c.c_int, c.c_int, c.c_int, c.c_int]),
         "oracle_rmsnorm": (None, [f32p, f32p, c.c_float, f32p, c.c_int, c.c_int]),
+        "oracle_qk_norm_rope": (None, [f32p, f32p, f32p, c.c_float, f32p, f32p, c.c_int, c.POINTER(c.c_int32), c.c_int, c.c_int, f32p, c.c_int]),
         "oracle_e4m3_encode_n": (None, [f32p, u8p, c.c_size_t]),
         "oracle_e4m3_decode_n": (None, [u8p, f32p, c.c_size_t]),
         "oracle_f32_to_f16_n": (None, [f32p, u16p, c.c_size_t]),
@@ -265,6 +266,26 @@ def rmsnorm(x, w, eps):
 def rmsnorm_quant(x, w, eps):
     """RMSNorm followed by the activation quantiser (1x128, transposed scales): (q [M,K], s [ceil(K/128), M])."""
     return quant_fp8(rmsnorm(x, w, eps), 1, True)
+
+
+def qk_norm_rope(x, qw, kw, eps, cos, sin, pos, n_q, n_kv):
+    """Per-head RMSNorm (head size 128; weights qw / kw [128] or None) and rotate-half RoPE of the query and key heads
+    of a QKV projection result x [M, (n_q + 2 n_kv) * 128]; cos / sin [rows, 64] fp32, pos [M] int32.  No reference
+    kernel (README.md:16 plans the fusion); arithmetic order in oracle.c."""
+    x = _f32(x)
+    M, N = x.shape
+    assert N == (n_q + 2 * n_kv) * 128
+    cos, sin = _f32(cos), _f32(sin)
+    assert cos.shape == sin.shape and cos.shape[1] == 64
+    pos = np.ascontiguousarray(pos, dtype=np.int32)
+    assert pos.shape == (M,)
+    qw = None if qw is None else _f32(qw)
+    kw = None if kw is None else _f32(kw)
+    y = np.empty((M, N), np.float32)
+    _lib.oracle_qk_norm_rope(_p(x, ctypes.c_float), None if qw is None else _p(qw, ctypes.c_float), None if kw is None else _p(kw, ctypes.c_float),
+                             ctypes.c_float(eps), _p(cos, ctypes.c_float), _p(sin, ctypes.c_float), cos.shape[0], _p(pos, ctypes.c_int32), n_q, n_kv,
+                             _p(y, ctypes.c_float), M)
+    return y
 
 
 # ----------------------------------------------------------------------------- offline layouts

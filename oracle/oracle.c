@@ -36,6 +36,14 @@
  *                                                            pinned: float64 evaluation, exact invariance under
  *                                                            power-of-two scaling (eps = 0), unit mean square
  *
+ *   oracle_qk_norm_rope      no reference kernel (fusing RMSNorm and RoPE into the GEMM is on the reference's plan,
+ *                            README.md:16): per-head RMSNorm (head size 128) and rotary embedding of the query and key
+ *                            heads of a QKV projection, value heads untouched
+ *                                                            pinned: float64 evaluation of the rotate-half formula,
+ *                                                            identity at angle 0, quarter turn, exact inverse
+ *                                                            and pair norm on an integer 3-4-5 rotation, the
+ *                                                            documented summation order rebuilt in numpy
+ *
  * Compile with -ffp-contract=off: every fused multiply-add below is written explicitly.
  */
 #include <math.h>
@@ -447,6 +455,63 @@ ORACLE_API void oracle_f32_to_bf16_n(const float* x, uint16_t* h, size_t n)
 ORACLE_API void oracle_bf16_to_f32_n(const uint16_t* h, float* x, size_t n)
 {
   for (size_t i = 0; i < n; ++i) x[i] = oracle_bf16_to_f32(h[i]);
+}
+
+/* Per-head RMSNorm and rotary position embedding behind a QKV projection (heads of 128 columns: n_q query heads, then
+ * n_kv key heads, then n_kv value heads; N = (n_q + 2 n_kv) * 128).  No reference kernel (README.md:16 plans the
+ * fusion); the arithmetic order is this build's definition, chosen so that 32 GPU lanes per head reproduce it:
+ *   norm (query heads with qw, key heads with kw; skipped when the weight pointer is NULL): lane l of 32 owns columns
+ *     4l .. 4l+3 and accumulates acc = fma(x, x, acc) over them in ascending order from 0; the 32 partial sums are
+ *     combined by a butterfly (p[l] += p[l ^ 16], then ^8, ^4, ^2, ^1); r = 1 / sqrt(total / 128 + eps);
+ *     x <- (x * r) * w[col]                                (w has 128 entries, shared by all heads of a kind)
+ *   rope (query and key heads; rotate-half pairing of column i with column i + 64, i < 64; angle row
+ *     p = clamp(pos[m], 0, table_rows - 1) of the cos / sin tables [table_rows, 64]):
+ *     y[i]      = fma(x[i],      cos[p,i], -(x[i + 64] * sin[p,i]))
+ *     y[i + 64] = fma(x[i + 64], cos[p,i],   x[i]      * sin[p,i])
+ *   value heads: y = x. */
+ORACLE_API void oracle_qk_norm_rope(const float* x, const float* qw, const float* kw, float eps, const float* cos_t, const float* sin_t,
+                                    int table_rows, const int32_t* pos, int n_q, int n_kv, float* y, int M)
+{
+  const int N = (n_q + 2 * n_kv) * 128;
+#pragma omp parallel for schedule(static)
+  for (int m = 0; m < M; ++m) {
+    int p = pos[m];
+    if (p < 0) p = 0;
+    if (p > table_rows - 1) p = table_rows - 1;
+    const float* c = cos_t + (size_t)p * 64;
+    const float* s = sin_t + (size_t)p * 64;
+    for (int h = 0; h < n_q + 2 * n_kv; ++h) {
+      const float* xr = x + (size_t)m * N + h * 128;
+      float*       yr = y + (size_t)m * N + h * 128;
+      if (h >= n_q + n_kv) {
+        for (int i = 0; i < 128; ++i) yr[i] = xr[i];
+        continue;
+      }
+      float        v[128];
+      const float* w = h < n_q ? qw : kw;
+      for (int i = 0; i < 128; ++i) v[i] = xr[i];
+      if (w) {
+        float part[32];
+        for (int l = 0; l < 32; ++l) {
+          float acc = 0.f;
+          for (int e = 0; e < 4; ++e) acc = fmaf(v[4 * l + e], v[4 * l + e], acc);
+          part[l] = acc;
+        }
+        for (int step = 16; step >= 1; step >>= 1) {
+          float t[32];
+          for (int l = 0; l < 32; ++l) t[l] = part[l] + part[l ^ step];
+          for (int l = 0; l < 32; ++l) part[l] = t[l];
+        }
+        const float r = 1.0f / sqrtf(part[0] / 128.0f + eps);
+        for (int i = 0; i < 128; ++i) v[i] = (v[i] * r) * w[i];
+      }
+      for (int i = 0; i < 64; ++i) {
+        const float lo = v[i], hi = v[i + 64];
+        yr[i]      = fmaf(lo, c[i], -(hi * s[i]));
+        yr[i + 64] = fmaf(hi, c[i], lo * s[i]);
+      }
+    }
+  }
 }
 
 /* RMSNorm in fp32: y[m,k] = (x[m,k] * r) * w[k], r = 1 / sqrt(sum_k x[m,k]^2 / K + eps).

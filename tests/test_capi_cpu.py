@@ -208,6 +208,58 @@ def test_rmsnorm_quant_validation_without_device():
     assert f(_lib.DTYPE_F16, ctypes.c_void_p(0x1008), FAKE, eps, FAKE, FAKE, 4, 128, None) == _lib.ERR_INVALID_ARGUMENT
 
 
+def test_gemm_add_rmsnorm_quant_validation_without_device():
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    f = lib.llmmm_fp8_gemm_add_rmsnorm_quant
+    eps = ctypes.c_float(1e-6)
+    M, N, K = 16, 2560, 4096
+    plane = M * N * 4
+
+    def call(dtype=_lib.DTYPE_BF16, res=FAKE, n=N, k=K, ws=FAKE, wsz=plane, cfg=None, e=eps, m=M):
+        return f(FAKE, FAKE, FAKE, FAKE, dtype, res, FAKE, FAKE, e, FAKE, FAKE, m, n, k, ws, wsz, cfg, None)
+
+    assert call(dtype=9) == _lib.ERR_UNSUPPORTED_TYPE
+    assert call(n=2500) == _lib.ERR_NOT_ALIGNED
+    assert call(k=100) == _lib.ERR_NOT_ALIGNED
+    assert call(res=None) == _lib.ERR_INVALID_ARGUMENT
+    assert call(n=10240 + 128) == _lib.ERR_INVALID_ARGUMENT
+    assert call(e=ctypes.c_float(-1.0)) == _lib.ERR_INVALID_ARGUMENT
+    assert call(ws=None, wsz=0) == _lib.ERR_WORKSPACE
+    assert call(wsz=plane - 4) == _lib.ERR_WORKSPACE
+    assert call(cfg=ctypes.byref(_lib.GemmCfg(_lib.TILE_SKINNY, 2, 0))) == _lib.ERR_WORKSPACE  # an explicit split never shrinks
+    assert call(cfg=ctypes.byref(_lib.GemmCfg(_lib.TILE_64x128, 1, 0)), m=256, wsz=256 * N * 4) == _lib.ERR_INVALID_ARGUMENT
+    assert call(cfg=ctypes.byref(_lib.GemmCfg(_lib.TILE_256x256, 1, 0)), m=128, wsz=128 * N * 4) == _lib.ERR_NOT_ALIGNED
+    need = lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K)
+    assert need >= plane and need % plane == 0
+    assert lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, 100, K) == 0
+
+
+def test_qkv_rope_validation_without_device():
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    f = lib.llmmm_fp8_gemm_qkv_rope
+    eps = ctypes.c_float(1e-6)
+    M, N, K = 16, 6144, 2560
+    plane = M * N * 4
+
+    def call(kind=_lib.OUT_BF16, out=FAKE, sc=FAKE, qw=FAKE, kw=FAKE, cos=FAKE, rows=64, pos=FAKE, nq=32, nkv=8, n=N, k=K, ws=FAKE, wsz=plane):
+        return f(kind, FAKE, FAKE, FAKE, FAKE, out, sc, qw, kw, eps, cos, FAKE, rows, pos, nq, nkv, M, n, k, ws, wsz, None, None)
+
+    assert call(kind=_lib.OUT_F32) == _lib.ERR_INVALID_ARGUMENT
+    assert call(k=100) == _lib.ERR_NOT_ALIGNED
+    assert call(nq=31) == _lib.ERR_INVALID_ARGUMENT          # head counts must add up to N / 128
+    assert call(out=None) == _lib.ERR_INVALID_ARGUMENT
+    assert call(kind=_lib.OUT_FP8Q, sc=None) == _lib.ERR_INVALID_ARGUMENT
+    assert call(rows=0) == _lib.ERR_INVALID_ARGUMENT
+    assert call(pos=None) == _lib.ERR_INVALID_ARGUMENT
+    assert call(pos=ctypes.c_void_p(0x1002)) == _lib.ERR_INVALID_ARGUMENT
+    assert call(cos=ctypes.c_void_p(0x1008)) == _lib.ERR_INVALID_ARGUMENT
+    assert call(ws=None, wsz=0) == _lib.ERR_WORKSPACE
+    assert call(wsz=plane - 4) == _lib.ERR_WORKSPACE
+    assert lib.llmmm_fp8_gemm_qkv_rope_workspace(M, N, K) >= plane
+
+
 def test_the_64x128_tile_is_fp16_only():
     from llmmm_amd import _lib
     lib = _lib.lib
