@@ -144,9 +144,10 @@ LLMMM_API int llmmm_rmsnorm_quant_fp8(int in_dtype, const void* x, const float* 
  *   h          = C32 + residual                          (fp32; residual [M,N] of hidden_dtype)
  *   hidden_out = hidden_dtype(h)                         (the new residual stream; may be the same buffer as residual)
  *   q, q_scale = llmmm_rmsnorm_quant_fp8(hidden_out, norm_weight, eps)   -- bit for bit what the separate call gives
- * so the next projection's A operand leaves this call, and neither the GEMM's result nor the normalised activations
- * make a round trip of their own.  The GEMM always goes through fp32 planes in `workspace`
- * (llmmm_fp8_gemm_add_rmsnorm_quant_workspace bytes; at least M * N * 4), which the fused kernel sums in split order.
+ * so the next projection's A operand leaves this call.  Small M (the weight-streaming kernel) and split-K runs go
+ * through fp32 planes in `workspace` (llmmm_fp8_gemm_add_rmsnorm_quant_workspace bytes), which one kernel sums in split
+ * order, adds the residual to, normalises and quantises; an unsplit tile kernel adds the residual in its own epilogue,
+ * the norm + quantiser kernel follows, and no workspace is needed (the query function then returns 0).
  * hidden_dtype: LLMMM_DTYPE_F32 / _BF16 / _F16.  N % 128 == 0, N <= 10240, K % 128 == 0, M as for llmmm_fp8_gemm.
  * cfg may be NULL (library's choice of kernel and split). */
 LLMMM_API int    llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As, const void* Bt, const float* Bs, int hidden_dtype,

@@ -393,6 +393,7 @@ size_t llmmm_fp8_gemm_add_rmsnorm_quant_workspace(int M, int N, int K)
   if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
   llmmm_gemm_cfg cfg;
   if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
+  if (cfg.tile != LLMMM_TILE_SKINNY && cfg.split_k <= 1) return 0;  // residual added inside the tile kernel
   return (size_t)(cfg.split_k < 1 ? 1 : cfg.split_k) * M * N * sizeof(float);
 }
 
@@ -478,8 +479,16 @@ int llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As, const void*
   if (!aligned16(residual) || !aligned16(hidden_out) || !aligned16(norm_weight) || !aligned16(q))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
   PlaneCfg pc;
-  int      rc = resolve_plane_cfg(A, As, Bt, Bs, M, N, K, workspace, workspace_bytes, user, false, &pc);
+  int      rc = resolve_plane_cfg(A, As, Bt, Bs, M, N, K, workspace, workspace_bytes, user, true, &pc);
   if (rc) return rc;
+  if (pc.split == 0) {
+    // a tile kernel without split: the residual is added in its epilogue, the norm + quantiser kernel follows on the
+    // stored hidden state (the same two operations on the same values as behind planes, without the fp32 round trip)
+    hipError_t e = llmmm::fp8_gemm_add_residual_launch(hidden_dtype, pc.tile, pc.b_layout, A, As, Bt, Bs, residual, hidden_out, M, N, K, (hipStream_t)stream);
+    if (e == hipSuccess) e = llmmm::rmsnorm_quant_launch(hidden_dtype, hidden_out, norm_weight, eps, q, q_scale, M, N, (hipStream_t)stream);
+    if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "fp8 gemm + add, rmsnorm + quantiser launch: %s", hipGetErrorString(e));
+    return LLMMM_OK;
+  }
   rc = launch_into_planes(pc, A, As, Bt, Bs, M, N, K, workspace, stream);
   if (rc) return rc;
   const hipError_t e = llmmm::planes_add_rmsnorm_quant_launch(hidden_dtype, (const float*)workspace, pc.split, residual, hidden_out, norm_weight, eps, q,

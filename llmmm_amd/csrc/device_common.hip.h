@@ -152,4 +152,45 @@ __device__ __forceinline__ float wave_xor_max(float v, int mask)
   return fmaxf(v, wave_xor_get(v, mask));
 }
 
+// Four consecutive row elements of type float / bf16 / fp16 <-> fp32 (one 16- or 8-byte access).
+template <typename IN_T>
+__device__ __forceinline__ f32x4 load_row4(const IN_T* p);
+template <>
+__device__ __forceinline__ f32x4 load_row4<float>(const float* p)
+{
+  return *(const f32x4*)p;
+}
+template <>
+__device__ __forceinline__ f32x4 load_row4<__bf16>(const __bf16* p)
+{
+  typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+  const bf16x4   v = *(const bf16x4*)p;
+  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+template <>
+__device__ __forceinline__ f32x4 load_row4<_Float16>(const _Float16* p)
+{
+  const f16x4 v = *(const f16x4*)p;
+  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+
+template <typename T>
+__device__ __forceinline__ void store_row4(T* p, f32x4 v);
+template <>
+__device__ __forceinline__ void store_row4<float>(float* p, f32x4 v)
+{
+  *(f32x4*)p = v;
+}
+template <>
+__device__ __forceinline__ void store_row4<__bf16>(__bf16* p, f32x4 v)
+{
+  typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+  *(bf16x4*)p = bf16x4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+}
+template <>
+__device__ __forceinline__ void store_row4<_Float16>(_Float16* p, f32x4 v)
+{
+  *(f16x4*)p = f16x4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+}
+
 }  // namespace llmmm

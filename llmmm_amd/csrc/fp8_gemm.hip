@@ -27,6 +27,7 @@
 //    128-column quantisation group, so the row amax needs the lane's 32 values and two
 //    cross-lane steps; scale = amax/448, codes = e4m3(C * (448/amax)), saturating.
 //    A group of zeros yields scale 0 and codes 0 (the reference's unguarded 0*inf gives NaN codes).
+#include <type_traits>
 #include "device_common.hip.h"
 #include "kernels.h"
 
@@ -34,7 +35,9 @@ namespace llmmm {
 
 enum { OUT_F32 = 0, OUT_BF16 = 1, OUT_FP8Q = 2, OUT_SWIGLU = 3,
        // internal: the bf16 / e4m3 epilogues behind the per-head RMSNorm + RoPE of a QKV projection (Fp8HeadOp)
-       OUT_ROPE_BF16 = 4, OUT_ROPE_FP8Q = 5 };
+       OUT_ROPE_BF16 = 4, OUT_ROPE_FP8Q = 5,
+       // internal: hidden = T(C + residual), T = float / bf16 / fp16 (Fp8HeadOp::residual, the output goes to Cv)
+       OUT_ADD_F32 = 6, OUT_ADD_BF16 = 7, OUT_ADD_F16 = 8 };
 
 __device__ __forceinline__ f32x4 mfma_fp8_k128(i32x8 x, i32x8 y)
 {
@@ -546,6 +549,24 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
       }
     }
   }
+  else if constexpr (OUT == OUT_ADD_F32 || OUT == OUT_ADD_BF16 || OUT == OUT_ADD_F16) {
+    // the fp32 staging of OUT_F32; each lane then adds the residual to its four columns in fp32 and stores T(sum)
+    typedef typename std::conditional<OUT == OUT_ADD_F32, float, typename std::conditional<OUT == OUT_ADD_BF16, __bf16, _Float16>::type>::type T;
+    const T* res = (const T*)op.residual;
+    T*       H   = (T*)Cv;
+#pragma unroll
+    for (int mf = 0; mf < MF; ++mf) {
+#pragma unroll
+      for (int nf = 0; nf < 8; ++nf) *(f32x4 LLMMM_LDS*)(stg + li * 512 + (((nf * 4 + g) ^ ((li & 7) << 1)) << 4)) = acc[nf][mf];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int    r   = 2 * j + (lane >> 5), c = lane & 31;
+        const f32x4  v   = *(const f32x4 LLMMM_LDS*)(stg + r * 512 + ((c ^ ((r & 7) << 1)) << 4));
+        const size_t idx = (size_t)(row0 + 16 * mf + r) * N + col0 + c * 4;
+        store_row4<T>(H + idx, v + load_row4<T>(res + idx));
+      }
+    }
+  }
   else if constexpr (OUT == OUT_BF16 || OUT == OUT_ROPE_BF16) {
     __bf16* C = (__bf16*)Cv;
     typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
@@ -826,8 +847,8 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
   }
   // split-K (or planes != nullptr with S = 1: an epilogue that only the second kernel has): S partial planes from
   // the fp32 instantiation, then the ordered sum + epilogue
-  if constexpr (OUT == OUT_ROPE_BF16 || OUT == OUT_ROPE_FP8Q) {
-    return hipErrorInvalidValue;  // the head op has a second kernel of its own behind planes (fp8_planes_qk_norm_rope_launch)
+  if constexpr (OUT >= OUT_ROPE_BF16) {
+    return hipErrorInvalidValue;  // these epilogues have second kernels of their own behind planes
   }
   else {
     if (S < 1) S = 1;
@@ -877,6 +898,20 @@ hipError_t fp8_gemm_qk_rope_launch(int out_kind, int tile, int b_layout, const v
   switch (out_kind) {
     case OUT_BF16: return dispatch_fp8<OUT_ROPE_BF16>(tile, A, As, Bt, Bs, C, Cs, M, N, K, 1, nullptr, bpre, op, stream);
     case OUT_FP8Q: return dispatch_fp8<OUT_ROPE_FP8Q>(tile, A, As, Bt, Bs, C, Cs, M, N, K, 1, nullptr, bpre, op, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+hipError_t fp8_gemm_add_residual_launch(int hidden_dtype, int tile, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs,
+                                        const void* residual, void* hidden, int M, int N, int K, hipStream_t stream)
+{
+  const bool bpre = b_layout == LLMMM_FP8_B_PRESHUFFLED;
+  Fp8HeadOp  op;
+  op.residual = residual;
+  switch (hidden_dtype) {
+    case LLMMM_DTYPE_F32: return dispatch_fp8<OUT_ADD_F32>(tile, A, As, Bt, Bs, hidden, nullptr, M, N, K, 1, nullptr, bpre, op, stream);
+    case LLMMM_DTYPE_BF16: return dispatch_fp8<OUT_ADD_BF16>(tile, A, As, Bt, Bs, hidden, nullptr, M, N, K, 1, nullptr, bpre, op, stream);
+    case LLMMM_DTYPE_F16: return dispatch_fp8<OUT_ADD_F16>(tile, A, As, Bt, Bs, hidden, nullptr, M, N, K, 1, nullptr, bpre, op, stream);
     default: return hipErrorInvalidValue;
   }
 }

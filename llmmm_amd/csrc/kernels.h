@@ -34,10 +34,15 @@ struct Fp8HeadOp {
   int          table_rows = 0;
   int          n_q        = 0;
   int          n_kv       = 0;
+  const void*  residual   = nullptr;  // fp8_gemm_add_residual_launch only: [M, N] of the hidden dtype
 };
 // A tile kernel (no split) with the head op in its epilogue; out_kind LLMMM_OUT_BF16 or LLMMM_OUT_FP8Q.
 hipError_t fp8_gemm_qk_rope_launch(int out_kind, int tile, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
                                    float* Cs, int M, int N, int K, const Fp8HeadOp& op, hipStream_t stream);
+// A tile kernel (no split) whose epilogue stores hidden = T(C + residual), T = hidden_dtype (LLMMM_DTYPE_*); hidden may be
+// the residual buffer.
+hipError_t fp8_gemm_add_residual_launch(int hidden_dtype, int tile, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs,
+                                        const void* residual, void* hidden, int M, int N, int K, hipStream_t stream);
 // Behind a QKV projection whose kernel wrote S fp32 planes: ordered plane sum, per-head RMSNorm (qw / kw [128] or
 // nullptr) and rotate-half RoPE (cos / sin tables [table_rows, 64], positions [M]) of the n_q query and n_kv key heads
 // of 128 columns, value heads untouched; out_kind LLMMM_OUT_BF16 or LLMMM_OUT_FP8Q (1x128 = per-head scales).

@@ -130,27 +130,6 @@ __global__ void __launch_bounds__(256) quant_128x128_kernel(const float* __restr
 //     single wavefront works through the row's 40 divisions per lane on its own), 6.9 instead of 9.4 us at M = 2048.
 //   * rmsnorm_quant_1x128_kernel: one wavefront per row (a lane plays four virtual lanes), the row read twice:
 //     longer rows.
-template <typename IN_T>
-__device__ __forceinline__ f32x4 load_row4(const IN_T* p);
-template <>
-__device__ __forceinline__ f32x4 load_row4<float>(const float* p)
-{
-  return *(const f32x4*)p;
-}
-template <>
-__device__ __forceinline__ f32x4 load_row4<__bf16>(const __bf16* p)
-{
-  typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-  const bf16x4   v = *(const bf16x4*)p;
-  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
-}
-template <>
-__device__ __forceinline__ f32x4 load_row4<_Float16>(const _Float16* p)
-{
-  const f16x4 v = *(const f16x4*)p;
-  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
-}
-
 // One chunk (4 elements) per lane of row m: normalise, take the amax of the 128-column group (the 32 chunks of this
 // half of the wavefront), quantise, store codes and the group's scale.
 __device__ __forceinline__ void rmsnorm_quant_chunk(f32x4 v, float r, const float* __restrict__ w, uint8_t* __restrict__ q,
@@ -284,25 +263,6 @@ __global__ void __launch_bounds__(256) rmsnorm_quant_row_kernel(const IN_T* __re
 // state, exactly what a separate kernel reading `hidden` would see, and follows the same fixed summation order
 // (rmsnorm_quant_row_kernel), so its codes and scales are those of the unfused sequence, bit for bit.
 // One 256-thread workgroup per row; N <= 1024 * NI columns.
-template <typename T>
-__device__ __forceinline__ void store_row4(T* p, f32x4 v);
-template <>
-__device__ __forceinline__ void store_row4<float>(float* p, f32x4 v)
-{
-  *(f32x4*)p = v;
-}
-template <>
-__device__ __forceinline__ void store_row4<__bf16>(__bf16* p, f32x4 v)
-{
-  typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-  *(bf16x4*)p = bf16x4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-}
-template <>
-__device__ __forceinline__ void store_row4<_Float16>(_Float16* p, f32x4 v)
-{
-  *(f16x4*)p = f16x4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-}
-
 template <typename T, int NI>
 __global__ void __launch_bounds__(256) planes_add_rmsnorm_quant_kernel(const float* __restrict__ planes, int S, const T* residual, T* hidden,
                                                                        const float* __restrict__ w, float eps, uint8_t* __restrict__ q,

@@ -69,6 +69,30 @@ def test_tile_kernels(lib, oracle, M, N, K, tile, split, dt):
     _check(lib, oracle, M, N, K, dt, TILES[tile], split)
 
 
+def test_unsplit_tile_kernels_add_the_residual_themselves(lib, oracle):
+    """Without split the tile kernel's epilogue adds the residual and the norm kernel follows: no planes, no workspace
+    (a 16-byte dummy here), the same bits."""
+    assert lib._lib.lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(2048, 2560, 4096) == 0
+    for dt in ("f32", "bf16", "f16"):
+        for tile in ("128x128", "256x128", "128x256", "256x256"):
+            M, N, K = 256, 512, 384
+            Aq, As, Bq, Bs, res, w = _operands(oracle, M, N, K, 3)
+            dA, dAs, dB, dBs = (torch.from_numpy(a).cuda() for a in (Aq, As, Bq, Bs))
+            C = torch.empty((M, N), dtype=torch.float32, device="cuda")
+            lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dA, dAs, dB, dBs, C, M, N, K, tile=TILES[tile], split_k=1)
+            hidden = torch.from_numpy(res).cuda().to(_TORCH[dt])  # in place
+            seen = hidden.float().cpu().numpy()
+            tiny = torch.empty(16, dtype=torch.uint8, device="cuda")
+            q, s = lib.fp8_gemm_add_rmsnorm_quant(dA, dAs, dB, dBs, hidden, hidden, torch.from_numpy(w).cuda(), 1e-6, M, N, K, workspace=tiny,
+                                                  tile=TILES[tile], split_k=1)
+            torch.cuda.synchronize()
+            want = torch.from_numpy(C.cpu().numpy() + seen).to(_TORCH[dt])
+            view = torch.int32 if dt == "f32" else torch.int16
+            assert torch.equal(hidden.cpu().view(view), want.view(view)), (dt, tile)
+            rq, rs = oracle.rmsnorm_quant(want.float().numpy(), w, 1e-6)
+            assert np.array_equal(s.cpu().numpy().view(np.uint32), rs.view(np.uint32)) and np.array_equal(q.cpu().numpy(), rq), (dt, tile)
+
+
 def test_preshuffled_weights_and_in_place_residual(lib, oracle):
     _check(lib, oracle, 16, 2560, 4096, "bf16", TILES["auto"], 0, pre=True, inplace=True)
     _check(lib, oracle, 256, 2560, 1024, "bf16", TILES["auto"], 0, pre=True, inplace=True)
