@@ -118,4 +118,20 @@ void fp8_gemm_blockwise_quant_A_1x128__B_128x128__add_rmsnorm__output_fp8(const 
                                                            eps, q, q_scale, M, N, K, workspace, workspace_bytes, nullptr, (void*)stream));
 }
 
+// The QKV projection with per-head RMSNorm (q_norm / k_norm weights [128], either may be nullptr) and the rotate-half
+// rotary embedding of the query and key heads fused behind it (planned by the reference, README.md:16; no reference
+// kernel).  Heads of 128 columns: n_q_heads query, n_kv_heads key, n_kv_heads value; cos / sin fp32 [table_rows, 64];
+// positions [M].  C: bf16 [M, N].  workspace: llmmm_fp8_gemm_qkv_rope_workspace(M, N, K) bytes (0 at prefill sizes).
+inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__qk_norm_rope__output_bf16(const fp8_t* A, const float* A_scale_transposed,
+                                                                                   const fp8_t* B_transposed, const float* B_scale_transposed, void* C,
+                                                                                   const float* q_norm_weight, const float* k_norm_weight, float eps,
+                                                                                   const float* cos_table, const float* sin_table, int table_rows,
+                                                                                   const int* positions, int n_q_heads, int n_kv_heads, int M, int N,
+                                                                                   int K, void* workspace, size_t workspace_bytes, hipStream_t stream)
+{
+  detail8::throw_on_error(llmmm_fp8_gemm_qkv_rope(LLMMM_OUT_BF16, A, A_scale_transposed, B_transposed, B_scale_transposed, C, nullptr, q_norm_weight,
+                                                  k_norm_weight, eps, cos_table, sin_table, table_rows, positions, n_q_heads, n_kv_heads, M, N, K,
+                                                  workspace, workspace_bytes, nullptr, (void*)stream));
+}
+
 }  // namespace LLMMM

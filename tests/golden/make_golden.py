@@ -65,6 +65,18 @@ def main():
     Hq, Hs = oracle.swiglu_requant(Cg)
     np.savez_compressed(os.path.join(HERE, "swiglu_128x512x256.npz"), aq=Sq, a_scale_t=Ss, bq_t=Wq, b_scale=Wsc, c_f32=Cg, h_f32=oracle.swiglu(Cg),
                         hq=Hq, h_scale_t=Hs)
+    # per-head RMSNorm + RoPE behind a QKV projection: 2 query, 1 key, 1 value head, positions beyond both table ends
+    xr = (rng.standard_normal((16, 4 * 128)) * 3).astype(np.float32)
+    qw = rng.uniform(0.5, 1.5, 128).astype(np.float32)
+    kw = rng.uniform(0.5, 1.5, 128).astype(np.float32)
+    inv = 1e6 ** (-np.arange(64, dtype=np.float64) / 64.0)
+    ang = np.arange(48, dtype=np.float64)[:, None] * inv[None, :]
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    pos = rng.integers(-2, 52, 16).astype(np.int32)
+    yr = oracle.qk_norm_rope(xr, qw, kw, 1e-6, cos, sin, pos, 2, 1)
+    yq, ys = oracle.requant_c_1x128(yr)
+    np.savez_compressed(os.path.join(HERE, "qk_norm_rope_16x512.npz"), x=xr, qw=qw, kw=kw, cos=cos, sin=sin, pos=pos, y=yr, y_bf16=oracle.f32_to_bf16_bits(yr),
+                        yq=yq, y_scale_t=ys)
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

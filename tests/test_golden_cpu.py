@@ -64,3 +64,23 @@ def test_swiglu_fixture(oracle):
     # closed-form cross-check of the stored activation: float64, tanh form
     g, u = C[:, :256].astype(np.float64), C[:, 256:].astype(np.float64)
     assert np.all(np.abs(d["h_f32"] - g * 0.5 * (1 + np.tanh(g / 2)) * u) <= 4e-7 * np.abs(g * u) + 1e-37)
+
+
+def test_qk_norm_rope_fixture(oracle):
+    d = np.load(os.path.join(G, "qk_norm_rope_16x512.npz"))
+    y = oracle.qk_norm_rope(d["x"], d["qw"], d["kw"], 1e-6, d["cos"], d["sin"], d["pos"], 2, 1)
+    assert np.array_equal(y.view(np.uint32), d["y"].view(np.uint32))
+    assert np.array_equal(oracle.f32_to_bf16_bits(y), d["y_bf16"])
+    yq, ys = oracle.requant_c_1x128(y)
+    assert np.array_equal(yq, d["yq"]) and np.array_equal(ys.view(np.uint32), d["y_scale_t"].view(np.uint32))
+    assert d["pos"].min() < 0 and d["pos"].max() >= d["cos"].shape[0], "the fixture does not exercise the clamp"
+    # closed-form cross-check of the stored result: float64 norm + rotate-half rotation
+    x = d["x"].astype(np.float64).reshape(16, 4, 128)
+    p = np.clip(d["pos"], 0, d["cos"].shape[0] - 1)
+    c, s = d["cos"][p].astype(np.float64), d["sin"][p].astype(np.float64)
+    ref = x.copy()
+    for h, w in ((0, d["qw"]), (1, d["qw"]), (2, d["kw"])):
+        v = x[:, h] / np.sqrt((x[:, h] ** 2).mean(axis=1, keepdims=True) + 1e-6) * w.astype(np.float64)
+        ref[:, h, :64] = v[:, :64] * c - v[:, 64:] * s
+        ref[:, h, 64:] = v[:, 64:] * c + v[:, :64] * s
+    assert np.abs(d["y"].reshape(16, 4, 128) - ref).max() <= 2e-6 * np.abs(ref).max()
