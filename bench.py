@@ -342,7 +342,7 @@ def main():
     ap.add_argument("--workload", default="fp16_gemm_4096",
                     help="fp16_gemm_4096 (headline) | fp8_gemm_fused_4096 | fp8_gemm_bf16_4096 | bf16_gemm_4096 | "
                          "decode_<qkv|o|gate_up|down>_m<M>[_pre] (_pre: weights pre-shuffled offline) | prefill_<qkv|o|gate_up|down>_m<M> | "
-                         "prefill_gate_up_swiglu_m<M> | copy_1g (counter calibration only)")
+                         "prefill_gate_up_swiglu_m<M> | fused_<o|down>_add_norm_m<M> | fused_qkv_rope_m<M> | copy_1g (counter calibration only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measured-peak probes")
@@ -386,6 +386,35 @@ def main():
                 "kernel": "fp8_gemm_kernel<256,256,%s>" % out}
         value, unit = r["tflops"], "TFLOP/s"
         cfg = {"workload": "FP8 e4m3 blockwise GEMM M=N=K=4096 (A 1x128, B 128x128 scales), output %s" % out, "M": M, "N": N, "K": K}
+    elif w.startswith("fused_"):
+        import re
+        mo = re.fullmatch(r"fused_(o|down)_add_norm_m(\d+)|fused_qkv_rope_m(\d+)", w)
+        if not mo:
+            print("unknown workload", w, file=sys.stderr)
+            sys.exit(2)
+        if mo.group(1):
+            name, M = mo.group(1), int(mo.group(2))
+            x = bench_proj_add_norm(name, M, args.steps, args.warmup)
+            what = "%s projection + residual add + RMSNorm + 1x128 quantisation (bf16 hidden state)" % name
+            nbytes = fp8_bytes(M, x["N"], x["K"], "fp8q") + 4.0 * M * x["N"]
+        else:
+            name, M = "qkv", int(mo.group(3))
+            x = bench_qkv_rope(M, args.steps, args.warmup)
+            what = "QKV projection + per-head RMSNorm + RoPE, bf16 output"
+            nbytes = fp8_bytes(M, x["N"], x["K"], "bf16")
+        N, K = x["N"], x["K"]
+        r = {"ms": x["us"] * 1e-3, "wall_ms": x["us"] * 1e-3, "bytes": nbytes}
+        dtype = "fp8"
+        if M <= 128:
+            roof = {"bound": "hbm", "achieved": x["hbm_gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": x["hbm_gbs"] / PEAK_HBM_GBS, "traffic": None,
+                    "kernel": "fp8_skinny_kernel + fused second kernel"}
+            value, unit = x["hbm_gbs"], "GB/s"
+        else:
+            roof = {"bound": "mfma", "achieved": x["tflops"], "peak": PEAK_TFLOPS["fp8"], "unit": "TFLOP/s", "frac": x["tflops"] / PEAK_TFLOPS["fp8"],
+                    "traffic": None, "kernel": "fp8_gemm_kernel with the fused epilogue"}
+            value, unit = x["tflops"], "TFLOP/s"
+        cfg = {"workload": "Qwen3-4B %s, M=%d N=%d K=%d, pre-shuffled weights rotated over %d copies; the same work as separate launches: %.2f us"
+                           % (what, M, N, K, x["weight_copies"], x.get("us_separate_launches", x.get("us_plain_bf16_gemm", 0.0))), "M": M, "N": N, "K": K}
     elif w.startswith("decode_"):
         import re
         mo = re.fullmatch(r"decode_(qkv|o|gate_up|down)_m(\d+)(_pre)?", w)
