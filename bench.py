@@ -287,6 +287,67 @@ def bench_qkv_rope(M, steps, warmup, rotate_bytes=768 << 20):
             "weight_copies": copies}
 
 
+def bench_decoder_layer(M, steps, warmup, rotate_bytes=768 << 20):
+    """The GEMM side of one Qwen3-4B decoder layer at decode-sized M as four entry points and no elementwise launch:
+    QKV + per-head RMSNorm + RoPE (bf16 out) -> [attention: not part of this library; a fixed quantised stand-in feeds O] ->
+    O + residual + RMSNorm + quant -> gate_up with SwiGLU output -> down + residual + RMSNorm + quant (the next layer's A).
+    Pre-shuffled weights, rotated over distinct copies so that they stream from HBM.  Algorithmic bytes: the four weight
+    matrices once (100.9 MB)."""
+    import llmmm_amd
+    from llmmm_amd import _lib
+    hidden, inter, n_q, n_kv = 2560, 9728, 32, 8
+    shapes = {"qkv": (6144, hidden), "o": (hidden, 4096), "gate_up": (2 * inter, hidden), "down": (hidden, inter)}
+    per_copy = sum(n * k for n, k in shapes.values())
+    copies = max(2, int(np.ceil(rotate_bytes / float(per_copy))))
+    g = torch.Generator(device="cuda").manual_seed(13)
+    weights = []
+    for _ in range(copies):
+        layer = {}
+        for name, (n, k) in shapes.items():
+            W = torch.randn((n, k), generator=g, device="cuda") * 0.02
+            q, sc = llmmm_amd.quantize_weight(W)
+            layer[name] = (llmmm_amd.preshuffle_weight(q), sc)
+            del W, q
+        weights.append(layer)
+    h0 = torch.randn((M, hidden), generator=g, device="cuda").to(torch.bfloat16)
+    h1, h2 = torch.empty_like(h0), torch.empty_like(h0)
+    wn = torch.ones(hidden, device="cuda")
+    wh = torch.ones(128, device="cuda")
+    Aq, As = llmmm_amd.rmsnorm_quantize_activation(h0, wn, 1e-6)
+    attn_q, attn_s = llmmm_amd.quantize_activation(torch.randn((M, 4096), generator=g, device="cuda"))
+    inv = 1e6 ** (-torch.arange(64, device="cuda", dtype=torch.float64) / 64)
+    ang = torch.arange(4096, device="cuda", dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang).float().contiguous(), torch.sin(ang).float().contiguous()
+    pos = torch.full((M,), 1234, device="cuda", dtype=torch.int32)
+    Hq = torch.empty((M, inter), dtype=torch.uint8, device="cuda")
+    Hs = torch.empty((inter // 128, M), dtype=torch.float32, device="cuda")
+
+    def ws_for(fn, n, k):
+        return torch.empty(max(16, int(fn(M, n, k))), dtype=torch.uint8, device="cuda")
+
+    ws_qkv = ws_for(_lib.lib.llmmm_fp8_gemm_qkv_rope_workspace, *shapes["qkv"])
+    ws_o = ws_for(_lib.lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace, *shapes["o"])
+    ws_gu = llmmm_amd.make_workspace(_lib.OUT_FP8Q_SWIGLU, M, *shapes["gate_up"])
+    ws_d = ws_for(_lib.lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace, *shapes["down"])
+    state = {"i": 0}
+
+    def step():
+        L = weights[state["i"] % copies]
+        state["i"] += 1
+        llmmm_amd.fp8_gemm_qkv_rope(Aq, As, L["qkv"][0], L["qkv"][1], wh, wh, 1e-6, cos, sin, pos, n_q, n_kv, M, 6144, hidden, workspace=ws_qkv,
+                                    b_preshuffled=True)
+        q2, s2 = llmmm_amd.fp8_gemm_add_rmsnorm_quant(attn_q, attn_s, L["o"][0], L["o"][1], h0, h1, wn, 1e-6, M, hidden, 4096, workspace=ws_o,
+                                                      b_preshuffled=True)
+        llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(q2, s2, L["gate_up"][0], L["gate_up"][1], Hq, Hs, M, 2 * inter,
+                                                                                           hidden, workspace=ws_gu, b_preshuffled=True)
+        llmmm_amd.fp8_gemm_add_rmsnorm_quant(Hq, Hs, L["down"][0], L["down"][1], h1, h2, wn, 1e-6, M, hidden, inter, workspace=ws_d, b_preshuffled=True)
+
+    ms, _ = _events_ms(step, steps, warmup, graph=True)
+    return {"name": "qwen3_4b_decoder_layer_gemms_m%d" % M, "M": M, "us": ms * 1e3, "weight_bytes": per_copy, "hbm_gbs": per_copy / ms * 1e-6,
+            "frac_of_hbm_peak": per_copy / ms * 1e-6 / PEAK_HBM_GBS, "weight_copies": copies,
+            "launches": "qkv+norm+rope (2 kernels), o+add+norm+quant (2), gate_up+swiglu (2), down+add+norm+quant (2); attention not included"}
+
+
 def measured_peaks():
     """What this GPU sustains, next to the nominal peaks: register-only MFMA loops (the counterpart of the reference's
     test_fp8_peak_work, examples/005.fp8.test.cu:19-71) on zero and on random operands, and a streaming read."""
@@ -522,6 +583,10 @@ def main():
         # QKV projection + per-head RMSNorm + RoPE in one entry point, beside the plain bf16-output GEMM
         for m in (1, 16, 128, 2048):
             shapes.append(bench_qkv_rope(m, s2 * 2 if m <= 16 else s2, w2))
+            torch.cuda.empty_cache()
+        # the GEMM side of a whole decoder layer through the four fused entry points
+        for m in (1, 16):
+            shapes.append(bench_decoder_layer(m, s2, w2))
             torch.cuda.empty_cache()
         line["shapes"] = shapes
 
