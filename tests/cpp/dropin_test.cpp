@@ -128,6 +128,66 @@ int main()
     if (!throws_with([&] { LLMMM::transpose_matrix__aligned_128(dT, dAq, 100, K, nullptr); }, "M or N can't be divided 128.")) { ++fails; printf("transpose misaligned: FAIL\n"); }
     if (!throws_with([&] { LLMMM::construct_m16n8k32_B_layout(dBp, dBq, N, 100, nullptr); }, "K must be greater than 0 and divisible by 128.")) { ++fails; printf("layout misaligned K: FAIL\n"); }
   }
+  // ---- fused decoder-block entry points (planned by the reference, README.md:16): closed forms
+  {
+    // residual = -C32  =>  hidden == 0 exactly, codes and scales all zero; residual = 0  =>  hidden == C32 bit for bit
+    std::vector<float> hC32(M * N), hNeg(M * N), hOnes(N, 1.f);
+    CHECK(hipMemcpy(hC32.data(), dC32, hC32.size() * 4, hipMemcpyDeviceToHost));
+    for (size_t i = 0; i < hC32.size(); ++i) hNeg[i] = -hC32[i];
+    float *dRes, *dHid, *dW, *dQs;
+    LLMMM::fp8_t* dQ;
+    void*         dWs;
+    const size_t  wsz = llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K) + 16 * (size_t)M * N * 4;
+    CHECK(hipMalloc(&dRes, M * N * 4)); CHECK(hipMalloc(&dHid, M * N * 4)); CHECK(hipMalloc(&dW, N * 4)); CHECK(hipMalloc(&dQ, M * N));
+    CHECK(hipMalloc(&dQs, (N / 128) * M * 4)); CHECK(hipMalloc(&dWs, wsz));
+    CHECK(hipMemcpy(dRes, hNeg.data(), hNeg.size() * 4, hipMemcpyHostToDevice));
+    CHECK(hipMemcpy(dW, hOnes.data(), hOnes.size() * 4, hipMemcpyHostToDevice));
+    LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__add_rmsnorm__output_fp8<float>(dAq, dAs, dBq, dBs, dRes, dHid, dW, 1e-6f, dQ, dQs, M, N, K, dWs, wsz, nullptr);
+    CHECK(hipDeviceSynchronize());
+    std::vector<float>         hHid(M * N), hQs((N / 128) * M);
+    std::vector<unsigned char> hQ(M * N);
+    CHECK(hipMemcpy(hHid.data(), dHid, hHid.size() * 4, hipMemcpyDeviceToHost));
+    CHECK(hipMemcpy(hQ.data(), dQ, hQ.size(), hipMemcpyDeviceToHost));
+    CHECK(hipMemcpy(hQs.data(), dQs, hQs.size() * 4, hipMemcpyDeviceToHost));
+    int ff = 0;
+    for (float v : hHid) if (v != 0.f) ++ff;
+    for (unsigned char v : hQ) if ((v & 0x7f) != 0) ++ff;
+    for (float v : hQs) if (v != 0.f) ++ff;
+    CHECK(hipMemset(dRes, 0, M * N * 4));
+    LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__add_rmsnorm__output_fp8<float>(dAq, dAs, dBq, dBs, dRes, dHid, dW, 1e-6f, dQ, dQs, M, N, K, dWs, wsz, nullptr);
+    CHECK(hipDeviceSynchronize());
+    CHECK(hipMemcpy(hHid.data(), dHid, hHid.size() * 4, hipMemcpyDeviceToHost));
+    if (memcmp(hHid.data(), hC32.data(), hC32.size() * 4) != 0) ++ff;
+    printf("GEMM + residual + RMSNorm + quant closed forms (residual = -C, residual = 0): %s\n", ff ? "FAIL" : "ok");
+    fails += ff;
+    // rope at angle 0 without norm == the plain bf16-output GEMM (3 heads: N = 384)
+    const int NH = 384;
+    std::vector<float> fB(NH * K);
+    for (auto& v : fB) { s = s * 1664525u + 1013904223u; v = ((s >> 8) / 16777216.0f) * 0.1f - 0.05f; }
+    float *dfB, *dBs3, *dCos, *dSin;
+    int*   dPos;
+    LLMMM::fp8_t* dBq3;
+    void *dY0, *dY1;
+    CHECK(hipMalloc(&dfB, fB.size() * 4)); CHECK(hipMalloc(&dBq3, NH * K)); CHECK(hipMalloc(&dBs3, (NH / 128) * (K / 128) * 4));
+    CHECK(hipMalloc(&dCos, 64 * 4)); CHECK(hipMalloc(&dSin, 64 * 4)); CHECK(hipMalloc(&dPos, M * 4)); CHECK(hipMalloc(&dY0, M * NH * 2)); CHECK(hipMalloc(&dY1, M * NH * 2));
+    std::vector<float> one64(64, 1.f);
+    CHECK(hipMemcpy(dfB, fB.data(), fB.size() * 4, hipMemcpyHostToDevice));
+    CHECK(hipMemcpy(dCos, one64.data(), 64 * 4, hipMemcpyHostToDevice));
+    CHECK(hipMemset(dSin, 0, 64 * 4)); CHECK(hipMemset(dPos, 0, M * 4));
+    LLMMM::fp8_blockwise_symmetric_quantization<128, 128, false>(dfB, dBq3, dBs3, NH, K, nullptr);
+    LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(dAq, dAs, dBq3, dBs3, dY0, M, NH, K, nullptr);
+    LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__qk_norm_rope__output_bf16(dAq, dAs, dBq3, dBs3, dY1, nullptr, nullptr, 1e-6f, dCos, dSin, 1, dPos, 1, 1, M, NH,
+                                                                                 K, dWs, wsz, nullptr);
+    CHECK(hipDeviceSynchronize());
+    std::vector<unsigned short> hY0(M * NH), hY1(M * NH);
+    CHECK(hipMemcpy(hY0.data(), dY0, hY0.size() * 2, hipMemcpyDeviceToHost));
+    CHECK(hipMemcpy(hY1.data(), dY1, hY1.size() * 2, hipMemcpyDeviceToHost));
+    const int fr = memcmp(hY0.data(), hY1.data(), hY0.size() * 2) != 0;
+    printf("QKV + rope at angle 0 == plain bf16 GEMM: %s\n", fr ? "FAIL" : "ok");
+    fails += fr;
+    if (!throws_with([&] { LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__add_rmsnorm__output_fp8<float>(dAq, dAs, dBq, dBs, dRes, dHid, dW, 1e-6f, dQ, dQs, M, 100, K, dWs, wsz, nullptr); },
+                     "M or N or K are not aligned.")) { ++fails; printf("fused misaligned N: FAIL\n"); }
+  }
   printf(fails ? "DROPIN FAIL (%d)\n" : "DROPIN OK\n", fails);
   return fails ? 1 : 0;
 }
