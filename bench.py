@@ -321,6 +321,7 @@ def bench_decoder_layer(M, steps, warmup, rotate_bytes=768 << 20):
     pos = torch.full((M,), 1234, device="cuda", dtype=torch.int32)
     Hq = torch.empty((M, inter), dtype=torch.uint8, device="cuda")
     Hs = torch.empty((inter // 128, M), dtype=torch.float32, device="cuda")
+    G32 = torch.empty((M, 2 * inter), dtype=torch.float32, device="cuda")
 
     def ws_for(fn, n, k):
         return torch.empty(max(16, int(fn(M, n, k))), dtype=torch.uint8, device="cuda")
@@ -338,14 +339,23 @@ def bench_decoder_layer(M, steps, warmup, rotate_bytes=768 << 20):
                                     b_preshuffled=True)
         q2, s2 = llmmm_amd.fp8_gemm_add_rmsnorm_quant(attn_q, attn_s, L["o"][0], L["o"][1], h0, h1, wn, 1e-6, M, hidden, 4096, workspace=ws_o,
                                                       b_preshuffled=True)
-        llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(q2, s2, L["gate_up"][0], L["gate_up"][1], Hq, Hs, M, 2 * inter,
-                                                                                           hidden, workspace=ws_gu, b_preshuffled=True)
-        llmmm_amd.fp8_gemm_add_rmsnorm_quant(Hq, Hs, L["down"][0], L["down"][1], h1, h2, wn, 1e-6, M, hidden, inter, workspace=ws_d, b_preshuffled=True)
+        if M <= 4:
+            # the activation on the consumer's side: gate_up with fp32 output (one kernel), the down projection's kernel quantises
+            # silu(gate) * up itself
+            llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(q2, s2, L["gate_up"][0], L["gate_up"][1], G32, M, 2 * inter, hidden,
+                                                                               b_preshuffled=True)
+            llmmm_amd.fp8_gemm_add_rmsnorm_quant(G32, None, L["down"][0], L["down"][1], h1, h2, wn, 1e-6, M, hidden, inter, workspace=ws_d, b_preshuffled=True,
+                                                 a_swiglu=True)
+        else:
+            llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(q2, s2, L["gate_up"][0], L["gate_up"][1], Hq, Hs, M, 2 * inter,
+                                                                                               hidden, workspace=ws_gu, b_preshuffled=True)
+            llmmm_amd.fp8_gemm_add_rmsnorm_quant(Hq, Hs, L["down"][0], L["down"][1], h1, h2, wn, 1e-6, M, hidden, inter, workspace=ws_d, b_preshuffled=True)
 
     ms, _ = _events_ms(step, steps, warmup, graph=True)
     return {"name": "qwen3_4b_decoder_layer_gemms_m%d" % M, "M": M, "us": ms * 1e3, "weight_bytes": per_copy, "hbm_gbs": per_copy / ms * 1e-6,
             "frac_of_hbm_peak": per_copy / ms * 1e-6 / PEAK_HBM_GBS, "weight_copies": copies,
-            "launches": "qkv+norm+rope (2 kernels), o+add+norm+quant (2), gate_up+swiglu (2), down+add+norm+quant (2); attention not included"}
+            "launches": ("qkv+norm+rope (2 kernels), o+add+norm+quant (2), gate_up fp32 (1), down on silu(gate)*up +add+norm+quant (2)" if M <= 4 else
+                         "qkv+norm+rope (2 kernels), o+add+norm+quant (2), gate_up+swiglu (2), down+add+norm+quant (2)") + "; attention not included"}
 
 
 def measured_peaks():

@@ -69,10 +69,17 @@ extern "C" {
 #define LLMMM_FP8_B_ROWS 0        /* Bt[N,K] row-major, the reference layout (examples/005.fp8.mm.cu:157) */
 #define LLMMM_FP8_B_PRESHUFFLED 1 /* the image llmmm_fp8_preshuffle_b writes */
 
+/* What the FP8 GEMM's A argument points at (llmmm_gemm_cfg.a_layout). */
+#define LLMMM_FP8_A_QUANTISED 0  /* A [M,K] e4m3 + As [K/128, M]: the reference's operand (examples/005.fp8.mm.cu:157) */
+#define LLMMM_FP8_A_SWIGLU_F32 1 /* A is the fp32 result G [M, 2K] of a gate_up projection (llmmm_fp8_gemm with LLMMM_OUT_F32), As is
+                                  * ignored: the GEMM runs on quantise_1x128(silu(G[:, :K]) * G[:, K:]), which the kernel makes itself --
+                                  * see llmmm_fp8_swiglu_a_workspace */
+
 typedef struct llmmm_gemm_cfg {
   int tile;
   int split_k;
   int b_layout; /* FP8 only: LLMMM_FP8_B_ROWS (0, the default) or LLMMM_FP8_B_PRESHUFFLED; the FP16 GEMM ignores it */
+  int a_layout; /* FP8 only: LLMMM_FP8_A_QUANTISED (0, the default) or LLMMM_FP8_A_SWIGLU_F32 */
 } llmmm_gemm_cfg;
 
 /* ---- FP16 / BF16 GEMM -------------------------------------------------------------------
@@ -179,6 +186,16 @@ LLMMM_API int    llmmm_fp8_gemm_qkv_rope(int out_kind, const void* A, const floa
                                          int n_q_heads, int n_kv_heads, int M, int N, int K, void* workspace, size_t workspace_bytes,
                                          const llmmm_gemm_cfg* cfg, void* stream);
 LLMMM_API size_t llmmm_fp8_gemm_qkv_rope_workspace(int M, int N, int K);
+
+/* The gated-MLP activation fused into the *consumer*: with cfg.a_layout = LLMMM_FP8_A_SWIGLU_F32, llmmm_fp8_gemm_ex and
+ * llmmm_fp8_gemm_add_rmsnorm_quant (the down projection) take the fp32 gate_up result G [M, 2K] as their A argument and run on
+ * h = silu(G[:, :K]) * G[:, K:] quantised 1x128 -- the operand LLMMM_OUT_FP8Q_SWIGLU would have written, bit for bit (planned by
+ * the reference, README.md:16; no reference kernel).  For M <= 4 every workgroup of the weight-streaming kernel makes the
+ * slices of h it needs while its first weights are in flight, so the activation costs no launch (gate_up: one kernel with fp32
+ * output; down: its usual kernels; K / 128 / split_k <= 32).  Otherwise the library quantises h into the front of the workspace
+ * first, which then must hold llmmm_fp8_swiglu_a_workspace(M, N, K) bytes (0 when the kernel does it itself) on top of what
+ * the GEMM wants. */
+LLMMM_API size_t llmmm_fp8_swiglu_a_workspace(int M, int N, int K);
 
 /* ---- offline layout helpers --------------------------------------------------------------
  * llmmm_fp8_preshuffle_b takes the role of  construct_m16n8k32_B_layout(dst, src_transposed, N, K,

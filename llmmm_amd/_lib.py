@@ -20,12 +20,13 @@ B_ROW_MAJOR, B_TRANSPOSED = 0, 1
 OUT_F32, OUT_BF16, OUT_FP8Q, OUT_FP8Q_SWIGLU = 0, 1, 2, 3
 QUANT_1x128_T, QUANT_128x128, QUANT_1x128, QUANT_128x128_T = 0, 1, 2, 3
 FP8_B_ROWS, FP8_B_PRESHUFFLED = 0, 1
+FP8_A_QUANTISED, FP8_A_SWIGLU_F32 = 0, 1
 PROBE_FP8 = 2
 TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_64x128, TILE_SKINNY = -1, 0, 1, 2, 3, 4, 8
 
 
 class GemmCfg(ctypes.Structure):
-    _fields_ = [("tile", ctypes.c_int), ("split_k", ctypes.c_int), ("b_layout", ctypes.c_int)]
+    _fields_ = [("tile", ctypes.c_int), ("split_k", ctypes.c_int), ("b_layout", ctypes.c_int), ("a_layout", ctypes.c_int)]
 
 
 # name -> (restype, argtypes); must list every symbol include/llmmm.h declares
@@ -46,6 +47,7 @@ SIGNATURES = {
     "llmmm_fp8_gemm_qkv_rope": (_i, [_i, _vp, _fp, _vp, _fp, _vp, _fp, _fp, _fp, _c.c_float, _fp, _fp, _i, _vp, _i, _i, _i, _i, _i, _vp, _sz,
                                      _c.POINTER(GemmCfg), _vp]),
     "llmmm_fp8_gemm_qkv_rope_workspace": (_sz, [_i, _i, _i]),
+    "llmmm_fp8_swiglu_a_workspace": (_sz, [_i, _i, _i]),
     "llmmm_fp8_preshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
     "llmmm_fp8_unshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
     "llmmm_transpose": (_i, [_i, _vp, _vp, _i, _i, _vp]),

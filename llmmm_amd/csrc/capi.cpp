@@ -114,6 +114,7 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
   cfg->tile     = -1;
   cfg->split_k  = 0;
   cfg->b_layout = LLMMM_FP8_B_ROWS;
+  cfg->a_layout = LLMMM_FP8_A_QUANTISED;
   if (M % 128 == 0)
     for (const auto& e : llmmm::kTileTune)
       if (e.M == M && e.N == N && e.K == K) {
@@ -248,6 +249,53 @@ size_t llmmm_fp8_gemm_workspace(int out_kind, int M, int N, int K)
   return (size_t)(s < 1 ? 1 : s) * M * N * sizeof(float);
 }
 
+// cfg.a_layout = LLMMM_FP8_A_SWIGLU_F32: the weight-streaming kernel makes the activations itself for M <= 4 when a
+// split's K range fits its staging buffer (32 slices of 128); otherwise h is quantised into the front of the workspace.
+// (Every column group's workgroup repeats the activation work of its K range, so its cost grows with M: measured on the
+// Qwen3-4B down projection, +0.8 us at M = 1, +1.8 at M = 4, +2.5 at M = 8, +4.6 at M = 16, against the 2.4 us that the
+// separate SwiGLU quantiser launch costs.  The kernel itself takes up to 16 rows.)
+constexpr int AGEN_MAX_M = 4, AGEN_MAX_SLICES = 32;
+static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+static size_t swiglu_a_bytes(int M, int K) { return align256((size_t)M * K) + align256((size_t)(K / 128) * M * sizeof(float)); }
+static int agen_min_split(int K) { return ((K / 128) + AGEN_MAX_SLICES - 1) / AGEN_MAX_SLICES; }
+
+size_t llmmm_fp8_swiglu_a_workspace(int M, int N, int K)
+{
+  llmmm_gemm_cfg cfg;
+  if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
+  if (cfg.tile == LLMMM_TILE_SKINNY && M <= AGEN_MAX_M) return 0;
+  return swiglu_a_bytes(M, K);
+}
+
+// Resolves a_layout for a call whose kernel choice is `tile`: either the kernel generates A (*agen = true, A stays the
+// fp32 pointer), or h is quantised into the workspace now and A / As / workspace are redirected to it.
+static int prepare_a(const llmmm_gemm_cfg* user, int tile, const void*& A, const float*& As, int M, int K, void*& workspace, size_t& workspace_bytes,
+                     void* stream, bool* agen)
+{
+  *agen = false;
+  if (!user || user->a_layout == LLMMM_FP8_A_QUANTISED) return LLMMM_OK;
+  if (user->a_layout != LLMMM_FP8_A_SWIGLU_F32) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown A layout %d", user->a_layout);
+  if ((long)M * 2 * K >= (1L << 31)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
+  if (tile == LLMMM_TILE_SKINNY && M <= AGEN_MAX_M) {
+    *agen = true;
+    return LLMMM_OK;
+  }
+  const size_t need = swiglu_a_bytes(M, K);
+  if (!workspace || workspace_bytes < need)
+    return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, quantising the SwiGLU activations first needs %zu", workspace ? workspace_bytes : (size_t)0, need);
+  if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+  uint8_t* hq = (uint8_t*)workspace;
+  float*   hs = (float*)(hq + align256((size_t)M * K));
+  const hipError_t e = llmmm::fp8_splitk_reduce_launch(LLMMM_OUT_FP8Q_SWIGLU, (const float*)A, 1, hq, hs, M, 2 * K, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "SwiGLU quantiser launch: %s", hipGetErrorString(e));
+  A               = hq;
+  As              = hs;
+  workspace       = hq + need;
+  workspace_bytes = workspace_bytes - need;
+  if (workspace_bytes == 0) workspace = nullptr;
+  return LLMMM_OK;
+}
+
 int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
                       int N, int K, void* workspace, size_t workspace_bytes, const llmmm_gemm_cfg* user, void* stream)
 {
@@ -256,7 +304,9 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
   llmmm_gemm_cfg cfg;
   const int      rc = choose_fp8_out(out_kind, M, N, K, &cfg);
   if (rc) return rc;
-  if (!A || !As || !Bt || !Bs || !C) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  const bool a_swiglu = user && user->a_layout == LLMMM_FP8_A_SWIGLU_F32;
+  if (!A || (!As && !a_swiglu) || !Bt || !Bs || !C) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (a_swiglu && swiglu) return fail(LLMMM_ERR_INVALID_ARGUMENT, "SwiGLU on both the A operand and the output");
   if ((out_kind == LLMMM_OUT_FP8Q || swiglu) && !Cs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "C_scale_transposed is required for fp8 output");
   if (!aligned16(A) || !aligned16(Bt) || !aligned16(C)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
   if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
@@ -269,18 +319,29 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
     cfg.b_layout = user->b_layout;
   }
   hipError_t e;
+  bool       agen = false;
+  if (cfg.tile == LLMMM_TILE_SKINNY && M > SKINNY_MAX_M) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the weight-streaming kernel handles M <= %d", SKINNY_MAX_M);
+  const int rca = prepare_a(user, cfg.tile, A, As, M, K, workspace, workspace_bytes, stream, &agen);
+  if (rca) return rca;
   if (cfg.tile == LLMMM_TILE_SKINNY) {
-    if (M > SKINNY_MAX_M) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the weight-streaming kernel handles M <= %d", SKINNY_MAX_M);
     int split = cfg.split_k;
     if (split > max_split_for(K)) split = max_split_for(K);
     if (split < 1) split = 1;
     if (!workspace) split = 1;  // documented: no workspace, no split
+    const int min_split = agen ? agen_min_split(K) : 1;  // generated activations: a split's K range must fit the staging buffer
+    if (split < min_split) {
+      if ((user && user->split_k > 0) || !workspace)
+        return fail(user && user->split_k > 0 ? LLMMM_ERR_INVALID_ARGUMENT : LLMMM_ERR_WORKSPACE,
+                    "generated activations need split-K >= %d for K = %d (at most %d slices of 128 per split), and a workspace for it", min_split, K, AGEN_MAX_SLICES);
+      split = min_split;
+    }
     float* partial = nullptr;
     if (swiglu && !workspace) return fail(LLMMM_ERR_WORKSPACE, "the SwiGLU output at M <= %d needs a workspace of at least M * N floats", SKINNY_MAX_M);
     if (split > 1 && !(user && user->split_k > 0)) {
       // a split the library chose itself shrinks to what the caller's workspace holds
       const size_t room = workspace_bytes / ((size_t)M * N * sizeof(float));
       if ((size_t)split > room) split = room < 2 ? 1 : (int)room;
+      if (split < min_split) split = min_split;  // (fails the size check below)
     }
     if (split > 1 || swiglu) {
       const size_t need = (size_t)split * M * N * sizeof(float);
@@ -288,7 +349,11 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
       if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
       partial = (float*)workspace;
     }
-    e = llmmm::fp8_skinny_launch(partial ? LLMMM_OUT_F32 : out_kind, cfg.b_layout, A, As, Bt, Bs, C, Cs, M, N, K, split, partial, (hipStream_t)stream);
+    if (agen)
+      e = llmmm::fp8_skinny_swiglu_a_launch(partial ? LLMMM_OUT_F32 : out_kind, cfg.b_layout, (const float*)A, Bt, Bs, C, Cs, M, N, K, split, partial,
+                                            (hipStream_t)stream);
+    else
+      e = llmmm::fp8_skinny_launch(partial ? LLMMM_OUT_F32 : out_kind, cfg.b_layout, A, As, Bt, Bs, C, Cs, M, N, K, split, partial, (hipStream_t)stream);
     if (e == hipSuccess && partial) e = llmmm::fp8_splitk_reduce_launch(out_kind, partial, split, C, Cs, M, N, (hipStream_t)stream);
   }
   else {
@@ -403,15 +468,16 @@ size_t llmmm_fp8_gemm_add_rmsnorm_quant_workspace(int M, int N, int K)
 // and the workspace has been checked to hold them.
 struct PlaneCfg {
   int  tile = 0, split = 0, b_layout = 0;
-  bool skinny = false;
+  bool skinny = false, agen = false;
 };
-static int resolve_plane_cfg(const void* A, const float* As, const void* Bt, const float* Bs, int M, int N, int K, void* workspace,
-                             size_t workspace_bytes, const llmmm_gemm_cfg* user, bool allow_direct, PlaneCfg* out)
+static int resolve_plane_cfg(const void*& A, const float*& As, const void* Bt, const float* Bs, int M, int N, int K, void*& workspace,
+                             size_t& workspace_bytes, const llmmm_gemm_cfg* user, bool allow_direct, PlaneCfg* out, void* stream)
 {
   llmmm_gemm_cfg cfg;
   const int      rc = choose_fp8(M, N, K, &cfg);
   if (rc) return rc;
-  if (!A || !As || !Bt || !Bs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  const bool a_swiglu = user && user->a_layout == LLMMM_FP8_A_SWIGLU_F32;
+  if (!A || (!As && !a_swiglu) || !Bt || !Bs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
   if (!aligned16(A) || !aligned16(Bt)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
   if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
@@ -432,10 +498,18 @@ static int resolve_plane_cfg(const void* A, const float* As, const void* Bt, con
     if (M % bm || N % bn) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
     if (user && user->tile != LLMMM_TILE_AUTO && user->split_k <= 0) cfg.split_k = heuristic_tile_split(cfg.tile, M, N, K);
   }
+  // the A operand given as the fp32 gate_up result: generated by the kernel, or quantised into the front of the workspace now
+  const int rca = prepare_a(user, cfg.tile, A, As, M, K, workspace, workspace_bytes, stream, &out->agen);
+  if (rca) return rca;
   int split = cfg.split_k < 1 ? 1 : cfg.split_k;
   if (split > max_split_for(K)) split = max_split_for(K);
   const size_t plane    = (size_t)M * N * sizeof(float);
   const bool   explicit_split = user && user->split_k > 0;
+  const int    min_split = out->agen ? agen_min_split(K) : 1;
+  if (split < min_split) {
+    if (explicit_split) return fail(LLMMM_ERR_INVALID_ARGUMENT, "generated activations need split-K >= %d for K = %d", min_split, K);
+    split = min_split;
+  }
   out->tile = cfg.tile, out->b_layout = cfg.b_layout, out->skinny = skinny;
   if (allow_direct && !skinny && (split == 1 || (!explicit_split && (!workspace || workspace_bytes < 2 * plane)))) {
     out->split = 0;  // also when a split the library chose itself finds no room for two planes
@@ -446,6 +520,7 @@ static int resolve_plane_cfg(const void* A, const float* As, const void* Bt, con
   if ((size_t)split * plane > workspace_bytes) {
     if (explicit_split) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace_bytes, split, (size_t)split * plane);
     split = (int)(workspace_bytes / plane);  // a split the library chose itself shrinks to the workspace (>= 1: checked above)
+    if (split < min_split) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, generated activations need split-K %d: %zu", workspace_bytes, min_split, (size_t)min_split * plane);
   }
   out->split = split;
   return LLMMM_OK;
@@ -456,7 +531,9 @@ static int launch_into_planes(const PlaneCfg& pc, const void* A, const float* As
 {
   float*     planes = (float*)workspace;
   hipError_t e;
-  if (pc.skinny)
+  if (pc.skinny && pc.agen)
+    e = llmmm::fp8_skinny_swiglu_a_launch(LLMMM_OUT_F32, pc.b_layout, (const float*)A, Bt, Bs, nullptr, nullptr, M, N, K, pc.split, planes, (hipStream_t)stream);
+  else if (pc.skinny)
     e = llmmm::fp8_skinny_launch(LLMMM_OUT_F32, pc.b_layout, A, As, Bt, Bs, nullptr, nullptr, M, N, K, pc.split, planes, (hipStream_t)stream);
   else
     e = llmmm::fp8_gemm_launch(LLMMM_OUT_F32, pc.tile, pc.b_layout, A, As, Bt, Bs, nullptr, nullptr, M, N, K, pc.split, planes, (hipStream_t)stream);
@@ -479,7 +556,7 @@ int llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As, const void*
   if (!aligned16(residual) || !aligned16(hidden_out) || !aligned16(norm_weight) || !aligned16(q))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
   PlaneCfg pc;
-  int      rc = resolve_plane_cfg(A, As, Bt, Bs, M, N, K, workspace, workspace_bytes, user, true, &pc);
+  int      rc = resolve_plane_cfg(A, As, Bt, Bs, M, N, K, workspace, workspace_bytes, user, true, &pc, stream);
   if (rc) return rc;
   if (pc.split == 0) {
     // a tile kernel without split: the residual is added in its epilogue, the norm + quantiser kernel follows on the
@@ -525,7 +602,7 @@ int llmmm_fp8_gemm_qkv_rope(int out_kind, const void* A, const float* As, const 
       (k_norm_weight && !aligned16(k_norm_weight)) || (reinterpret_cast<uintptr_t>(positions) & 3u))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned (positions: 4-byte)");
   PlaneCfg pc;
-  int      rc = resolve_plane_cfg(A, As, Bt, Bs, M, N, K, workspace, workspace_bytes, user, true, &pc);
+  int      rc = resolve_plane_cfg(A, As, Bt, Bs, M, N, K, workspace, workspace_bytes, user, true, &pc, stream);
   if (rc) return rc;
   if (pc.split == 0) {  // a tile kernel without split: norm and rope run on the accumulators, no planes
     llmmm::Fp8HeadOp op;

@@ -193,4 +193,12 @@ __device__ __forceinline__ void store_row4<_Float16>(_Float16* p, f32x4 v)
   *(f16x4*)p = f16x4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
 }
 
+// silu(g) * u with the hardware's exp2 and reciprocal (each within about one ulp of fp32): far below the
+// resolution of the e4m3 codes the result is quantised to.  g -> -inf gives -0, g -> +inf gives g * u.
+__device__ __forceinline__ float silu_mul(float g, float u)
+{
+  const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896340736f);  // exp(-g)
+  return g * __builtin_amdgcn_rcpf(1.f + e) * u;
+}
+
 }  // namespace llmmm

@@ -247,14 +247,6 @@ __device__ __forceinline__ uint32_t pack_e4m3x4_in_range(float a, float b, float
   return (uint32_t)v;
 }
 
-// silu(g) * u with the hardware's exp2 and reciprocal (each within about one ulp of fp32): far below the
-// resolution of the e4m3 codes the result is quantised to.  g -> -inf gives -0, g -> +inf gives g * u.
-__device__ __forceinline__ float silu_mul(float g, float u)
-{
-  const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896340736f);  // exp(-g)
-  return g * __builtin_amdgcn_rcpf(1.f + e) * u;
-}
-
 // SwiGLU exchange: the fragments mf = SEND0 .. SEND0 + MF/2 - 1 go to the partner wave through LDS, lane for lane.
 template <int MF, int SEND0>
 __device__ __forceinline__ void swiglu_send(const f32x4 (&acc)[8][MF], char LLMMM_LDS* region, int lane)

@@ -63,7 +63,7 @@ __device__ __forceinline__ void skinny_stream_lds_16B(const void* gptr, unsigned
 
 // All vector-memory loads of a slot, in a fixed order, as inline assembly (see device_common.hip.h):
 // the kernel counts them itself.
-template <int MBLK, bool APRE>
+template <int MBLK, bool APRE, bool SA_LDS = false>
 __device__ __forceinline__ void skinny_fetch(SkinnySlot<MBLK, APRE>& t, unsigned ring_slot, const uint8_t* wrow, int w_kstep,
                                              unsigned w_off0, unsigned w_off1, const uint8_t* const (&ap)[MBLK], const float* const (&asp)[MBLK],
                                              const float* bsp, int kb, int M)
@@ -76,18 +76,21 @@ __device__ __forceinline__ void skinny_fetch(SkinnySlot<MBLK, APRE>& t, unsigned
       asm_load_16B(t.a[mb][0], ap[mb] + (size_t)kb * 128);
       asm_load_16B(t.a[mb][1], ap[mb] + (size_t)kb * 128 + 16);
     }
-    asm_load_f32(t.sa[mb], asp[mb] + (size_t)kb * M);
+    if constexpr (!SA_LDS) asm_load_f32(t.sa[mb], asp[mb] + (size_t)kb * M);
   }
   t.sb = bsp[kb];
 }
 
 // s_waitcnt vmcnt(N) that also "touches" the slot's registers, so that nothing reading them can
 // be moved in front of it.
-template <int N, int MBLK, bool APRE>
+template <int N, int MBLK, bool APRE, bool SA_LDS = false>
 __device__ __forceinline__ void skinny_wait(SkinnySlot<MBLK, APRE>& t)
 {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-  if constexpr (APRE) {
+  if constexpr (SA_LDS) {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");  // the slot holds no registers of its own: everything it waits for lands in LDS
+  }
+  else if constexpr (APRE) {
     if constexpr (MBLK == 1)
       asm volatile("s_waitcnt vmcnt(%1)" : "+v"(t.sa[0]) : "n"(N) : "memory");
     else if constexpr (MBLK == 2)
@@ -117,9 +120,11 @@ __device__ __forceinline__ void skinny_wait(SkinnySlot<MBLK, APRE>& t)
 
 // With APRE the activation fragments come from the workgroup's staged copy: a_slice points at
 // the MBLK x 2 KB block of this slice, a_rd is the lane's SWZ_ROWS16 offset of (row i, chunk 2g).
-template <int MBLK, bool APRE>
+// With SA_LDS the row scales of the slice come from LDS as well (sa_slice: 16 floats, row i at [i]).
+template <int MBLK, bool APRE, bool SA_LDS = false>
 __device__ __forceinline__ void skinny_consume(const SkinnySlot<MBLK, APRE>& t, const char LLMMM_LDS* ring_slot, int w_rd, bool valid,
-                                               f32x4 (&acc)[MBLK], const char LLMMM_LDS* a_slice, int a_rd)
+                                               f32x4 (&acc)[MBLK], const char LLMMM_LDS* a_slice, int a_rd, const float LLMMM_LDS* sa_slice = nullptr,
+                                               int row = 0)
 {
   union {
     i32x4 h[2];
@@ -137,7 +142,12 @@ __device__ __forceinline__ void skinny_consume(const SkinnySlot<MBLK, APRE>& t, 
       af.h[0] = t.a[mb][0];
       af.h[1] = t.a[mb][1];
     }
-    const float s = valid ? t.sa[mb] * t.sb : 0.f;
+    float sa;
+    if constexpr (SA_LDS)
+      sa = sa_slice[row];
+    else
+      sa = t.sa[mb];
+    const float s = valid ? sa * t.sb : 0.f;
     const f32x4 z = {0.f, 0.f, 0.f, 0.f};
     const f32x4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf.v, af.v, z, 0, 0, 0, 0, 0, 0);
 #pragma unroll
@@ -149,14 +159,19 @@ __device__ __forceinline__ void skinny_consume(const SkinnySlot<MBLK, APRE>& t, 
 // the number of slices of the shortest split.
 // ASTG = bytes of LDS in which the workgroup stages its activation rows for the whole K range
 // of its split before the loop starts (0: the rows are fetched slice by slice into registers).
-template <int MBLK, int OUT, int D, int ASTG>
+// AGEN: the activations are not given quantised -- the workgroup makes them itself from the fp32 result G [M, 2K] of
+// the gate_up projection: h = silu(G[:, :K]) * G[:, K:], quantised 1x128, for the 16 rows and the K range it works on
+// (the arithmetic of the reduce kernel's SwiGLU output, so the codes and scales are the ones that kernel would have
+// written).  M <= 16.  A (then: G) and As (unused) keep their places in the argument list.
+template <int MBLK, int OUT, int D, int ASTG, bool AGEN = false>
 __global__ void __launch_bounds__(512)
 fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
                   const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int S,
                   float* __restrict__ partial, int bpre)
 {
   constexpr bool APRE  = ASTG > 0;
-  constexpr int  LOADS = SKINNY_LOADS_PER_SLOT_BASE + (APRE ? 1 : 3) * MBLK;  // vector-memory loads per slot, issued in slot order
+  static_assert(!AGEN || (MBLK == 1 && APRE), "generated activations: 16 rows, staged in LDS");
+  constexpr int  LOADS = SKINNY_LOADS_PER_SLOT_BASE + (AGEN ? 0 : (APRE ? 1 : 3) * MBLK);  // vector-memory loads per slot, issued in slot order
   static_assert(D * LOADS < 64, "vmcnt is a 6-bit counter");
   static_assert(MBLK <= 4 || APRE, "128-row groups only with staged activations");
   __shared__ __attribute__((aligned(1024))) char a_stage[APRE ? ASTG : 16];
@@ -170,6 +185,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   __shared__ __attribute__((aligned(1024))) char ring6[D > 4 ? 8 * 2048 : 16];
   __shared__ __attribute__((aligned(1024))) char ring7[D > 4 ? 8 * 2048 : 16];
   __shared__ float    wave_amax[8][MBLK][16];
+  __shared__ float    a_scale[AGEN ? (ASTG / 2048) * 16 : 1];  // AGEN: the generated row scales, [slice][row]
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -222,7 +238,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   // they have landed.
   const char LLMMM_LDS* const a_tile = (const char LLMMM_LDS*)a_stage;
   const int                   a_rd   = kmajor_offset<SWZ_ROWS16>(i, 2 * g);
-  if constexpr (APRE) {
+  if constexpr (APRE && !AGEN) {
     const unsigned a_addr = (unsigned)(size_t)(char LLMMM_LDS*)a_stage;
     const int      units  = (kb1 - kb0) * 2 * MBLK;
     for (int u = wave; u < units; u += 8) {
@@ -241,10 +257,53 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   SkinnySlot<MBLK, APRE> slot[D];
 #pragma unroll
   for (int u = 0; u < D; ++u) {
-    skinny_fetch<MBLK, APRE>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb0 + u, kb1 - 1), M);
+    skinny_fetch<MBLK, APRE, AGEN>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb0 + u, kb1 - 1), M);
     __builtin_amdgcn_sched_barrier(0);
   }
-  if constexpr (APRE) {
+  if constexpr (AGEN) {
+    // Behind the ring prologue (the weights are on their way): half a wavefront per row, a lane per four columns of a
+    // slice.  The loads below are ordinary ones; the waits the compiler puts behind them also cover the ring loads
+    // issued above, which only makes the hand-counted waits of the loop trivially true for the first pass.
+    const float* G   = (const float*)A;
+    const int    l32 = tid & 31;
+    if (M < 16) {  // rows M .. 15 of every slice: zero codes, zero scales (their products are never stored)
+      for (int x = tid; x < (kb1 - kb0) * 128; x += 512) *(i32x4 LLMMM_LDS*)((char LLMMM_LDS*)a_stage + x * 16) = i32x4{0, 0, 0, 0};
+      for (int x = tid; x < (kb1 - kb0) * 16; x += 512) a_scale[x] = 0.f;
+      __syncthreads();
+    }
+    // (row, slice) tasks are dealt round-robin to the 16 half-waves: for M = 1 every half-wave has one slice to make
+    const int nsl = kb1 - kb0, rows = min(M, 16), tasks = nsl * rows;
+    for (int t0 = tid >> 5; t0 < tasks; t0 += 16 * 4) {  // four tasks of a half-wave in flight
+      f32x4 gv[4], uv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int    t  = min(t0 + 16 * u, tasks - 1), j = t / rows, r = t - j * rows;
+        const float* gp = G + (size_t)r * 2 * K + (size_t)(kb0 + j) * 128 + 4 * l32;
+        gv[u]           = *(const f32x4*)gp;
+        uv[u]           = *(const f32x4*)(gp + K);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int t = t0 + 16 * u;
+        if (t < tasks) {  // uniform over the half-wave
+          const int j = t / rows, r = t - j * rows;
+          f32x4     h;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) h[q] = silu_mul(gv[u][q], uv[u][q]);
+          float a = fmaxf(fmaxf(__builtin_fabsf(h[0]), __builtin_fabsf(h[1])), fmaxf(__builtin_fabsf(h[2]), __builtin_fabsf(h[3])));
+#pragma unroll
+          for (int step = 1; step <= 16; step <<= 1) a = wave_xor_max(a, step);
+          const float scale = a / 448.f;
+          const float inv   = a > 0.f ? 448.f / a : 0.f;
+          *(uint32_t LLMMM_LDS*)((char LLMMM_LDS*)a_stage + j * 2048 + kmajor_offset<SWZ_ROWS16>(r, l32 >> 2) + (l32 & 3) * 4) =
+            sk_pack_e4m3x4(h[0] * inv, h[1] * inv, h[2] * inv, h[3] * inv);
+          if (l32 == 0) a_scale[j * 16 + r] = scale;
+        }
+      }
+    }
+    __syncthreads();
+  }
+  else if constexpr (APRE) {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * LOADS) : "memory");
     __syncthreads();  // every wave's share of the staged activations is in LDS
   }
@@ -252,18 +311,20 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   for (; kb + D < kb1; kb += D) {  // passes followed by another pass: consume a slot, refill it
 #pragma unroll
     for (int u = 0; u < D; ++u) {
-      skinny_wait<(D - 1) * LOADS, MBLK, APRE>(slot[u]);
-      skinny_consume<MBLK, APRE>(slot[u], ring[u], w_rd, true, acc, a_tile + (kb + u - kb0) * (MBLK * 2048), a_rd);
+      skinny_wait<(D - 1) * LOADS, MBLK, APRE, AGEN>(slot[u]);
+      skinny_consume<MBLK, APRE, AGEN>(slot[u], ring[u], w_rd, true, acc, a_tile + (kb + u - kb0) * (MBLK * 2048), a_rd,
+                                       (const float LLMMM_LDS*)a_scale + (AGEN ? (kb + u - kb0) * 16 : 0), i);
       __builtin_amdgcn_sched_barrier(0);
-      skinny_fetch<MBLK, APRE>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb + u + D, kb1 - 1), M);
+      skinny_fetch<MBLK, APRE, AGEN>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb + u + D, kb1 - 1), M);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
 #define LLMMM_LAST(u)                                                              \
   if constexpr ((u) < D) {                                                         \
-    skinny_wait<(D - 1 - (u)) * LOADS, MBLK, APRE>(slot[u]);                       \
-    skinny_consume<MBLK, APRE>(slot[u], ring[u], w_rd, kb + (u) < kb1, acc,        \
-                               a_tile + (min(kb + (u), kb1 - 1) - kb0) * (MBLK * 2048), a_rd); \
+    skinny_wait<(D - 1 - (u)) * LOADS, MBLK, APRE, AGEN>(slot[u]);                 \
+    skinny_consume<MBLK, APRE, AGEN>(slot[u], ring[u], w_rd, kb + (u) < kb1, acc,  \
+                               a_tile + (min(kb + (u), kb1 - 1) - kb0) * (MBLK * 2048), a_rd, \
+                               (const float LLMMM_LDS*)a_scale + (AGEN ? (min(kb + (u), kb1 - 1) - kb0) * 16 : 0), i); \
     __builtin_amdgcn_sched_barrier(0);                                             \
   }
   LLMMM_LAST(0) LLMMM_LAST(1) LLMMM_LAST(2) LLMMM_LAST(3) LLMMM_LAST(4) LLMMM_LAST(5) LLMMM_LAST(6) LLMMM_LAST(7)
@@ -339,6 +400,37 @@ static hipError_t launch_skinny(const void* A, const float* As, const void* Bt, 
   hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D, ASTG>), dim3(N / 128, S, MBLK == 8 ? (M + 127) / 128 : (M + 63) / 64), dim3(512), 0, stream,
                      (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial, bpre);
   return hipGetLastError();
+}
+
+// Generated activations (AGEN): M <= 16, the K range of a split must fit the staging buffer.
+template <int OUT>
+static hipError_t dispatch_skinny_agen(const float* G, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K, int S, float* partial,
+                                       int bpre, hipStream_t stream)
+{
+  const int KB = K / 128, slices = KB / S, longest = (KB + S - 1) / S, need = 2048 * longest;
+  if (M > 16 || need > 65536) return hipErrorInvalidValue;
+#define LLMMM_GO(D, ASTG)                                                                                                                   \
+  {                                                                                                                                         \
+    hipLaunchKernelGGL((fp8_skinny_kernel<1, OUT, D, ASTG, true>), dim3(N / 128, S, 1), dim3(512), 0, stream, (const uint8_t*)G, (const float*)nullptr, \
+                       (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial, bpre);                                                           \
+    return hipGetLastError();                                                                                                               \
+  }
+  if (slices >= 8 && need <= 28672) LLMMM_GO(8, 28672);
+  if (slices >= 4) LLMMM_GO(4, 65536);
+  LLMMM_GO(2, 65536);
+#undef LLMMM_GO
+}
+
+hipError_t fp8_skinny_swiglu_a_launch(int out_kind, int b_layout, const float* G, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N,
+                                      int K, int S, float* partial, hipStream_t stream)
+{
+  const int bpre = b_layout == LLMMM_FP8_B_PRESHUFFLED;
+  switch (out_kind) {
+    case SK_OUT_F32: return dispatch_skinny_agen<SK_OUT_F32>(G, Bt, Bs, C, Cs, M, N, K, S, partial, bpre, stream);
+    case SK_OUT_BF16: return dispatch_skinny_agen<SK_OUT_BF16>(G, Bt, Bs, C, Cs, M, N, K, S, partial, bpre, stream);
+    case SK_OUT_FP8Q: return dispatch_skinny_agen<SK_OUT_FP8Q>(G, Bt, Bs, C, Cs, M, N, K, S, partial, bpre, stream);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 // Ring depth D: the largest that does not exceed the slices of the shortest split.  Activation

@@ -56,6 +56,11 @@ hipError_t fp8_splitk_reduce_launch(int out_kind, const float* planes, int S, vo
 hipError_t fp8_skinny_launch(int out_kind, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
                              float* Cs, int M, int N, int K, int S, float* partial, hipStream_t stream);
 
+// The same kernel making its activations itself from the fp32 gate_up result G [M, 2K]: A = quantise_1x128(silu(G[:, :K]) *
+// G[:, K:]), M <= 16, at most 32 slices of 128 per split (hipErrorInvalidValue otherwise).  partial as above.
+hipError_t fp8_skinny_swiglu_a_launch(int out_kind, int b_layout, const float* G, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N,
+                                      int K, int S, float* partial, hipStream_t stream);
+
 // Weights Bt[N,K] e4m3 (N % 16 == 0, K % 128 == 0) -> 2 KB blocks in MFMA operand order, or back (inverse != 0).
 hipError_t fp8_preshuffle_launch(int inverse, const void* src, void* dst, int N, int K, hipStream_t stream);
 

@@ -143,45 +143,53 @@ def query_config(out_kind, M, N, K):
     return cfg.tile, cfg.split_k
 
 
-def _fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, workspace, tile, split_k, stream, b_preshuffled=False):
+def _a_operand(A, As, M, K, a_swiglu):
+    """Pointers of the A operand: quantised codes + transposed scales, or (a_swiglu) the fp32 gate_up result [M, 2K]."""
+    kb = K // 128 if K % 128 == 0 else 0
+    if a_swiglu:
+        return _ptr(A, "A (fp32 gate_up result)", (torch.float32,), M * 2 * K), None
+    return _ptr(A, "A", _FP8_DTYPES, M * K), _ptr(As, "A_scale_transposed", (torch.float32,), kb * M)
+
+
+def _fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, workspace, tile, split_k, stream, b_preshuffled=False, a_swiglu=False):
     kb = K // 128 if K % 128 == 0 else 0
     c_dtypes = {_lib.OUT_F32: (torch.float32,), _lib.OUT_BF16: (torch.bfloat16,), _lib.OUT_FP8Q: _FP8_DTYPES, _lib.OUT_FP8Q_SWIGLU: _FP8_DTYPES}[out_kind]
     n_out = N // 2 if out_kind == _lib.OUT_FP8Q_SWIGLU else N  # SwiGLU halves the width
-    a_p = _ptr(A, "A", _FP8_DTYPES, M * K)
-    as_p = _ptr(As, "A_scale_transposed", (torch.float32,), kb * M)
+    a_p, as_p = _a_operand(A, As, M, K, a_swiglu)
     b_p = _ptr(Bt, "B_transposed", _FP8_DTYPES, N * K)
     bs_p = _ptr(Bs, "B_scale_transposed", (torch.float32,), ((N + 127) // 128) * kb)
     c_p = _ptr(C, "C", c_dtypes, M * n_out)
     cs_p = _ptr(Cs, "C_scale_transposed", (torch.float32,), ((n_out + 127) // 128) * M) if out_kind in (_lib.OUT_FP8Q, _lib.OUT_FP8Q_SWIGLU) else None
     ws_p, ws_n = (ctypes.c_void_p(workspace.data_ptr()), workspace.numel() * workspace.element_size()) if workspace is not None else (None, 0)
-    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS)
+    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS, _lib.FP8_A_SWIGLU_F32 if a_swiglu else _lib.FP8_A_QUANTISED)
     check(lib.llmmm_fp8_gemm_ex(out_kind, a_p, as_p, b_p, bs_p, c_p, cs_p, M, N, K, ws_p, ws_n, ctypes.byref(cfg), _stream(stream)))
 
 
 def fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(A, A_scale_transposed, B_transposed, B_scale_transposed, C, M, N, K,
                                                              stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0,
-                                                             b_preshuffled=False):
+                                                             b_preshuffled=False, a_swiglu=False):
     """examples/005.fp8.mm.cu:217-246.  C [M,N] float32.  ``b_preshuffled``: B_transposed is the image written by
-    :func:`construct_mfma_B_layout` instead of row-major [N,K] (same results, bit for bit)."""
+    :func:`construct_mfma_B_layout` instead of row-major [N,K] (same results, bit for bit).  ``a_swiglu``: A is the fp32
+    result [M, 2K] of a gate_up projection and the GEMM runs on quantise(silu(gate) * up) (A_scale_transposed: None)."""
     _fp8_gemm(_lib.OUT_F32, A, A_scale_transposed, B_transposed, B_scale_transposed, C, None, M, N, K, workspace, tile, split_k, stream,
-              b_preshuffled)
+              b_preshuffled, a_swiglu)
 
 
 def fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(A, A_scale_transposed, B_transposed, B_scale_transposed, C, M, N, K,
                                                              stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0,
-                                                             b_preshuffled=False):
+                                                             b_preshuffled=False, a_swiglu=False):
     """The fp32 variant's result rounded to bfloat16 (no reference kernel; same signature)."""
     _fp8_gemm(_lib.OUT_BF16, A, A_scale_transposed, B_transposed, B_scale_transposed, C, None, M, N, K, workspace, tile, split_k, stream,
-              b_preshuffled)
+              b_preshuffled, a_swiglu)
 
 
 def fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(A, A_scale_transposed, B_transposed, B_scale_transposed, C,
                                                                      C_scale_transposed, M, N, K, stream=None, workspace=None,
-                                                                     tile=_lib.TILE_AUTO, split_k=0, b_preshuffled=False):
+                                                                     tile=_lib.TILE_AUTO, split_k=0, b_preshuffled=False, a_swiglu=False):
     """examples/005.fp8.mm.cu:2467-2500 / examples/005.fp8.mm.opt.cu:468-508.  C e4m3 codes [M,N],
     C_scale_transposed float32 [N/128, M]."""
     _fp8_gemm(_lib.OUT_FP8Q, A, A_scale_transposed, B_transposed, B_scale_transposed, C, C_scale_transposed, M, N, K, workspace, tile,
-              split_k, stream, b_preshuffled)
+              split_k, stream, b_preshuffled, a_swiglu)
 
 
 def fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(A, A_scale_transposed, B_transposed, B_scale_transposed, C,
@@ -190,13 +198,14 @@ def fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(A, 
     """The gate_up projection of a gated MLP with the activation fused in front of the C quantisation (the fusion
     the reference plans, README.md:16; no reference kernel).  B_transposed [N,K] holds the gate rows in [0, N/2) and
     the up rows in [N/2, N); C = e4m3 codes of silu(gate) * up [M, N/2], C_scale_transposed float32 [N/256, M].
-    M <= 128 needs a workspace (``make_workspace(OUT_FP8Q_SWIGLU, ...)``)."""
+    M <= 128 needs a workspace (``make_workspace(OUT_FP8Q_SWIGLU, ...)``).  (The other way to fuse the activation is on the
+    consumer's side: run gate_up with fp32 output and pass it to the down projection with ``a_swiglu=True``.)"""
     _fp8_gemm(_lib.OUT_FP8Q_SWIGLU, A, A_scale_transposed, B_transposed, B_scale_transposed, C, C_scale_transposed, M, N, K, workspace,
               tile, split_k, stream, b_preshuffled)
 
 
 def fp8_gemm_add_rmsnorm_quant(A, A_scale_transposed, B_transposed, B_scale_transposed, residual, hidden_out, norm_weight, eps, M, N, K,
-                               stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0, b_preshuffled=False):
+                               stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0, b_preshuffled=False, a_swiglu=False):
     """A projection back to the hidden size (O, down) with the decoder block's epilogue behind it (the fusion the reference
     plans, README.md:16): ``hidden_out = residual + A @ B`` (stored in the residual's dtype; may be the same tensor), then
     RMSNorm(hidden_out) * norm_weight quantised 1x128 with transposed scales.  Returns (codes uint8 [M,N], scales float32
@@ -206,13 +215,14 @@ def fp8_gemm_add_rmsnorm_quant(A, A_scale_transposed, B_transposed, B_scale_tran
         raise RuntimeError("T is not supported.")
     kb = K // 128 if K % 128 == 0 else 0
     if workspace is None:
-        n = int(lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K))
+        n = int(lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K)) + (int(lib.llmmm_fp8_swiglu_a_workspace(M, N, K)) if a_swiglu else 0)
         workspace = torch.empty(max(n, 16), dtype=torch.uint8, device=residual.device)
     q = torch.empty((M, N), dtype=torch.uint8, device=residual.device)
     s = torch.empty(((N + 127) // 128, M), dtype=torch.float32, device=residual.device)
-    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS)
+    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS, _lib.FP8_A_SWIGLU_F32 if a_swiglu else _lib.FP8_A_QUANTISED)
+    a_p, as_p = _a_operand(A, A_scale_transposed, M, K, a_swiglu)
     check(lib.llmmm_fp8_gemm_add_rmsnorm_quant(
-        _ptr(A, "A", _FP8_DTYPES, M * K), _ptr(A_scale_transposed, "A_scale_transposed", (torch.float32,), kb * M),
+        a_p, as_p,
         _ptr(B_transposed, "B_transposed", _FP8_DTYPES, N * K), _ptr(B_scale_transposed, "B_scale_transposed", (torch.float32,), ((N + 127) // 128) * kb),
         code, _ptr(residual, "residual", numel=M * N), _ptr(hidden_out, "hidden_out", numel=M * N), _ptr(norm_weight, "norm_weight", (torch.float32,), N),
         ctypes.c_float(eps), _ptr(q, "q"), _ptr(s, "q_scale"), M, N, K, ctypes.c_void_p(workspace.data_ptr()),
