@@ -75,6 +75,9 @@ extern "C" {
                                   * ignored: the GEMM runs on quantise_1x128(silu(G[:, :K]) * G[:, K:]), which the kernel makes itself --
                                   * see llmmm_fp8_swiglu_a_workspace */
 
+#define LLMMM_FP8_A_PLANES_RMSNORM 2 /* A points at a llmmm_a_planes_rmsnorm (host memory): the operand is the RMSNorm of a hidden
+                                      * state that is still in pieces, see llmmm_fp8_gemm_planes */
+
 typedef struct llmmm_gemm_cfg {
   int tile;
   int split_k;
@@ -196,6 +199,33 @@ LLMMM_API size_t llmmm_fp8_gemm_qkv_rope_workspace(int M, int N, int K);
  * first, which then must hold llmmm_fp8_swiglu_a_workspace(M, N, K) bytes (0 when the kernel does it itself) on top of what
  * the GEMM wants. */
 LLMMM_API size_t llmmm_fp8_swiglu_a_workspace(int M, int N, int K);
+
+/* The block epilogue fused into the *consumer* (single-stream decode).  llmmm_fp8_gemm_planes runs a projection back to the
+ * hidden size (O, down) and stops at its fp32 partial sums: `planes` [*splits][M][N] (llmmm_fp8_gemm_planes_bytes bytes hold
+ * the library's choice of split; with less room the split shrinks; cfg as for llmmm_fp8_gemm_ex, `workspace` only serves an
+ * a_layout that has to be quantised first).  The next projection (QKV, gate_up; any FP8 entry point) then takes
+ * cfg.a_layout = LLMMM_FP8_A_PLANES_RMSNORM and a llmmm_a_planes_rmsnorm in place of A (As ignored; K of that call = N of
+ * the planes), and runs on
+ *   h = sum of the planes in split order + residual;  hidden_out = hidden_dtype(h);  A = quantise_1x128(rmsnorm(hidden_out) * w)
+ * -- exactly the hidden state, codes and scales llmmm_fp8_gemm_add_rmsnorm_quant delivers, bit for bit.  For M <= 4 and
+ * K <= 3072 every workgroup of the weight-streaming kernel makes the operand itself while its first weights are in flight
+ * (no reduce kernel, no norm kernel: one launch per projection); hidden_out must then be a buffer of its own, not the
+ * residual.  Otherwise the library runs the fused reduce + norm + quantise kernel into the front of the workspace first
+ * (llmmm_fp8_planes_rmsnorm_a_workspace extra bytes).  Planned by the reference (README.md:16), no reference kernel. */
+typedef struct llmmm_a_planes_rmsnorm {
+  const float* planes;      /* [splits][M][K] fp32, from llmmm_fp8_gemm_planes */
+  int          splits;
+  int          hidden_dtype; /* LLMMM_DTYPE_F32 / _BF16 / _F16 */
+  const void*  residual;    /* [M, K] */
+  void*        hidden_out;  /* [M, K] */
+  const float* norm_weight; /* [K] */
+  float        eps;
+} llmmm_a_planes_rmsnorm;
+LLMMM_API int    llmmm_fp8_gemm_planes(const void* A, const float* As, const void* Bt, const float* Bs, int M, int N, int K, float* planes,
+                                       size_t planes_bytes, int* splits, void* workspace, size_t workspace_bytes, const llmmm_gemm_cfg* cfg,
+                                       void* stream);
+LLMMM_API size_t llmmm_fp8_gemm_planes_bytes(int M, int N, int K);
+LLMMM_API size_t llmmm_fp8_planes_rmsnorm_a_workspace(int M, int N, int K);
 
 /* ---- offline layout helpers --------------------------------------------------------------
  * llmmm_fp8_preshuffle_b takes the role of  construct_m16n8k32_B_layout(dst, src_transposed, N, K,

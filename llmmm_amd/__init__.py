@@ -9,7 +9,9 @@ from .mm import (  # noqa: F401
     fp16_gemm,
     fp16_mm,
     fp8_blockwise_symmetric_quantization,
+    PlanesRmsnorm,
     fp8_gemm_add_rmsnorm_quant,
+    fp8_gemm_planes,
     fp8_gemm_qkv_rope,
     fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8,
     fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16,

@@ -20,7 +20,13 @@ B_ROW_MAJOR, B_TRANSPOSED = 0, 1
 OUT_F32, OUT_BF16, OUT_FP8Q, OUT_FP8Q_SWIGLU = 0, 1, 2, 3
 QUANT_1x128_T, QUANT_128x128, QUANT_1x128, QUANT_128x128_T = 0, 1, 2, 3
 FP8_B_ROWS, FP8_B_PRESHUFFLED = 0, 1
-FP8_A_QUANTISED, FP8_A_SWIGLU_F32 = 0, 1
+FP8_A_QUANTISED, FP8_A_SWIGLU_F32, FP8_A_PLANES_RMSNORM = 0, 1, 2
+
+
+class APlanesRmsnorm(ctypes.Structure):
+    """llmmm_a_planes_rmsnorm: the A operand of cfg.a_layout = FP8_A_PLANES_RMSNORM."""
+    _fields_ = [("planes", ctypes.c_void_p), ("splits", ctypes.c_int), ("hidden_dtype", ctypes.c_int), ("residual", ctypes.c_void_p),
+                ("hidden_out", ctypes.c_void_p), ("norm_weight", ctypes.c_void_p), ("eps", ctypes.c_float)]
 PROBE_FP8 = 2
 TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_64x128, TILE_SKINNY = -1, 0, 1, 2, 3, 4, 8
 
@@ -48,6 +54,9 @@ SIGNATURES = {
                                      _c.POINTER(GemmCfg), _vp]),
     "llmmm_fp8_gemm_qkv_rope_workspace": (_sz, [_i, _i, _i]),
     "llmmm_fp8_swiglu_a_workspace": (_sz, [_i, _i, _i]),
+    "llmmm_fp8_gemm_planes": (_i, [_vp, _fp, _vp, _fp, _i, _i, _i, _vp, _sz, _c.POINTER(_c.c_int), _vp, _sz, _c.POINTER(GemmCfg), _vp]),
+    "llmmm_fp8_gemm_planes_bytes": (_sz, [_i, _i, _i]),
+    "llmmm_fp8_planes_rmsnorm_a_workspace": (_sz, [_i, _i, _i]),
     "llmmm_fp8_preshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
     "llmmm_fp8_unshuffle_b": (_i, [_vp, _vp, _i, _i, _vp]),
     "llmmm_transpose": (_i, [_i, _vp, _vp, _i, _i, _vp]),

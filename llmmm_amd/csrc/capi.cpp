@@ -267,27 +267,72 @@ size_t llmmm_fp8_swiglu_a_workspace(int M, int N, int K)
   return swiglu_a_bytes(M, K);
 }
 
-// Resolves a_layout for a call whose kernel choice is `tile`: either the kernel generates A (*agen = true, A stays the
-// fp32 pointer), or h is quantised into the workspace now and A / As / workspace are redirected to it.
-static int prepare_a(const llmmm_gemm_cfg* user, int tile, const void*& A, const float*& As, int M, int K, void*& workspace, size_t& workspace_bytes,
-                     void* stream, bool* agen)
+// How a call gets its A operand: given quantised (agen 0), generated by the weight-streaming kernel from the fp32 gate_up
+// result (1) or from a hidden state still in pieces (2, with what the kernel needs in `ag`).
+struct APrep {
+  int               agen         = 0;
+  int               hidden_dtype = 0;
+  llmmm::SkinnyGenA ag;
+};
+constexpr int AGEN2_MAX_M = 2, AGEN2_MAX_K = 3072;
+
+size_t llmmm_fp8_planes_rmsnorm_a_workspace(int M, int N, int K)
 {
-  *agen = false;
+  llmmm_gemm_cfg cfg;
+  if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
+  if (cfg.tile == LLMMM_TILE_SKINNY && M <= AGEN2_MAX_M && K <= AGEN2_MAX_K) return 0;
+  return swiglu_a_bytes(M, K);  // the same codes + scales block
+}
+
+// Resolves a_layout for a call whose kernel choice is `tile`: either the kernel generates A (prep->agen != 0; A is not
+// used as an operand pointer any more), or the operand is quantised into the front of the workspace now and A / As /
+// workspace are redirected to it.
+static int prepare_a(const llmmm_gemm_cfg* user, int tile, const void*& A, const float*& As, int M, int K, void*& workspace, size_t& workspace_bytes,
+                     void* stream, APrep* prep)
+{
+  *prep = APrep();
   if (!user || user->a_layout == LLMMM_FP8_A_QUANTISED) return LLMMM_OK;
-  if (user->a_layout != LLMMM_FP8_A_SWIGLU_F32) return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown A layout %d", user->a_layout);
+  if (user->a_layout != LLMMM_FP8_A_SWIGLU_F32 && user->a_layout != LLMMM_FP8_A_PLANES_RMSNORM)
+    return fail(LLMMM_ERR_INVALID_ARGUMENT, "unknown A layout %d", user->a_layout);
   if ((long)M * 2 * K >= (1L << 31)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
-  if (tile == LLMMM_TILE_SKINNY && M <= AGEN_MAX_M) {
-    *agen = true;
+  const llmmm_a_planes_rmsnorm* d = nullptr;
+  if (user->a_layout == LLMMM_FP8_A_PLANES_RMSNORM) {
+    d = (const llmmm_a_planes_rmsnorm*)A;  // a host structure
+    if (!d->planes || !d->residual || !d->hidden_out || !d->norm_weight) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+    if (d->hidden_dtype != LLMMM_DTYPE_F16 && d->hidden_dtype != LLMMM_DTYPE_BF16 && d->hidden_dtype != LLMMM_DTYPE_F32)
+      return fail(LLMMM_ERR_UNSUPPORTED_TYPE, "T is not supported.");
+    if (d->splits < 1 || d->splits > MAX_SPLIT_K) return fail(LLMMM_ERR_INVALID_ARGUMENT, "splits must be 1..%d (got %d)", MAX_SPLIT_K, d->splits);
+    if (!(d->eps >= 0.f)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "eps must be non-negative");
+    if (K > 10240) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the fused norm handles rows of at most 10240 columns (got %d)", K);
+    if (!aligned16(d->planes) || !aligned16(d->residual) || !aligned16(d->hidden_out) || !aligned16(d->norm_weight))
+      return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+    if (tile == LLMMM_TILE_SKINNY && M <= AGEN2_MAX_M && K <= AGEN2_MAX_K) {
+      // every workgroup reads the residual while one writes the hidden state: they must be different buffers
+      if (d->hidden_out == d->residual) return fail(LLMMM_ERR_INVALID_ARGUMENT, "hidden_out must not be the residual buffer when the kernel generates its activations (M <= %d)", AGEN2_MAX_M);
+      prep->agen         = 2;
+      prep->hidden_dtype = d->hidden_dtype;
+      prep->ag.planes = d->planes, prep->ag.residual = d->residual, prep->ag.hidden = d->hidden_out, prep->ag.w = d->norm_weight;
+      prep->ag.eps = d->eps, prep->ag.splits = d->splits;
+      return LLMMM_OK;
+    }
+  }
+  else if (tile == LLMMM_TILE_SKINNY && M <= AGEN_MAX_M) {
+    prep->agen = 1;
     return LLMMM_OK;
   }
   const size_t need = swiglu_a_bytes(M, K);
   if (!workspace || workspace_bytes < need)
-    return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, quantising the SwiGLU activations first needs %zu", workspace ? workspace_bytes : (size_t)0, need);
+    return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, quantising the activations first needs %zu", workspace ? workspace_bytes : (size_t)0, need);
   if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
-  uint8_t* hq = (uint8_t*)workspace;
-  float*   hs = (float*)(hq + align256((size_t)M * K));
-  const hipError_t e = llmmm::fp8_splitk_reduce_launch(LLMMM_OUT_FP8Q_SWIGLU, (const float*)A, 1, hq, hs, M, 2 * K, (hipStream_t)stream);
-  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "SwiGLU quantiser launch: %s", hipGetErrorString(e));
+  uint8_t*   hq = (uint8_t*)workspace;
+  float*     hs = (float*)(hq + align256((size_t)M * K));
+  hipError_t e;
+  if (d)
+    e = llmmm::planes_add_rmsnorm_quant_launch(d->hidden_dtype, d->planes, d->splits, d->residual, d->hidden_out, d->norm_weight, d->eps, hq, hs, M, K,
+                                               (hipStream_t)stream);
+  else
+    e = llmmm::fp8_splitk_reduce_launch(LLMMM_OUT_FP8Q_SWIGLU, (const float*)A, 1, hq, hs, M, 2 * K, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "activation quantiser launch: %s", hipGetErrorString(e));
   A               = hq;
   As              = hs;
   workspace       = hq + need;
@@ -305,7 +350,8 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
   const int      rc = choose_fp8_out(out_kind, M, N, K, &cfg);
   if (rc) return rc;
   const bool a_swiglu = user && user->a_layout == LLMMM_FP8_A_SWIGLU_F32;
-  if (!A || (!As && !a_swiglu) || !Bt || !Bs || !C) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  const bool a_made   = user && user->a_layout != LLMMM_FP8_A_QUANTISED;  // A is not the quantised operand: As is not used
+  if (!A || (!As && !a_made) || !Bt || !Bs || !C) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
   if (a_swiglu && swiglu) return fail(LLMMM_ERR_INVALID_ARGUMENT, "SwiGLU on both the A operand and the output");
   if ((out_kind == LLMMM_OUT_FP8Q || swiglu) && !Cs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "C_scale_transposed is required for fp8 output");
   if (!aligned16(A) || !aligned16(Bt) || !aligned16(C)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
@@ -319,10 +365,11 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
     cfg.b_layout = user->b_layout;
   }
   hipError_t e;
-  bool       agen = false;
+  APrep      prep;
   if (cfg.tile == LLMMM_TILE_SKINNY && M > SKINNY_MAX_M) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the weight-streaming kernel handles M <= %d", SKINNY_MAX_M);
-  const int rca = prepare_a(user, cfg.tile, A, As, M, K, workspace, workspace_bytes, stream, &agen);
+  const int rca = prepare_a(user, cfg.tile, A, As, M, K, workspace, workspace_bytes, stream, &prep);
   if (rca) return rca;
+  const int agen = prep.agen;
   if (cfg.tile == LLMMM_TILE_SKINNY) {
     int split = cfg.split_k;
     if (split > max_split_for(K)) split = max_split_for(K);
@@ -343,13 +390,16 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
       if ((size_t)split > room) split = room < 2 ? 1 : (int)room;
       if (split < min_split) split = min_split;  // (fails the size check below)
     }
-    if (split > 1 || swiglu) {
+    // (the norm-generating kernel only writes fp32: any other output goes through one plane and the reduce kernel)
+    if (split > 1 || swiglu || (agen == 2 && out_kind != LLMMM_OUT_F32)) {
       const size_t need = (size_t)split * M * N * sizeof(float);
-      if (workspace_bytes < need) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace_bytes, split, need);
+      if (!workspace || workspace_bytes < need) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, split-K %d needs %zu", workspace ? workspace_bytes : (size_t)0, split, need);
       if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
       partial = (float*)workspace;
     }
-    if (agen)
+    if (agen == 2)
+      e = llmmm::fp8_skinny_rmsnorm_a_launch(prep.hidden_dtype, cfg.b_layout, prep.ag, Bt, Bs, (float*)C, M, N, K, split, partial, (hipStream_t)stream);
+    else if (agen)
       e = llmmm::fp8_skinny_swiglu_a_launch(partial ? LLMMM_OUT_F32 : out_kind, cfg.b_layout, (const float*)A, Bt, Bs, C, Cs, M, N, K, split, partial,
                                             (hipStream_t)stream);
     else
@@ -468,7 +518,8 @@ size_t llmmm_fp8_gemm_add_rmsnorm_quant_workspace(int M, int N, int K)
 // and the workspace has been checked to hold them.
 struct PlaneCfg {
   int  tile = 0, split = 0, b_layout = 0;
-  bool skinny = false, agen = false;
+  bool  skinny = false;
+  APrep prep;
 };
 static int resolve_plane_cfg(const void*& A, const float*& As, const void* Bt, const float* Bs, int M, int N, int K, void*& workspace,
                              size_t& workspace_bytes, const llmmm_gemm_cfg* user, bool allow_direct, PlaneCfg* out, void* stream)
@@ -476,8 +527,8 @@ static int resolve_plane_cfg(const void*& A, const float*& As, const void* Bt, c
   llmmm_gemm_cfg cfg;
   const int      rc = choose_fp8(M, N, K, &cfg);
   if (rc) return rc;
-  const bool a_swiglu = user && user->a_layout == LLMMM_FP8_A_SWIGLU_F32;
-  if (!A || (!As && !a_swiglu) || !Bt || !Bs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  const bool a_made = user && user->a_layout != LLMMM_FP8_A_QUANTISED;
+  if (!A || (!As && !a_made) || !Bt || !Bs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
   if (!aligned16(A) || !aligned16(Bt)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
   if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
@@ -499,13 +550,13 @@ static int resolve_plane_cfg(const void*& A, const float*& As, const void* Bt, c
     if (user && user->tile != LLMMM_TILE_AUTO && user->split_k <= 0) cfg.split_k = heuristic_tile_split(cfg.tile, M, N, K);
   }
   // the A operand given as the fp32 gate_up result: generated by the kernel, or quantised into the front of the workspace now
-  const int rca = prepare_a(user, cfg.tile, A, As, M, K, workspace, workspace_bytes, stream, &out->agen);
+  const int rca = prepare_a(user, cfg.tile, A, As, M, K, workspace, workspace_bytes, stream, &out->prep);
   if (rca) return rca;
   int split = cfg.split_k < 1 ? 1 : cfg.split_k;
   if (split > max_split_for(K)) split = max_split_for(K);
   const size_t plane    = (size_t)M * N * sizeof(float);
   const bool   explicit_split = user && user->split_k > 0;
-  const int    min_split = out->agen ? agen_min_split(K) : 1;
+  const int    min_split = out->prep.agen ? agen_min_split(K) : 1;
   if (split < min_split) {
     if (explicit_split) return fail(LLMMM_ERR_INVALID_ARGUMENT, "generated activations need split-K >= %d for K = %d", min_split, K);
     split = min_split;
@@ -531,13 +582,54 @@ static int launch_into_planes(const PlaneCfg& pc, const void* A, const float* As
 {
   float*     planes = (float*)workspace;
   hipError_t e;
-  if (pc.skinny && pc.agen)
+  if (pc.skinny && pc.prep.agen == 2)
+    e = llmmm::fp8_skinny_rmsnorm_a_launch(pc.prep.hidden_dtype, pc.b_layout, pc.prep.ag, Bt, Bs, nullptr, M, N, K, pc.split, planes, (hipStream_t)stream);
+  else if (pc.skinny && pc.prep.agen == 1)
     e = llmmm::fp8_skinny_swiglu_a_launch(LLMMM_OUT_F32, pc.b_layout, (const float*)A, Bt, Bs, nullptr, nullptr, M, N, K, pc.split, planes, (hipStream_t)stream);
   else if (pc.skinny)
     e = llmmm::fp8_skinny_launch(LLMMM_OUT_F32, pc.b_layout, A, As, Bt, Bs, nullptr, nullptr, M, N, K, pc.split, planes, (hipStream_t)stream);
   else
     e = llmmm::fp8_gemm_launch(LLMMM_OUT_F32, pc.tile, pc.b_layout, A, As, Bt, Bs, nullptr, nullptr, M, N, K, pc.split, planes, (hipStream_t)stream);
   if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "fp8 gemm launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
+size_t llmmm_fp8_gemm_planes_bytes(int M, int N, int K)
+{
+  if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
+  llmmm_gemm_cfg cfg;
+  if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
+  return (size_t)(cfg.split_k < 1 ? 1 : cfg.split_k) * M * N * sizeof(float);
+}
+
+int llmmm_fp8_gemm_planes(const void* A, const float* As, const void* Bt, const float* Bs, int M, int N, int K, float* planes, size_t planes_bytes,
+                          int* splits, void* workspace, size_t workspace_bytes, const llmmm_gemm_cfg* user, void* stream)
+{
+  if (!splits || !planes) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  llmmm_gemm_cfg probe;
+  int            rc = choose_fp8(M, N, K, &probe);
+  if (rc) return rc;
+  llmmm_gemm_cfg inner;
+  inner.tile = LLMMM_TILE_AUTO, inner.split_k = 0, inner.b_layout = LLMMM_FP8_B_ROWS, inner.a_layout = LLMMM_FP8_A_QUANTISED;
+  if (user) inner = *user;
+  if (inner.a_layout != LLMMM_FP8_A_QUANTISED) {
+    // an operand the library has to quantise first goes to `workspace` (the planes have a buffer of their own); one the
+    // kernel generates is resolved a second time inside resolve_plane_cfg, which launches nothing for it
+    if (!A) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+    const int tile = inner.tile != LLMMM_TILE_AUTO ? inner.tile : probe.tile;
+    APrep     prep;
+    rc = prepare_a(&inner, tile, A, As, M, K, workspace, workspace_bytes, stream, &prep);
+    if (rc) return rc;
+    if (prep.agen == 0) inner.a_layout = LLMMM_FP8_A_QUANTISED;
+  }
+  PlaneCfg pc;
+  void*    pw = planes;
+  size_t   pb = planes_bytes;
+  rc = resolve_plane_cfg(A, As, Bt, Bs, M, N, K, pw, pb, &inner, false, &pc, stream);
+  if (rc) return rc;
+  rc = launch_into_planes(pc, A, As, Bt, Bs, M, N, K, pw, stream);
+  if (rc) return rc;
+  *splits = pc.split;
   return LLMMM_OK;
 }
 

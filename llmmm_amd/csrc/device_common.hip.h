@@ -91,6 +91,10 @@ __device__ __forceinline__ void asm_load_16B(i32x4& dst, const void* gptr)
 {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(gptr) : "memory");
 }
+__device__ __forceinline__ void asm_load_8B(i32x2& dst, const void* gptr)
+{
+  asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(dst) : "v"(gptr) : "memory");
+}
 __device__ __forceinline__ void asm_load_f32(float& dst, const void* gptr)
 {
   asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(gptr) : "memory");

@@ -163,15 +163,19 @@ __device__ __forceinline__ void skinny_consume(const SkinnySlot<MBLK, APRE>& t, 
 // the gate_up projection: h = silu(G[:, :K]) * G[:, K:], quantised 1x128, for the 16 rows and the K range it works on
 // (the arithmetic of the reduce kernel's SwiGLU output, so the codes and scales are the ones that kernel would have
 // written).  M <= 16.  A (then: G) and As (unused) keep their places in the argument list.
-template <int MBLK, int OUT, int D, int ASTG, bool AGEN = false>
+// AGEN == 2: the activations are the RMSNorm of a hidden state that is itself still in pieces -- the fp32 planes of the
+// projection before (summed in split order), plus the residual: h = sum + residual, hidden = HT(h) (stored by workgroup
+// (0, 0, 0); it must not alias the residual, which every workgroup reads), A = quantise_1x128(rmsnorm(hidden) * w), in the
+// arithmetic and order of planes_add_rmsnorm_quant_kernel, bit for bit.  M <= 2, K <= 3072 (the row lives in registers).
+template <int MBLK, int OUT, int D, int ASTG, int AGEN = 0, typename HT = float>
 __global__ void __launch_bounds__(512)
 fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
                   const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int S,
-                  float* __restrict__ partial, int bpre)
+                  float* __restrict__ partial, int bpre, SkinnyGenA ag)
 {
   constexpr bool APRE  = ASTG > 0;
-  static_assert(!AGEN || (MBLK == 1 && APRE), "generated activations: 16 rows, staged in LDS");
-  constexpr int  LOADS = SKINNY_LOADS_PER_SLOT_BASE + (AGEN ? 0 : (APRE ? 1 : 3) * MBLK);  // vector-memory loads per slot, issued in slot order
+  static_assert(AGEN == 0 || (MBLK == 1 && APRE), "generated activations: 16 rows, staged in LDS");
+  constexpr int  LOADS = SKINNY_LOADS_PER_SLOT_BASE + (AGEN != 0 ? 0 : (APRE ? 1 : 3) * MBLK);  // vector-memory loads per slot, issued in slot order
   static_assert(D * LOADS < 64, "vmcnt is a 6-bit counter");
   static_assert(MBLK <= 4 || APRE, "128-row groups only with staged activations");
   __shared__ __attribute__((aligned(1024))) char a_stage[APRE ? ASTG : 16];
@@ -185,7 +189,8 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   __shared__ __attribute__((aligned(1024))) char ring6[D > 4 ? 8 * 2048 : 16];
   __shared__ __attribute__((aligned(1024))) char ring7[D > 4 ? 8 * 2048 : 16];
   __shared__ float    wave_amax[8][MBLK][16];
-  __shared__ float    a_scale[AGEN ? (ASTG / 2048) * 16 : 1];  // AGEN: the generated row scales, [slice][row]
+  __shared__ float    a_scale[AGEN != 0 ? (ASTG / 2048) * 16 : 1];  // AGEN: the generated row scales, [slice][row]
+  __shared__ float    gen_sum[AGEN == 2 ? 8 : 1];                        // AGEN == 2: sums of squares of the 64-lane groups, two rows
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -238,7 +243,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   // they have landed.
   const char LLMMM_LDS* const a_tile = (const char LLMMM_LDS*)a_stage;
   const int                   a_rd   = kmajor_offset<SWZ_ROWS16>(i, 2 * g);
-  if constexpr (APRE && !AGEN) {
+  if constexpr (APRE && AGEN == 0) {
     const unsigned a_addr = (unsigned)(size_t)(char LLMMM_LDS*)a_stage;
     const int      units  = (kb1 - kb0) * 2 * MBLK;
     for (int u = wave; u < units; u += 8) {
@@ -254,13 +259,146 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   // slot order so that "at most n loads outstanding" pins down which slots have landed.
   // Slice indices beyond the split are clamped to its last slice (a repeated, cached load) and
   // consumed with a zero scale; the last pass issues nothing and counts its waits down.
+  // AGEN == 2: everything the generated operand needs is requested first, as hand-counted loads like the ring's, so that
+  // it is the oldest traffic in flight: "at most D * LOADS outstanding" behind the ring prologue then means it has landed,
+  // and the norm runs while the first weights are still on their way.
+  constexpr int GP = 10;  // planes requested up front (the split counts in use are 1 .. 10); more follow in a second batch
+  i32x4         g_res[AGEN == 2 ? 3 : 1], g_w[AGEN == 2 ? 3 : 1], g_p[AGEN == 2 ? GP : 1][AGEN == 2 ? 3 : 1];
+  i32x2         g_res2[AGEN == 2 ? 3 : 1];  // the residual chunk of a 2-byte hidden type (nothing may read these before the wait)
+  if constexpr (AGEN == 2) {
+    const int    vl = tid & 255, r = min(tid >> 8, M - 1), chunks = K >> 2;
+    const size_t pplane = (size_t)M * K;
+    // (waves without a row of their own and planes beyond the split count request nothing: both conditions are uniform
+    // over a wave, and fewer old loads in flight only make the counted wait below easier to meet)
+    if ((tid >> 8) < M) {
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      const int c = min(vl + 256 * u, chunks - 1);
+      if constexpr (sizeof(HT) == 4)
+        asm_load_16B(g_res[u], (const HT*)ag.residual + (size_t)r * K + 4 * c);
+      else
+        asm_load_8B(g_res2[u], (const HT*)ag.residual + (size_t)r * K + 4 * c);
+      asm_load_16B(g_w[u], ag.w + 4 * c);
+    }
+#pragma unroll
+    for (int v = 0; v < GP; ++v)
+      if (v < ag.splits) {
+#pragma unroll
+        for (int u = 0; u < 3; ++u) {
+          const int c = min(vl + 256 * u, chunks - 1);
+          asm_load_16B(g_p[v][u], ag.planes + (size_t)v * pplane + (size_t)r * K + 4 * c);
+        }
+      }
+    }
+  }
   SkinnySlot<MBLK, APRE> slot[D];
 #pragma unroll
   for (int u = 0; u < D; ++u) {
-    skinny_fetch<MBLK, APRE, AGEN>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb0 + u, kb1 - 1), M);
+    skinny_fetch<MBLK, APRE, AGEN != 0>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb0 + u, kb1 - 1), M);
     __builtin_amdgcn_sched_barrier(0);
   }
-  if constexpr (AGEN) {
+  if constexpr (AGEN == 2) {
+    HT*          hid    = (HT*)ag.hidden;
+    const int    vl     = tid & 255, rsel = tid >> 8;  // 256 virtual lanes per row; rows 0 and 1 side by side (M <= 2)
+    const int    chunks = K >> 2, nsl = kb1 - kb0;
+    const size_t pplane = (size_t)M * K;
+    const bool   writer = blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0;
+    const int    r      = min(rsel, M - 1);
+    const bool   live   = rsel < M;
+    for (int x = tid; x < nsl * 128; x += 512) *(i32x4 LLMMM_LDS*)((char LLMMM_LDS*)a_stage + x * 16) = i32x4{0, 0, 0, 0};
+    for (int x = tid; x < nsl * 16; x += 512) a_scale[x] = 0.f;
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * LOADS) : "memory");  // the operand's loads are in; the ring's stay in flight
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      if constexpr (sizeof(HT) == 4)
+        asm volatile("" : "+v"(g_res[u]), "+v"(g_w[u]));
+      else
+        asm volatile("" : "+v"(g_res2[u]), "+v"(g_w[u]));
+#pragma unroll
+      for (int v = 0; v < GP; ++v) asm volatile("" : "+v"(g_p[v][u]));
+    }
+    f32x4 held[3], rv[3], wv[3];
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      wv[u] = __builtin_bit_cast(f32x4, g_w[u]);
+      if constexpr (sizeof(HT) == 4)
+        rv[u] = __builtin_bit_cast(f32x4, g_res[u]);
+      else {
+        typedef HT     ht4 __attribute__((ext_vector_type(4)));
+        const ht4      t  = __builtin_bit_cast(ht4, g_res2[u]);
+        rv[u]             = f32x4{(float)t[0], (float)t[1], (float)t[2], (float)t[3]};
+      }
+      held[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int v = 0; v < GP; ++v)
+      if (v < ag.splits) {
+#pragma unroll
+        for (int u = 0; u < 3; ++u) held[u] += __builtin_bit_cast(f32x4, g_p[v][u]);
+      }
+    for (int s0 = GP; s0 < ag.splits; s0 += 8) {  // (more than GP planes: ordinary loads, eight in flight)
+      f32x4 p[8][3];
+#pragma unroll
+      for (int v = 0; v < 8; ++v)
+#pragma unroll
+        for (int u = 0; u < 3; ++u) {
+          const int c = min(vl + 256 * u, chunks - 1);
+          p[v][u]     = *(const f32x4*)(ag.planes + (size_t)min(s0 + v, ag.splits - 1) * pplane + (size_t)r * K + 4 * c);
+        }
+#pragma unroll
+      for (int v = 0; v < 8; ++v)
+        if (s0 + v < ag.splits) {
+#pragma unroll
+          for (int u = 0; u < 3; ++u) held[u] += p[v][u];
+        }
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      const int c = vl + 256 * u;
+      if (c < chunks) {
+        const f32x4 h = held[u] + rv[u];
+        if (writer && live) store_row4<HT>(hid + (size_t)r * K + 4 * c, h);
+        if constexpr (sizeof(HT) == 4)
+          held[u] = h;
+        else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) held[u][e] = (float)(HT)h[e];  // the norm reads the hidden state as stored
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_fmaf(held[u][e], held[u][e], acc);
+      }
+      else
+        held[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1) acc = acc + wave_xor_get(acc, step);
+    if (lane == 0) gen_sum[wave] = acc;
+    __syncthreads();  // (also: the zero fill is complete)
+    const float total = (gen_sum[4 * rsel] + gen_sum[4 * rsel + 1]) + (gen_sum[4 * rsel + 2] + gen_sum[4 * rsel + 3]);
+    const float ms    = total / (float)K;
+    const float rn    = 1.0f / __builtin_sqrtf(ms + ag.eps);
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      const int c = vl + 256 * u;
+      const int j = (c >> 5) - kb0;  // the chunk's 128-column block as a slice of this workgroup
+      // only the blocks of this workgroup's K range are quantised (uniform over the 32 lanes that share a block)
+      if (c < chunks && live && j >= 0 && j < nsl) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) held[u][e] = (held[u][e] * rn) * wv[u][e];
+        float a = fmaxf(fmaxf(__builtin_fabsf(held[u][0]), __builtin_fabsf(held[u][1])), fmaxf(__builtin_fabsf(held[u][2]), __builtin_fabsf(held[u][3])));
+#pragma unroll
+        for (int step = 1; step <= 16; step <<= 1) a = wave_xor_max(a, step);
+        const float sc = a / 448.f;
+        uint32_t    cd = 0;
+        if (sc != 0.f) cd = sk_pack_e4m3x4(held[u][0] / sc, held[u][1] / sc, held[u][2] / sc, held[u][3] / sc);
+        *(uint32_t LLMMM_LDS*)((char LLMMM_LDS*)a_stage + j * 2048 + kmajor_offset<SWZ_ROWS16>(r, (c & 31) >> 2) + (c & 3) * 4) = cd;
+        if ((c & 31) == 0) a_scale[j * 16 + r] = sc;
+      }
+    }
+    __syncthreads();  // the staged tile is complete
+  }
+  else if constexpr (AGEN == 1) {
     // Behind the ring prologue (the weights are on their way): half a wavefront per row, a lane per four columns of a
     // slice.  The loads below are ordinary ones; the waits the compiler puts behind them also cover the ring loads
     // issued above, which only makes the hand-counted waits of the loop trivially true for the first pass.
@@ -311,20 +449,20 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   for (; kb + D < kb1; kb += D) {  // passes followed by another pass: consume a slot, refill it
 #pragma unroll
     for (int u = 0; u < D; ++u) {
-      skinny_wait<(D - 1) * LOADS, MBLK, APRE, AGEN>(slot[u]);
-      skinny_consume<MBLK, APRE, AGEN>(slot[u], ring[u], w_rd, true, acc, a_tile + (kb + u - kb0) * (MBLK * 2048), a_rd,
-                                       (const float LLMMM_LDS*)a_scale + (AGEN ? (kb + u - kb0) * 16 : 0), i);
+      skinny_wait<(D - 1) * LOADS, MBLK, APRE, AGEN != 0>(slot[u]);
+      skinny_consume<MBLK, APRE, AGEN != 0>(slot[u], ring[u], w_rd, true, acc, a_tile + (kb + u - kb0) * (MBLK * 2048), a_rd,
+                                       (const float LLMMM_LDS*)a_scale + (AGEN != 0 ? (kb + u - kb0) * 16 : 0), i);
       __builtin_amdgcn_sched_barrier(0);
-      skinny_fetch<MBLK, APRE, AGEN>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb + u + D, kb1 - 1), M);
+      skinny_fetch<MBLK, APRE, AGEN != 0>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb + u + D, kb1 - 1), M);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
 #define LLMMM_LAST(u)                                                              \
   if constexpr ((u) < D) {                                                         \
-    skinny_wait<(D - 1 - (u)) * LOADS, MBLK, APRE, AGEN>(slot[u]);                 \
-    skinny_consume<MBLK, APRE, AGEN>(slot[u], ring[u], w_rd, kb + (u) < kb1, acc,  \
+    skinny_wait<(D - 1 - (u)) * LOADS, MBLK, APRE, AGEN != 0>(slot[u]);                 \
+    skinny_consume<MBLK, APRE, AGEN != 0>(slot[u], ring[u], w_rd, kb + (u) < kb1, acc,  \
                                a_tile + (min(kb + (u), kb1 - 1) - kb0) * (MBLK * 2048), a_rd, \
-                               (const float LLMMM_LDS*)a_scale + (AGEN ? (min(kb + (u), kb1 - 1) - kb0) * 16 : 0), i); \
+                               (const float LLMMM_LDS*)a_scale + (AGEN != 0 ? (min(kb + (u), kb1 - 1) - kb0) * 16 : 0), i); \
     __builtin_amdgcn_sched_barrier(0);                                             \
   }
   LLMMM_LAST(0) LLMMM_LAST(1) LLMMM_LAST(2) LLMMM_LAST(3) LLMMM_LAST(4) LLMMM_LAST(5) LLMMM_LAST(6) LLMMM_LAST(7)
@@ -398,7 +536,7 @@ static hipError_t launch_skinny(const void* A, const float* As, const void* Bt, 
                                 int N, int K, int S, float* partial, int bpre, hipStream_t stream)
 {
   hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D, ASTG>), dim3(N / 128, S, MBLK == 8 ? (M + 127) / 128 : (M + 63) / 64), dim3(512), 0, stream,
-                     (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial, bpre);
+                     (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial, bpre, SkinnyGenA{});
   return hipGetLastError();
 }
 
@@ -411,8 +549,8 @@ static hipError_t dispatch_skinny_agen(const float* G, const void* Bt, const flo
   if (M > 16 || need > 65536) return hipErrorInvalidValue;
 #define LLMMM_GO(D, ASTG)                                                                                                                   \
   {                                                                                                                                         \
-    hipLaunchKernelGGL((fp8_skinny_kernel<1, OUT, D, ASTG, true>), dim3(N / 128, S, 1), dim3(512), 0, stream, (const uint8_t*)G, (const float*)nullptr, \
-                       (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial, bpre);                                                           \
+    hipLaunchKernelGGL((fp8_skinny_kernel<1, OUT, D, ASTG, 1>), dim3(N / 128, S, 1), dim3(512), 0, stream, (const uint8_t*)G, (const float*)nullptr, \
+                       (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial, bpre, SkinnyGenA{});                                            \
     return hipGetLastError();                                                                                                               \
   }
   if (slices >= 8 && need <= 28672) LLMMM_GO(8, 28672);
@@ -429,6 +567,36 @@ hipError_t fp8_skinny_swiglu_a_launch(int out_kind, int b_layout, const float* G
     case SK_OUT_F32: return dispatch_skinny_agen<SK_OUT_F32>(G, Bt, Bs, C, Cs, M, N, K, S, partial, bpre, stream);
     case SK_OUT_BF16: return dispatch_skinny_agen<SK_OUT_BF16>(G, Bt, Bs, C, Cs, M, N, K, S, partial, bpre, stream);
     case SK_OUT_FP8Q: return dispatch_skinny_agen<SK_OUT_FP8Q>(G, Bt, Bs, C, Cs, M, N, K, S, partial, bpre, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <typename HT>
+static hipError_t dispatch_skinny_gen2(const SkinnyGenA& ag, const void* Bt, const float* Bs, float* C, int M, int N, int K, int S, float* partial, int bpre,
+                                       hipStream_t stream)
+{
+  const int KB = K / 128, slices = KB / S, longest = (KB + S - 1) / S, need = 2048 * longest;
+  if (M > 2 || K > 3072 || need > 65536 || ag.splits < 1 || ag.hidden == ag.residual) return hipErrorInvalidValue;
+#define LLMMM_GO(D, ASTG)                                                                                                                       \
+  {                                                                                                                                             \
+    hipLaunchKernelGGL((fp8_skinny_kernel<1, SK_OUT_F32, D, ASTG, 2, HT>), dim3(N / 128, S, 1), dim3(512), 0, stream, (const uint8_t*)nullptr,  \
+                       (const float*)nullptr, (const uint8_t*)Bt, Bs, (void*)C, (float*)nullptr, M, N, K, S, partial, bpre, ag);                \
+    return hipGetLastError();                                                                                                                   \
+  }
+  if (slices >= 8 && need <= 28672) LLMMM_GO(8, 28672);
+  if (slices >= 4) LLMMM_GO(4, 65536);
+  LLMMM_GO(2, 65536);
+#undef LLMMM_GO
+}
+
+hipError_t fp8_skinny_rmsnorm_a_launch(int hidden_dtype, int b_layout, const SkinnyGenA& ag, const void* Bt, const float* Bs, float* C, int M, int N, int K,
+                                       int S, float* partial, hipStream_t stream)
+{
+  const int bpre = b_layout == LLMMM_FP8_B_PRESHUFFLED;
+  switch (hidden_dtype) {
+    case LLMMM_DTYPE_F32: return dispatch_skinny_gen2<float>(ag, Bt, Bs, C, M, N, K, S, partial, bpre, stream);
+    case LLMMM_DTYPE_BF16: return dispatch_skinny_gen2<__bf16>(ag, Bt, Bs, C, M, N, K, S, partial, bpre, stream);
+    case LLMMM_DTYPE_F16: return dispatch_skinny_gen2<_Float16>(ag, Bt, Bs, C, M, N, K, S, partial, bpre, stream);
     default: return hipErrorInvalidValue;
   }
 }

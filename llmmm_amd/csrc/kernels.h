@@ -56,6 +56,20 @@ hipError_t fp8_splitk_reduce_launch(int out_kind, const float* planes, int S, vo
 hipError_t fp8_skinny_launch(int out_kind, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
                              float* Cs, int M, int N, int K, int S, float* partial, hipStream_t stream);
 
+// What the weight-streaming kernel needs to make its activations from a hidden state that is still in pieces.
+struct SkinnyGenA {
+  const float* planes   = nullptr;  // [splits][M][K] fp32 partial sums of the projection before
+  const void*  residual = nullptr;  // [M, K] of the hidden dtype
+  void*        hidden   = nullptr;  // [M, K] out: hidden dtype(sum + residual); must not alias the residual
+  const float* w        = nullptr;  // [K] RMSNorm weights
+  float        eps      = 0.f;
+  int          splits   = 0;
+};
+// The kernel with A = quantise_1x128(rmsnorm(hidden) * w), hidden = T(sum of planes + residual): M <= 2, K <= 3072, fp32
+// output (C, or planes `partial` as above).  hipErrorInvalidValue outside these limits.
+hipError_t fp8_skinny_rmsnorm_a_launch(int hidden_dtype, int b_layout, const SkinnyGenA& ag, const void* Bt, const float* Bs, float* C, int M, int N, int K,
+                                       int S, float* partial, hipStream_t stream);
+
 // The same kernel making its activations itself from the fp32 gate_up result G [M, 2K]: A = quantise_1x128(silu(G[:, :K]) *
 // G[:, K:]), M <= 16, at most 32 slices of 128 per split (hipErrorInvalidValue otherwise).  partial as above.
 hipError_t fp8_skinny_swiglu_a_launch(int out_kind, int b_layout, const float* G, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N,

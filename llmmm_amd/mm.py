@@ -143,25 +143,46 @@ def query_config(out_kind, M, N, K):
     return cfg.tile, cfg.split_k
 
 
+class PlanesRmsnorm:
+    """The A operand of a projection whose input is the RMSNorm of a hidden state still in pieces (llmmm_a_planes_rmsnorm):
+    ``planes`` [splits, M, K] float32 from :func:`fp8_gemm_planes`, ``residual`` / ``hidden_out`` [M, K] (float32, bfloat16 or
+    float16; different tensors for M <= 4), ``norm_weight`` [K] float32."""
+
+    def __init__(self, planes, splits, residual, hidden_out, norm_weight, eps):
+        self.planes, self.splits, self.residual, self.hidden_out, self.norm_weight, self.eps = planes, splits, residual, hidden_out, norm_weight, eps
+
+    def c_struct(self, M, K):
+        code = {torch.float32: _lib.DTYPE_F32, torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16}.get(self.residual.dtype)
+        if code is None or self.hidden_out.dtype != self.residual.dtype:
+            raise RuntimeError("T is not supported.")
+        return _lib.APlanesRmsnorm(_ptr(self.planes, "planes", (torch.float32,), self.splits * M * K).value, self.splits, code,
+                                   _ptr(self.residual, "residual", numel=M * K).value, _ptr(self.hidden_out, "hidden_out", numel=M * K).value,
+                                   _ptr(self.norm_weight, "norm_weight", (torch.float32,), K).value, self.eps)
+
+
 def _a_operand(A, As, M, K, a_swiglu):
-    """Pointers of the A operand: quantised codes + transposed scales, or (a_swiglu) the fp32 gate_up result [M, 2K]."""
+    """(A pointer, As pointer, a_layout, keep-alive) of the A operand: quantised codes + transposed scales, the fp32 gate_up result
+    [M, 2K] (a_swiglu), or a :class:`PlanesRmsnorm`."""
     kb = K // 128 if K % 128 == 0 else 0
+    if isinstance(A, PlanesRmsnorm):
+        st = A.c_struct(M, K)
+        return ctypes.cast(ctypes.pointer(st), ctypes.c_void_p), None, _lib.FP8_A_PLANES_RMSNORM, st
     if a_swiglu:
-        return _ptr(A, "A (fp32 gate_up result)", (torch.float32,), M * 2 * K), None
-    return _ptr(A, "A", _FP8_DTYPES, M * K), _ptr(As, "A_scale_transposed", (torch.float32,), kb * M)
+        return _ptr(A, "A (fp32 gate_up result)", (torch.float32,), M * 2 * K), None, _lib.FP8_A_SWIGLU_F32, None
+    return _ptr(A, "A", _FP8_DTYPES, M * K), _ptr(As, "A_scale_transposed", (torch.float32,), kb * M), _lib.FP8_A_QUANTISED, None
 
 
 def _fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, workspace, tile, split_k, stream, b_preshuffled=False, a_swiglu=False):
     kb = K // 128 if K % 128 == 0 else 0
     c_dtypes = {_lib.OUT_F32: (torch.float32,), _lib.OUT_BF16: (torch.bfloat16,), _lib.OUT_FP8Q: _FP8_DTYPES, _lib.OUT_FP8Q_SWIGLU: _FP8_DTYPES}[out_kind]
     n_out = N // 2 if out_kind == _lib.OUT_FP8Q_SWIGLU else N  # SwiGLU halves the width
-    a_p, as_p = _a_operand(A, As, M, K, a_swiglu)
+    a_p, as_p, a_layout, _keep = _a_operand(A, As, M, K, a_swiglu)
     b_p = _ptr(Bt, "B_transposed", _FP8_DTYPES, N * K)
     bs_p = _ptr(Bs, "B_scale_transposed", (torch.float32,), ((N + 127) // 128) * kb)
     c_p = _ptr(C, "C", c_dtypes, M * n_out)
     cs_p = _ptr(Cs, "C_scale_transposed", (torch.float32,), ((n_out + 127) // 128) * M) if out_kind in (_lib.OUT_FP8Q, _lib.OUT_FP8Q_SWIGLU) else None
     ws_p, ws_n = (ctypes.c_void_p(workspace.data_ptr()), workspace.numel() * workspace.element_size()) if workspace is not None else (None, 0)
-    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS, _lib.FP8_A_SWIGLU_F32 if a_swiglu else _lib.FP8_A_QUANTISED)
+    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS, a_layout)
     check(lib.llmmm_fp8_gemm_ex(out_kind, a_p, as_p, b_p, bs_p, c_p, cs_p, M, N, K, ws_p, ws_n, ctypes.byref(cfg), _stream(stream)))
 
 
@@ -219,8 +240,8 @@ def fp8_gemm_add_rmsnorm_quant(A, A_scale_transposed, B_transposed, B_scale_tran
         workspace = torch.empty(max(n, 16), dtype=torch.uint8, device=residual.device)
     q = torch.empty((M, N), dtype=torch.uint8, device=residual.device)
     s = torch.empty(((N + 127) // 128, M), dtype=torch.float32, device=residual.device)
-    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS, _lib.FP8_A_SWIGLU_F32 if a_swiglu else _lib.FP8_A_QUANTISED)
-    a_p, as_p = _a_operand(A, A_scale_transposed, M, K, a_swiglu)
+    a_p, as_p, a_layout, _keep = _a_operand(A, A_scale_transposed, M, K, a_swiglu)
+    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS, a_layout)
     check(lib.llmmm_fp8_gemm_add_rmsnorm_quant(
         a_p, as_p,
         _ptr(B_transposed, "B_transposed", _FP8_DTYPES, N * K), _ptr(B_scale_transposed, "B_scale_transposed", (torch.float32,), ((N + 127) // 128) * kb),
@@ -230,13 +251,32 @@ def fp8_gemm_add_rmsnorm_quant(A, A_scale_transposed, B_transposed, B_scale_tran
     return q, s
 
 
+def fp8_gemm_planes(A, A_scale_transposed, B_transposed, B_scale_transposed, M, N, K, planes=None, stream=None, workspace=None, tile=_lib.TILE_AUTO,
+                    split_k=0, b_preshuffled=False, a_swiglu=False):
+    """A projection that stops at its fp32 partial sums: returns (planes float32 [>= splits, M, N], splits).  Feed them to the next
+    projection as a :class:`PlanesRmsnorm` (residual add, RMSNorm and quantisation then happen in that projection's kernel)."""
+    if planes is None:
+        planes = torch.empty(max(int(lib.llmmm_fp8_gemm_planes_bytes(M, N, K)) // 4, max(split_k, 1) * M * N), dtype=torch.float32,
+                             device=B_transposed.device)
+    kb = K // 128 if K % 128 == 0 else 0
+    a_p, as_p, a_layout, _keep = _a_operand(A, A_scale_transposed, M, K, a_swiglu)
+    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS, a_layout)
+    splits = ctypes.c_int(0)
+    ws_p, ws_n = (ctypes.c_void_p(workspace.data_ptr()), workspace.numel() * workspace.element_size()) if workspace is not None else (None, 0)
+    check(lib.llmmm_fp8_gemm_planes(a_p, as_p, _ptr(B_transposed, "B_transposed", _FP8_DTYPES, N * K),
+                                    _ptr(B_scale_transposed, "B_scale_transposed", (torch.float32,), ((N + 127) // 128) * kb), M, N, K,
+                                    _ptr(planes, "planes", (torch.float32,), M * N), planes.numel() * 4, ctypes.byref(splits), ws_p, ws_n, ctypes.byref(cfg),
+                                    _stream(stream)))
+    return planes, splits.value
+
+
 def fp8_gemm_qkv_rope(A, A_scale_transposed, B_transposed, B_scale_transposed, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, positions,
                       n_q_heads, n_kv_heads, M, N, K, out_fp8=False, stream=None, workspace=None, tile=_lib.TILE_AUTO, split_k=0,
                       b_preshuffled=False):
     """The QKV projection with per-head RMSNorm (weights [128] or None) and rotate-half RoPE of the query and key heads fused
     behind it (planned by the reference, README.md:16).  Heads are 128 wide; cos_table / sin_table [rows, 64] float32,
     positions [M] int32.  Returns the bf16 tensor [M,N], or (codes uint8 [M,N], scales float32 [N/128, M]) with out_fp8."""
-    dev = A.device
+    dev = B_transposed.device
     kb = K // 128 if K % 128 == 0 else 0
     if workspace is None:
         n = int(lib.llmmm_fp8_gemm_qkv_rope_workspace(M, N, K))
@@ -244,9 +284,10 @@ def fp8_gemm_qkv_rope(A, A_scale_transposed, B_transposed, B_scale_transposed, q
     out = torch.empty((M, N), dtype=torch.uint8 if out_fp8 else torch.bfloat16, device=dev)
     sc = torch.empty(((N + 127) // 128, M), dtype=torch.float32, device=dev) if out_fp8 else None
     rows = cos_table.shape[0]
-    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS)
+    a_p, as_p, a_layout, _keep = _a_operand(A, A_scale_transposed, M, K, False)
+    cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS, a_layout)
     check(lib.llmmm_fp8_gemm_qkv_rope(
-        _lib.OUT_FP8Q if out_fp8 else _lib.OUT_BF16, _ptr(A, "A", _FP8_DTYPES, M * K), _ptr(A_scale_transposed, "A_scale_transposed", (torch.float32,), kb * M),
+        _lib.OUT_FP8Q if out_fp8 else _lib.OUT_BF16, a_p, as_p,
         _ptr(B_transposed, "B_transposed", _FP8_DTYPES, N * K), _ptr(B_scale_transposed, "B_scale_transposed", (torch.float32,), ((N + 127) // 128) * kb),
         _ptr(out, "out"), _ptr(sc, "out_scale") if out_fp8 else None,
         _ptr(q_norm_weight, "q_norm_weight", (torch.float32,), 128) if q_norm_weight is not None else None,

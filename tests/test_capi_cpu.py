@@ -260,6 +260,24 @@ def test_qkv_rope_validation_without_device():
     assert lib.llmmm_fp8_gemm_qkv_rope_workspace(M, N, K) >= plane
 
 
+def test_a_layout_validation_without_device():
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    M, N, K = 4, 2560, 9728
+
+    def call(cfg, As=None, ws=FAKE, wsz=1 << 30, kind=_lib.OUT_F32, m=M):
+        return lib.llmmm_fp8_gemm_ex(kind, FAKE, As, FAKE, FAKE, FAKE, FAKE, m, N, K, ws, wsz, ctypes.byref(cfg), None)
+
+    assert call(_lib.GemmCfg(-1, 0, 0, 7)) == _lib.ERR_INVALID_ARGUMENT                       # unknown A layout
+    assert call(_lib.GemmCfg(-1, 0, 0, 0)) == _lib.ERR_INVALID_ARGUMENT                       # quantised A needs its scales
+    assert call(_lib.GemmCfg(-1, 0, 0, 1), kind=_lib.OUT_FP8Q_SWIGLU) == _lib.ERR_INVALID_ARGUMENT  # SwiGLU on both sides
+    assert call(_lib.GemmCfg(_lib.TILE_SKINNY, 2, 0, 1)) == _lib.ERR_INVALID_ARGUMENT        # 76 slices: split-K >= 3
+    assert call(_lib.GemmCfg(_lib.TILE_SKINNY, 0, 0, 1), ws=None, wsz=0) == _lib.ERR_WORKSPACE
+    assert call(_lib.GemmCfg(_lib.TILE_SKINNY, 0, 0, 1), m=32, ws=None, wsz=0) == _lib.ERR_WORKSPACE  # M > 4: quantises into the workspace
+    assert lib.llmmm_fp8_swiglu_a_workspace(4, N, K) == 0
+    assert lib.llmmm_fp8_swiglu_a_workspace(32, N, K) >= 32 * K + (K // 128) * 32 * 4
+
+
 def test_the_64x128_tile_is_fp16_only():
     from llmmm_amd import _lib
     lib = _lib.lib
