@@ -287,12 +287,14 @@ def bench_qkv_rope(M, steps, warmup, rotate_bytes=768 << 20):
             "weight_copies": copies}
 
 
-def bench_decoder_layer(M, steps, warmup, rotate_bytes=768 << 20):
-    """The GEMM side of one Qwen3-4B decoder layer at decode-sized M as four entry points and no elementwise launch:
-    QKV + per-head RMSNorm + RoPE (bf16 out) -> [attention: not part of this library; a fixed quantised stand-in feeds O] ->
-    O + residual + RMSNorm + quant -> gate_up with SwiGLU output -> down + residual + RMSNorm + quant (the next layer's A).
-    Pre-shuffled weights, rotated over distinct copies so that they stream from HBM.  Algorithmic bytes: the four weight
-    matrices once (100.9 MB)."""
+def bench_decoder_layer(M, steps, warmup, rotate_bytes=768 << 20, consumer_side=False):
+    """The GEMM side of one Qwen3-4B decoder layer at decode-sized M with no elementwise launch between the projections
+    (attention is not part of this library; a fixed quantised stand-in feeds O).  Pre-shuffled weights, rotated over distinct
+    copies so that they stream from HBM.  Algorithmic bytes: the four weight matrices once (100.9 MB).
+      producer side: QKV + per-head RMSNorm + RoPE -> O + residual + RMSNorm + quant -> gate_up (fp32 out for M <= 4, the down
+                     kernel then makes silu(gate) * up itself; SwiGLU output otherwise) -> down + residual + RMSNorm + quant
+      consumer side (M <= 2): O and down stop at their fp32 planes; the next projection's kernel (gate_up; the next layer's QKV)
+                     sums them, adds the residual, normalises and quantises its own operand: five kernels per layer"""
     import llmmm_amd
     from llmmm_amd import _lib
     hidden, inter, n_q, n_kv = 2560, 9728, 32, 8
@@ -310,7 +312,7 @@ def bench_decoder_layer(M, steps, warmup, rotate_bytes=768 << 20):
             del W, q
         weights.append(layer)
     h0 = torch.randn((M, hidden), generator=g, device="cuda").to(torch.bfloat16)
-    h1, h2 = torch.empty_like(h0), torch.empty_like(h0)
+    h1, h2 = torch.empty_like(h0), torch.zeros_like(h0)
     wn = torch.ones(hidden, device="cuda")
     wh = torch.ones(128, device="cuda")
     Aq, As = llmmm_amd.rmsnorm_quantize_activation(h0, wn, 1e-6)
@@ -322,40 +324,49 @@ def bench_decoder_layer(M, steps, warmup, rotate_bytes=768 << 20):
     Hq = torch.empty((M, inter), dtype=torch.uint8, device="cuda")
     Hs = torch.empty((inter // 128, M), dtype=torch.float32, device="cuda")
     G32 = torch.empty((M, 2 * inter), dtype=torch.float32, device="cuda")
-
-    def ws_for(fn, n, k):
-        return torch.empty(max(16, int(fn(M, n, k))), dtype=torch.uint8, device="cuda")
-
-    ws_qkv = ws_for(_lib.lib.llmmm_fp8_gemm_qkv_rope_workspace, *shapes["qkv"])
-    ws_o = ws_for(_lib.lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace, *shapes["o"])
+    planes_o = torch.zeros((16, M, hidden), dtype=torch.float32, device="cuda")
+    planes_d = torch.zeros((16, M, hidden), dtype=torch.float32, device="cuda")
+    ws = torch.empty(32 << 20, dtype=torch.uint8, device="cuda")
     ws_gu = llmmm_amd.make_workspace(_lib.OUT_FP8Q_SWIGLU, M, *shapes["gate_up"])
-    ws_d = ws_for(_lib.lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace, *shapes["down"])
-    state = {"i": 0}
+    state = {"i": 0, "s_d": 10}
 
-    def step():
+    def producer_step():
         L = weights[state["i"] % copies]
         state["i"] += 1
-        llmmm_amd.fp8_gemm_qkv_rope(Aq, As, L["qkv"][0], L["qkv"][1], wh, wh, 1e-6, cos, sin, pos, n_q, n_kv, M, 6144, hidden, workspace=ws_qkv,
-                                    b_preshuffled=True)
-        q2, s2 = llmmm_amd.fp8_gemm_add_rmsnorm_quant(attn_q, attn_s, L["o"][0], L["o"][1], h0, h1, wn, 1e-6, M, hidden, 4096, workspace=ws_o,
-                                                      b_preshuffled=True)
+        llmmm_amd.fp8_gemm_qkv_rope(Aq, As, L["qkv"][0], L["qkv"][1], wh, wh, 1e-6, cos, sin, pos, n_q, n_kv, M, 6144, hidden, workspace=ws, b_preshuffled=True)
+        q2, s2 = llmmm_amd.fp8_gemm_add_rmsnorm_quant(attn_q, attn_s, L["o"][0], L["o"][1], h0, h1, wn, 1e-6, M, hidden, 4096, workspace=ws, b_preshuffled=True)
         if M <= 4:
-            # the activation on the consumer's side: gate_up with fp32 output (one kernel), the down projection's kernel quantises
-            # silu(gate) * up itself
             llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(q2, s2, L["gate_up"][0], L["gate_up"][1], G32, M, 2 * inter, hidden,
                                                                                b_preshuffled=True)
-            llmmm_amd.fp8_gemm_add_rmsnorm_quant(G32, None, L["down"][0], L["down"][1], h1, h2, wn, 1e-6, M, hidden, inter, workspace=ws_d, b_preshuffled=True,
+            llmmm_amd.fp8_gemm_add_rmsnorm_quant(G32, None, L["down"][0], L["down"][1], h1, h2, wn, 1e-6, M, hidden, inter, workspace=ws, b_preshuffled=True,
                                                  a_swiglu=True)
         else:
             llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(q2, s2, L["gate_up"][0], L["gate_up"][1], Hq, Hs, M, 2 * inter,
                                                                                                hidden, workspace=ws_gu, b_preshuffled=True)
-            llmmm_amd.fp8_gemm_add_rmsnorm_quant(Hq, Hs, L["down"][0], L["down"][1], h1, h2, wn, 1e-6, M, hidden, inter, workspace=ws_d, b_preshuffled=True)
+            llmmm_amd.fp8_gemm_add_rmsnorm_quant(Hq, Hs, L["down"][0], L["down"][1], h1, h2, wn, 1e-6, M, hidden, inter, workspace=ws, b_preshuffled=True)
 
-    ms, _ = _events_ms(step, steps, warmup, graph=True)
-    return {"name": "qwen3_4b_decoder_layer_gemms_m%d" % M, "M": M, "us": ms * 1e3, "weight_bytes": per_copy, "hbm_gbs": per_copy / ms * 1e-6,
-            "frac_of_hbm_peak": per_copy / ms * 1e-6 / PEAK_HBM_GBS, "weight_copies": copies,
-            "launches": ("qkv+norm+rope (2 kernels), o+add+norm+quant (2), gate_up fp32 (1), down on silu(gate)*up +add+norm+quant (2)" if M <= 4 else
-                         "qkv+norm+rope (2 kernels), o+add+norm+quant (2), gate_up+swiglu (2), down+add+norm+quant (2)") + "; attention not included"}
+    def consumer_step():
+        L = weights[state["i"] % copies]
+        state["i"] += 1
+        # this layer's QKV reads the previous layer's down planes (h2 = the residual they are added to, h0 = the new hidden state)
+        a_qkv = llmmm_amd.PlanesRmsnorm(planes_d, state["s_d"], h2, h0, wn, 1e-6)
+        llmmm_amd.fp8_gemm_qkv_rope(a_qkv, None, L["qkv"][0], L["qkv"][1], wh, wh, 1e-6, cos, sin, pos, n_q, n_kv, M, 6144, hidden, workspace=ws, b_preshuffled=True)
+        _, s_o = llmmm_amd.fp8_gemm_planes(attn_q, attn_s, L["o"][0], L["o"][1], M, hidden, 4096, planes=planes_o, b_preshuffled=True)
+        a_gu = llmmm_amd.PlanesRmsnorm(planes_o, s_o, h0, h1, wn, 1e-6)
+        llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(a_gu, None, L["gate_up"][0], L["gate_up"][1], G32, M, 2 * inter, hidden, b_preshuffled=True)
+        _, state["s_d"] = llmmm_amd.fp8_gemm_planes(G32, None, L["down"][0], L["down"][1], M, hidden, inter, planes=planes_d, b_preshuffled=True, a_swiglu=True,
+                                                   workspace=ws)
+
+    ms, _ = _events_ms(consumer_step if consumer_side else producer_step, steps, warmup, graph=True)
+    if consumer_side:
+        launches = "qkv on norm(down planes + residual) +norm+rope (2 kernels), o planes (1), gate_up fp32 on norm(o planes + residual) (1), down planes on silu(gate)*up (1)"
+    elif M <= 4:
+        launches = "qkv+norm+rope (2 kernels), o+add+norm+quant (2), gate_up fp32 (1), down on silu(gate)*up +add+norm+quant (2)"
+    else:
+        launches = "qkv+norm+rope (2 kernels), o+add+norm+quant (2), gate_up+swiglu (2), down+add+norm+quant (2)"
+    return {"name": "qwen3_4b_decoder_layer_gemms_m%d%s" % (M, "_consumer_side" if consumer_side else ""), "M": M, "us": ms * 1e3, "weight_bytes": per_copy,
+            "hbm_gbs": per_copy / ms * 1e-6, "frac_of_hbm_peak": per_copy / ms * 1e-6 / PEAK_HBM_GBS, "weight_copies": copies,
+            "launches": launches + "; attention not included"}
 
 
 def measured_peaks():
@@ -595,8 +606,8 @@ def main():
             shapes.append(bench_qkv_rope(m, s2 * 2 if m <= 16 else s2, w2))
             torch.cuda.empty_cache()
         # the GEMM side of a whole decoder layer through the four fused entry points
-        for m in (1, 16):
-            shapes.append(bench_decoder_layer(m, s2, w2))
+        for m, cs in ((1, False), (1, True), (2, True), (16, False)):
+            shapes.append(bench_decoder_layer(m, s2, w2, consumer_side=cs))
             torch.cuda.empty_cache()
         line["shapes"] = shapes
 

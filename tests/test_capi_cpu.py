@@ -278,6 +278,38 @@ def test_a_layout_validation_without_device():
     assert lib.llmmm_fp8_swiglu_a_workspace(32, N, K) >= 32 * K + (K // 128) * 32 * 4
 
 
+def test_planes_and_planes_rmsnorm_validation_without_device():
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    M, N, K = 1, 2560, 4096
+    splits = ctypes.c_int(0)
+    f = lib.llmmm_fp8_gemm_planes
+    need = lib.llmmm_fp8_gemm_planes_bytes(M, N, K)
+    assert need >= M * N * 4 and need % (M * N * 4) == 0
+    assert f(FAKE, FAKE, FAKE, FAKE, M, N, K, None, need, ctypes.byref(splits), None, 0, None, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(FAKE, FAKE, FAKE, FAKE, M, N, K, FAKE, need, None, None, 0, None, None) == _lib.ERR_INVALID_ARGUMENT
+    assert f(FAKE, FAKE, FAKE, FAKE, M, 100, K, FAKE, need, ctypes.byref(splits), None, 0, None, None) == _lib.ERR_NOT_ALIGNED
+    assert f(FAKE, FAKE, FAKE, FAKE, M, N, K, FAKE, M * N * 4 - 4, ctypes.byref(splits), None, 0, None, None) == _lib.ERR_WORKSPACE
+    cfg2 = _lib.GemmCfg(_lib.TILE_SKINNY, 2, 0, 0)
+    assert f(FAKE, FAKE, FAKE, FAKE, M, N, K, FAKE, M * N * 4, ctypes.byref(splits), None, 0, ctypes.byref(cfg2), None) == _lib.ERR_WORKSPACE
+    # the descriptor of a_layout = PLANES_RMSNORM is validated on the host
+    K2, N2 = 2560, 6144
+    cfg = _lib.GemmCfg(_lib.TILE_SKINNY, 0, 0, _lib.FP8_A_PLANES_RMSNORM)
+
+    def call(d):
+        return lib.llmmm_fp8_gemm_ex(_lib.OUT_F32, ctypes.byref(d), None, FAKE, FAKE, FAKE, None, M, N2, K2, FAKE, 1 << 30, ctypes.byref(cfg), None)
+
+    good = dict(planes=0x1000, splits=8, hidden_dtype=_lib.DTYPE_BF16, residual=0x2000, hidden_out=0x3000, norm_weight=0x4000, eps=1e-6)
+    assert call(_lib.APlanesRmsnorm(**dict(good, planes=None))) == _lib.ERR_INVALID_ARGUMENT
+    assert call(_lib.APlanesRmsnorm(**dict(good, splits=0))) == _lib.ERR_INVALID_ARGUMENT
+    assert call(_lib.APlanesRmsnorm(**dict(good, hidden_dtype=9))) == _lib.ERR_UNSUPPORTED_TYPE
+    assert call(_lib.APlanesRmsnorm(**dict(good, eps=-1.0))) == _lib.ERR_INVALID_ARGUMENT
+    assert call(_lib.APlanesRmsnorm(**dict(good, hidden_out=0x2000))) == _lib.ERR_INVALID_ARGUMENT  # in place: not when the kernel generates
+    assert call(_lib.APlanesRmsnorm(**dict(good, residual=0x2004))) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.llmmm_fp8_planes_rmsnorm_a_workspace(2, N2, K2) == 0
+    assert lib.llmmm_fp8_planes_rmsnorm_a_workspace(16, N2, K2) > 0
+
+
 def test_the_64x128_tile_is_fp16_only():
     from llmmm_amd import _lib
     lib = _lib.lib
