@@ -166,7 +166,8 @@ __device__ __forceinline__ void skinny_consume(const SkinnySlot<MBLK, APRE>& t, 
 // AGEN == 2: the activations are the RMSNorm of a hidden state that is itself still in pieces -- the fp32 planes of the
 // projection before (summed in split order), plus the residual: h = sum + residual, hidden = HT(h) (stored by workgroup
 // (0, 0, 0); it must not alias the residual, which every workgroup reads), A = quantise_1x128(rmsnorm(hidden) * w), in the
-// arithmetic and order of planes_add_rmsnorm_quant_kernel, bit for bit.  M <= 2, K <= 3072 (the row lives in registers).
+// arithmetic and order of planes_add_rmsnorm_quant_kernel, bit for bit.  M <= 2, K <= 3072 (the row lives in registers),
+// at most SKINNY_GEN_MAX_PLANES planes.
 template <int MBLK, int OUT, int D, int ASTG, int AGEN = 0, typename HT = float>
 __global__ void __launch_bounds__(512)
 fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
@@ -262,33 +263,50 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   // AGEN == 2: everything the generated operand needs is requested first, as hand-counted loads like the ring's, so that
   // it is the oldest traffic in flight: "at most D * LOADS outstanding" behind the ring prologue then means it has landed,
   // and the norm runs while the first weights are still on their way.
-  constexpr int GP = 10;  // planes requested up front (the split counts in use are 1 .. 10); more follow in a second batch
+  constexpr int GP = SKINNY_GEN_MAX_PLANES;  // all planes are requested up front (the split counts in use are 1 .. 10)
   i32x4         g_res[AGEN == 2 ? 3 : 1], g_w[AGEN == 2 ? 3 : 1], g_p[AGEN == 2 ? GP : 1][AGEN == 2 ? 3 : 1];
   i32x2         g_res2[AGEN == 2 ? 3 : 1];  // the residual chunk of a 2-byte hidden type (nothing may read these before the wait)
   if constexpr (AGEN == 2) {
     const int    vl = tid & 255, r = min(tid >> 8, M - 1), chunks = K >> 2;
     const size_t pplane = (size_t)M * K;
-    // (waves without a row of their own and planes beyond the split count request nothing: both conditions are uniform
-    // over a wave, and fewer old loads in flight only make the counted wait below easier to meet)
-    if ((tid >> 8) < M) {
+    // Straight-line code, every load unconditional: a register written by a load the compiler cannot see in flight must
+    // not pass through a copy before the counted wait, and conditional definitions invite such copies.  Loads that
+    // are not needed (waves without a row of their own, planes beyond the split count) all read one common address
+    // instead, which costs a single cache line per instruction.
+    const bool  own  = (tid >> 8) < M;
+    const char* idle = (const char*)ag.w;
 #pragma unroll
     for (int u = 0; u < 3; ++u) {
-      const int c = min(vl + 256 * u, chunks - 1);
+      const int   c  = min(vl + 256 * u, chunks - 1);
+      const char* rp = (const char*)((const HT*)ag.residual + (size_t)r * K + 4 * c);
       if constexpr (sizeof(HT) == 4)
-        asm_load_16B(g_res[u], (const HT*)ag.residual + (size_t)r * K + 4 * c);
+        asm_load_16B(g_res[u], own ? rp : idle);
       else
-        asm_load_8B(g_res2[u], (const HT*)ag.residual + (size_t)r * K + 4 * c);
-      asm_load_16B(g_w[u], ag.w + 4 * c);
+        asm_load_8B(g_res2[u], own ? rp : idle);
+      asm_load_16B(g_w[u], own ? (const char*)(ag.w + 4 * c) : idle);
     }
 #pragma unroll
     for (int v = 0; v < GP; ++v)
-      if (v < ag.splits) {
 #pragma unroll
-        for (int u = 0; u < 3; ++u) {
-          const int c = min(vl + 256 * u, chunks - 1);
-          asm_load_16B(g_p[v][u], ag.planes + (size_t)v * pplane + (size_t)r * K + 4 * c);
-        }
+      for (int u = 0; u < 3; ++u) {
+        const int   c  = min(vl + 256 * u, chunks - 1);
+        const char* pp = (const char*)(ag.planes + (size_t)min(v, ag.splits - 1) * pplane + (size_t)r * K + 4 * c);
+        asm_load_16B(g_p[v][u], own && v < ag.splits ? pp : idle);
       }
+  }
+  // AGEN == 1: likewise the gate and up values of the first four (row, slice) tasks of every half-wave (all of them for
+  // M * slices <= 64; later batches use ordinary loads)
+  i32x4 g_gate[AGEN == 1 ? 4 : 1], g_up[AGEN == 1 ? 4 : 1];
+  if constexpr (AGEN == 1) {
+    const float* G    = (const float*)A;
+    const int    rows = min(M, 16), tasks = (kb1 - kb0) * rows;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {  // unconditional loads (see above); tasks that do not exist read G's first bytes
+      const int    t  = (tid >> 5) + 16 * u, tc = min(t, tasks - 1);
+      const int    j  = tc / rows, r = tc - j * rows;
+      const float* gp = G + (size_t)r * 2 * K + (size_t)(kb0 + j) * 128 + 4 * (tid & 31);
+      asm_load_16B(g_gate[u], t < tasks ? gp : G);
+      asm_load_16B(g_up[u], t < tasks ? gp + K : G);
     }
   }
   SkinnySlot<MBLK, APRE> slot[D];
@@ -336,22 +354,6 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
 #pragma unroll
         for (int u = 0; u < 3; ++u) held[u] += __builtin_bit_cast(f32x4, g_p[v][u]);
       }
-    for (int s0 = GP; s0 < ag.splits; s0 += 8) {  // (more than GP planes: ordinary loads, eight in flight)
-      f32x4 p[8][3];
-#pragma unroll
-      for (int v = 0; v < 8; ++v)
-#pragma unroll
-        for (int u = 0; u < 3; ++u) {
-          const int c = min(vl + 256 * u, chunks - 1);
-          p[v][u]     = *(const f32x4*)(ag.planes + (size_t)min(s0 + v, ag.splits - 1) * pplane + (size_t)r * K + 4 * c);
-        }
-#pragma unroll
-      for (int v = 0; v < 8; ++v)
-        if (s0 + v < ag.splits) {
-#pragma unroll
-          for (int u = 0; u < 3; ++u) held[u] += p[v][u];
-        }
-    }
     float acc = 0.f;
 #pragma unroll
     for (int u = 0; u < 3; ++u) {
@@ -399,9 +401,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
     __syncthreads();  // the staged tile is complete
   }
   else if constexpr (AGEN == 1) {
-    // Behind the ring prologue (the weights are on their way): half a wavefront per row, a lane per four columns of a
-    // slice.  The loads below are ordinary ones; the waits the compiler puts behind them also cover the ring loads
-    // issued above, which only makes the hand-counted waits of the loop trivially true for the first pass.
+    // Half a wavefront per (row, slice) task, a lane per four columns of the slice.
     const float* G   = (const float*)A;
     const int    l32 = tid & 31;
     if (M < 16) {  // rows M .. 15 of every slice: zero codes, zero scales (their products are never stored)
@@ -409,16 +409,26 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
       for (int x = tid; x < (kb1 - kb0) * 16; x += 512) a_scale[x] = 0.f;
       __syncthreads();
     }
-    // (row, slice) tasks are dealt round-robin to the 16 half-waves: for M = 1 every half-wave has one slice to make
+    // (row, slice) tasks are dealt round-robin to the 16 half-waves: for M = 1 every half-wave has one slice to make.
+    // The first batch was requested in front of the ring prologue: once at most D * LOADS loads are outstanding it is in.
     const int nsl = kb1 - kb0, rows = min(M, 16), tasks = nsl * rows;
-    for (int t0 = tid >> 5; t0 < tasks; t0 += 16 * 4) {  // four tasks of a half-wave in flight
-      f32x4 gv[4], uv[4];
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * LOADS) : "memory");
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int    t  = min(t0 + 16 * u, tasks - 1), j = t / rows, r = t - j * rows;
-        const float* gp = G + (size_t)r * 2 * K + (size_t)(kb0 + j) * 128 + 4 * l32;
-        gv[u]           = *(const f32x4*)gp;
-        uv[u]           = *(const f32x4*)(gp + K);
+    for (int u = 0; u < 4; ++u) asm volatile("" : "+v"(g_gate[u]), "+v"(g_up[u]));
+    for (int t0 = tid >> 5; t0 < tasks; t0 += 16 * 4) {  // four tasks of a half-wave per batch
+      f32x4 gv[4], uv[4];
+      if (t0 < 16) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) gv[u] = __builtin_bit_cast(f32x4, g_gate[u]), uv[u] = __builtin_bit_cast(f32x4, g_up[u]);
+      }
+      else {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int    t  = min(t0 + 16 * u, tasks - 1), j = t / rows, r = t - j * rows;
+          const float* gp = G + (size_t)r * 2 * K + (size_t)(kb0 + j) * 128 + 4 * l32;
+          gv[u]           = *(const f32x4*)gp;
+          uv[u]           = *(const f32x4*)(gp + K);
+        }
       }
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
@@ -576,7 +586,7 @@ static hipError_t dispatch_skinny_gen2(const SkinnyGenA& ag, const void* Bt, con
                                        hipStream_t stream)
 {
   const int KB = K / 128, slices = KB / S, longest = (KB + S - 1) / S, need = 2048 * longest;
-  if (M > 2 || K > 3072 || need > 65536 || ag.splits < 1 || ag.hidden == ag.residual) return hipErrorInvalidValue;
+  if (M > 2 || K > 3072 || need > 65536 || ag.splits < 1 || ag.splits > SKINNY_GEN_MAX_PLANES || ag.hidden == ag.residual) return hipErrorInvalidValue;
 #define LLMMM_GO(D, ASTG)                                                                                                                       \
   {                                                                                                                                             \
     hipLaunchKernelGGL((fp8_skinny_kernel<1, SK_OUT_F32, D, ASTG, 2, HT>), dim3(N / 128, S, 1), dim3(512), 0, stream, (const uint8_t*)nullptr,  \

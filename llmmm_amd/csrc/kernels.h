@@ -57,6 +57,7 @@ hipError_t fp8_skinny_launch(int out_kind, int b_layout, const void* A, const fl
                              float* Cs, int M, int N, int K, int S, float* partial, hipStream_t stream);
 
 // What the weight-streaming kernel needs to make its activations from a hidden state that is still in pieces.
+constexpr int SKINNY_GEN_MAX_PLANES = 10;
 struct SkinnyGenA {
   const float* planes   = nullptr;  // [splits][M][K] fp32 partial sums of the projection before
   const void*  residual = nullptr;  // [M, K] of the hidden dtype
@@ -65,7 +66,7 @@ struct SkinnyGenA {
   float        eps      = 0.f;
   int          splits   = 0;
 };
-// The kernel with A = quantise_1x128(rmsnorm(hidden) * w), hidden = T(sum of planes + residual): M <= 2, K <= 3072, fp32
+// The kernel with A = quantise_1x128(rmsnorm(hidden) * w), hidden = T(sum of planes + residual): M <= 2, K <= 3072, at most SKINNY_GEN_MAX_PLANES planes, fp32
 // output (C, or planes `partial` as above).  hipErrorInvalidValue outside these limits.
 hipError_t fp8_skinny_rmsnorm_a_launch(int hidden_dtype, int b_layout, const SkinnyGenA& ag, const void* Bt, const float* Bs, float* C, int M, int N, int K,
                                        int S, float* partial, hipStream_t stream);
