@@ -424,7 +424,7 @@ def main():
     ap.add_argument("--workload", default="fp16_gemm_4096",
                     help="fp16_gemm_4096 (headline) | fp8_gemm_fused_4096 | fp8_gemm_bf16_4096 | bf16_gemm_4096 | "
                          "decode_<qkv|o|gate_up|down>_m<M>[_pre] (_pre: weights pre-shuffled offline) | prefill_<qkv|o|gate_up|down>_m<M> | "
-                         "prefill_gate_up_swiglu_m<M> | fused_<o|down>_add_norm_m<M> | fused_qkv_rope_m<M> | copy_1g (counter calibration only)")
+                         "prefill_gate_up_swiglu_m<M> | fused_<o|down>_add_norm_m<M> | fused_qkv_rope_m<M> | layer_[consumer_]m<M> | copy_1g (counter calibration only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measured-peak probes")
@@ -468,6 +468,22 @@ def main():
                 "kernel": "fp8_gemm_kernel<256,256,%s>" % out}
         value, unit = r["tflops"], "TFLOP/s"
         cfg = {"workload": "FP8 e4m3 blockwise GEMM M=N=K=4096 (A 1x128, B 128x128 scales), output %s" % out, "M": M, "N": N, "K": K}
+    elif w.startswith("layer_"):
+        import re
+        mo = re.fullmatch(r"layer_(consumer_)?m(\d+)", w)
+        if not mo or (mo.group(1) and int(mo.group(2)) > 2):
+            print("unknown workload", w, file=sys.stderr)
+            sys.exit(2)
+        M = int(mo.group(2))
+        x = bench_decoder_layer(M, args.steps, args.warmup, consumer_side=bool(mo.group(1)))
+        N, K = 0, 0
+        r = {"ms": x["us"] * 1e-3, "wall_ms": x["us"] * 1e-3, "bytes": float(x["weight_bytes"])}
+        dtype = "fp8"
+        roof = {"bound": "hbm", "achieved": x["hbm_gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": x["hbm_gbs"] / PEAK_HBM_GBS, "traffic": None,
+                "kernel": "fp8_skinny_kernel x 4 projections + second kernels"}
+        value, unit = x["hbm_gbs"], "GB/s"
+        cfg = {"workload": "GEMM side of one Qwen3-4B decoder layer at M=%d: %s; pre-shuffled weights rotated over %d copies"
+                           % (M, x["launches"], x["weight_copies"]), "M": M}
     elif w.startswith("fused_"):
         import re
         mo = re.fullmatch(r"fused_(o|down)_add_norm_m(\d+)|fused_qkv_rope_m(\d+)", w)
