@@ -209,9 +209,10 @@ LLMMM_API size_t llmmm_fp8_swiglu_a_workspace(int M, int N, int K);
  *   h = sum of the planes in split order + residual;  hidden_out = hidden_dtype(h);  A = quantise_1x128(rmsnorm(hidden_out) * w)
  * -- exactly the hidden state, codes and scales llmmm_fp8_gemm_add_rmsnorm_quant delivers, bit for bit.  For M <= 4 and
  * K <= 3072 every workgroup of the weight-streaming kernel makes the operand itself while its first weights are in flight
- * (no reduce kernel, no norm kernel: one launch per projection); hidden_out must then be a buffer of its own, not the
- * residual.  Otherwise the library runs the fused reduce + norm + quantise kernel into the front of the workspace first
- * (llmmm_fp8_planes_rmsnorm_a_workspace extra bytes).  Planned by the reference (README.md:16), no reference kernel. */
+ * (no reduce kernel, no norm kernel: one launch per projection), provided hidden_out is a buffer of its own, not the
+ * residual, and there are at most 10 planes.  Otherwise the library runs the fused reduce + norm + quantise kernel into the
+ * front of the workspace first (llmmm_fp8_planes_rmsnorm_a_workspace extra bytes, or M * K + K / 128 * M * 4 rounded up to
+ * 256 each when one of the provisos fails).  Planned by the reference (README.md:16), no reference kernel. */
 typedef struct llmmm_a_planes_rmsnorm {
   const float* planes;      /* [splits][M][K] fp32, from llmmm_fp8_gemm_planes */
   int          splits;

@@ -306,9 +306,9 @@ static int prepare_a(const llmmm_gemm_cfg* user, int tile, const void*& A, const
     if (K > 10240) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the fused norm handles rows of at most 10240 columns (got %d)", K);
     if (!aligned16(d->planes) || !aligned16(d->residual) || !aligned16(d->hidden_out) || !aligned16(d->norm_weight))
       return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
-    if (tile == LLMMM_TILE_SKINNY && M <= AGEN2_MAX_M && K <= AGEN2_MAX_K && d->splits <= llmmm::SKINNY_GEN_MAX_PLANES) {
-      // every workgroup reads the residual while one writes the hidden state: they must be different buffers
-      if (d->hidden_out == d->residual) return fail(LLMMM_ERR_INVALID_ARGUMENT, "hidden_out must not be the residual buffer when the kernel generates its activations (M <= %d)", AGEN2_MAX_M);
+    // (every generating workgroup reads the residual while one writes the hidden state: an in-place update takes the
+    // quantise-first route below, where one workgroup owns each row)
+    if (tile == LLMMM_TILE_SKINNY && M <= AGEN2_MAX_M && K <= AGEN2_MAX_K && d->splits <= llmmm::SKINNY_GEN_MAX_PLANES && d->hidden_out != d->residual) {
       prep->agen         = 2;
       prep->hidden_dtype = d->hidden_dtype;
       prep->ag.planes = d->planes, prep->ag.residual = d->residual, prep->ag.hidden = d->hidden_out, prep->ag.w = d->norm_weight;

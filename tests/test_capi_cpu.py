@@ -304,7 +304,6 @@ def test_planes_and_planes_rmsnorm_validation_without_device():
     assert call(_lib.APlanesRmsnorm(**dict(good, splits=0))) == _lib.ERR_INVALID_ARGUMENT
     assert call(_lib.APlanesRmsnorm(**dict(good, hidden_dtype=9))) == _lib.ERR_UNSUPPORTED_TYPE
     assert call(_lib.APlanesRmsnorm(**dict(good, eps=-1.0))) == _lib.ERR_INVALID_ARGUMENT
-    assert call(_lib.APlanesRmsnorm(**dict(good, hidden_out=0x2000))) == _lib.ERR_INVALID_ARGUMENT  # in place: not when the kernel generates
     assert call(_lib.APlanesRmsnorm(**dict(good, residual=0x2004))) == _lib.ERR_INVALID_ARGUMENT
     assert lib.llmmm_fp8_planes_rmsnorm_a_workspace(2, N2, K2) == 0
     assert lib.llmmm_fp8_planes_rmsnorm_a_workspace(16, N2, K2) > 0

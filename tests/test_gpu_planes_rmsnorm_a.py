@@ -97,7 +97,8 @@ def test_errors(lib, oracle):
     res = torch.zeros((M, H), dtype=torch.bfloat16, device="cuda")
     w = torch.ones(H, device="cuda")
     C = torch.empty((M, N2), device="cuda")
-    with pytest.raises(RuntimeError, match="must not be the residual"):
+    # an in-place hidden state cannot be generated by every workgroup: the quantise-first route takes over and needs its scratch
+    with pytest.raises(RuntimeError, match="workspace"):
         lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(lib.PlanesRmsnorm(planes, S, res, res, w, 1e-6), None, W2, W2s, C, M, N2, H, tile=SKINNY)
     with pytest.raises(RuntimeError, match="splits"):
         lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(lib.PlanesRmsnorm(planes, 0, res, torch.empty_like(res), w, 1e-6), None, W2, W2s, C, M, N2, H,
@@ -110,3 +111,26 @@ def test_errors(lib, oracle):
     lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(lib.PlanesRmsnorm(planes, S, res, hid, w, 1e-6), None, W2, W2s, C, M, N2, H, tile=SKINNY)
     torch.cuda.synchronize()
     assert float(hid.float().abs().max()) == 0.0 and float(C.abs().max()) == 0.0
+
+
+def test_in_place_hidden_state_falls_back_to_the_two_kernel_route(lib, oracle):
+    M, H, K1, N2 = 2, 2560, 1024, 512
+    rng = np.random.default_rng(11)
+    Aq, As = oracle.quant_fp8(rng.standard_normal((M, K1)).astype(np.float32), 1, True)
+    dA, dAs = torch.from_numpy(Aq).cuda(), torch.from_numpy(As).cuda()
+    W1, W1s = _weights(oracle, rng, H, K1)
+    W2, W2s = _weights(oracle, rng, N2, H)
+    res = torch.from_numpy(rng.standard_normal((M, H)).astype(np.float32)).cuda().to(torch.bfloat16)
+    w = torch.from_numpy(rng.uniform(0.5, 1.5, H).astype(np.float32)).cuda()
+    planes, S = lib.fp8_gemm_planes(dA, dAs, W1, W1s, M, H, K1, tile=SKINNY, split_k=4)
+    ws = torch.full((1 << 20,), 0xFF, dtype=torch.uint8, device="cuda")
+    out_of_place, in_place = torch.empty((M, N2), device="cuda"), torch.empty((M, N2), device="cuda")
+    hid = torch.empty_like(res)
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(lib.PlanesRmsnorm(planes, S, res, hid, w, 1e-6), None, W2, W2s, out_of_place, M, N2, H,
+                                                                 workspace=ws, tile=SKINNY, split_k=1)
+    res2 = res.clone()
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(lib.PlanesRmsnorm(planes, S, res2, res2, w, 1e-6), None, W2, W2s, in_place, M, N2, H,
+                                                                 workspace=ws, tile=SKINNY, split_k=1)
+    torch.cuda.synchronize()
+    assert torch.equal(res2.view(torch.int16), hid.view(torch.int16))
+    assert torch.equal(in_place.view(torch.int32), out_of_place.view(torch.int32))
