@@ -579,6 +579,11 @@ def main():
                      "frac_of_fp8_peak": x["tflops"] / PEAK_TFLOPS["fp8"], "tile": x["tile"], "split_k": x["split_k"]}
                 if m <= 128:
                     e.update({"hbm_gbs": x["gbs"], "frac_of_hbm_peak": x["gbs"] / PEAK_HBM_GBS, "weight_copies": x["weight_copies"]})
+                if m <= 16 and pre:
+                    # the same launch on one weight copy: served from the L2 / memory-side cache instead of HBM ("hot" next to the
+                    # "cold" figure above, which rotates over more copies than the caches hold)
+                    xh = bench_fp8(m, n, k, "fp8q", s2 * 2, w2, rotate_bytes=0, preshuffled=True)
+                    e["us_hot_cache"] = xh["ms"] * 1e3
                 shapes.append(e)
                 torch.cuda.empty_cache()
         # the gate_up projection with the SwiGLU activation fused in front of the C quantisation (output N/2 wide)
