@@ -12,15 +12,20 @@
 //
 // fp8_t stands for the reference's __nv_fp8_e4m3: one byte of OCP E4M3.  The launchers follow the
 // reference's rule M % 128 == 0, N % 128 == 0, K % 128 == 0 (examples/005.fp8.mm.cu:2490-2492) and
-// additionally accept 1 <= M <= 128 (decode), which the reference does not cover; small-M calls run
-// without split-K here because the reference signature has no workspace -- use llmmm_fp8_gemm()
-// with a workspace for the split-K path.
+// additionally accept 1 <= M <= 128 (decode), which the reference does not cover.  The reference
+// signatures have no workspace argument, so the split-K scratch of the small-M shapes comes from a
+// buffer these shims keep per host thread and stream (detail8::cached_workspace: allocated with
+// hipMalloc on first need, grown when a later call needs more, kept until the process ends).  Calls
+// on one stream are ordered, so one buffer per stream is race-free; a call that has to allocate must
+// not happen inside a stream capture -- run each shape once before capturing, or use llmmm_fp8_gemm()
+// with a workspace of your own.
 #pragma once
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 #include <stdexcept>
 #include <type_traits>
 #include <string>
+#include <unordered_map>
 
 #include "../../../llmmm.h"
 
@@ -38,6 +43,35 @@ inline void throw_on_error(int code)
   if (code == LLMMM_ERR_NOT_ALIGNED || code == LLMMM_ERR_UNSUPPORTED_TYPE) throw std::runtime_error(llmmm_error_string(code));
   throw std::runtime_error(std::string(llmmm_error_string(code)) + ": " + llmmm_last_error());
 }
+
+// Scratch for the split-K planes of a shim call: at least `bytes` (nullptr for 0), private to this host thread and
+// stream.  Growing frees the old buffer first (hipFree waits for the device, so no kernel still uses it).
+inline void* cached_workspace(hipStream_t stream, size_t bytes)
+{
+  struct Slot {
+    void*  ptr   = nullptr;
+    size_t bytes = 0;
+  };
+  static thread_local std::unordered_map<hipStream_t, Slot> slots;
+  if (bytes == 0) return nullptr;
+  Slot& s = slots[stream];
+  if (s.bytes < bytes) {
+    size_t want = size_t(1) << 20;
+    while (want < bytes) want <<= 1;
+    if (s.ptr) (void)hipFree(s.ptr);
+    s.ptr = nullptr, s.bytes = 0;
+    const hipError_t e = hipMalloc(&s.ptr, want);
+    if (e != hipSuccess) throw std::runtime_error(std::string("workspace allocation failed: ") + hipGetErrorString(e));
+    s.bytes = want;
+  }
+  return s.ptr;
+}
+
+inline void gemm(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K, hipStream_t stream)
+{
+  const size_t need = llmmm_fp8_gemm_workspace(out_kind, M, N, K);  // 0 for shapes that run unsplit (and for invalid ones)
+  throw_on_error(llmmm_fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, cached_workspace(stream, need), need, (void*)stream));
+}
 }  // namespace detail8
 
 template <int QUANT_M, int QUANT_N, bool SCALE_TRANSPOSE>
@@ -54,16 +88,14 @@ inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(const fp8_t
                                                                      const fp8_t* B_transposed, const float* B_scale_transposed,
                                                                      float* C, int M, int N, int K, hipStream_t stream)
 {
-  detail8::throw_on_error(
-    llmmm_fp8_gemm(LLMMM_OUT_F32, A, A_scale_transposed, B_transposed, B_scale_transposed, C, nullptr, M, N, K, nullptr, 0, (void*)stream));
+  detail8::gemm(LLMMM_OUT_F32, A, A_scale_transposed, B_transposed, B_scale_transposed, C, nullptr, M, N, K, stream);
 }
 
 inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(const fp8_t* A, const float* A_scale_transposed,
                                                                      const fp8_t* B_transposed, const float* B_scale_transposed,
                                                                      void* C, int M, int N, int K, hipStream_t stream)
 {
-  detail8::throw_on_error(
-    llmmm_fp8_gemm(LLMMM_OUT_BF16, A, A_scale_transposed, B_transposed, B_scale_transposed, C, nullptr, M, N, K, nullptr, 0, (void*)stream));
+  detail8::gemm(LLMMM_OUT_BF16, A, A_scale_transposed, B_transposed, B_scale_transposed, C, nullptr, M, N, K, stream);
 }
 
 inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(const fp8_t* A, const float* A_scale_transposed,
@@ -72,8 +104,7 @@ inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(con
                                                                              float* C_scale_transposed, int M, int N, int K,
                                                                              hipStream_t stream)
 {
-  detail8::throw_on_error(llmmm_fp8_gemm(LLMMM_OUT_FP8Q, A, A_scale_transposed, B_transposed, B_scale_transposed, C, C_scale_transposed, M,
-                                         N, K, nullptr, 0, (void*)stream));
+  detail8::gemm(LLMMM_OUT_FP8Q, A, A_scale_transposed, B_transposed, B_scale_transposed, C, C_scale_transposed, M, N, K, stream);
 }
 
 // RMSNorm fused in front of the 1x128 activation quantiser (planned by the reference, README.md:16; no reference
@@ -90,16 +121,14 @@ void rmsnorm_fp8_blockwise_symmetric_quantization(const T* x, const float* weigh
 
 // The gate_up projection of a gated MLP with silu(gate) * up fused in front of the C quantisation -- the
 // fusion the reference plans (README.md:16), no reference kernel.  B_transposed [N,K]: gate rows in
-// [0, N/2), up rows in [N/2, N); C [M, N/2] e4m3, C_scale_transposed [N/256, M].  M % 128 == 0 through
-// this signature (smaller M needs a workspace: llmmm_fp8_gemm with LLMMM_OUT_FP8Q_SWIGLU).
+// [0, N/2), up rows in [N/2, N); C [M, N/2] e4m3, C_scale_transposed [N/256, M].
 inline void fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(const fp8_t* A, const float* A_scale_transposed,
                                                                                      const fp8_t* B_transposed,
                                                                                      const float* B_scale_transposed, fp8_t* C,
                                                                                      float* C_scale_transposed, int M, int N, int K,
                                                                                      hipStream_t stream)
 {
-  detail8::throw_on_error(llmmm_fp8_gemm(LLMMM_OUT_FP8Q_SWIGLU, A, A_scale_transposed, B_transposed, B_scale_transposed, C,
-                                         C_scale_transposed, M, N, K, nullptr, 0, (void*)stream));
+  detail8::gemm(LLMMM_OUT_FP8Q_SWIGLU, A, A_scale_transposed, B_transposed, B_scale_transposed, C, C_scale_transposed, M, N, K, stream);
 }
 
 // A projection back to the hidden size (O, down) with the decoder block's epilogue behind it -- residual add, the next

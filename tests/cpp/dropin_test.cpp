@@ -188,6 +188,44 @@ int main()
     if (!throws_with([&] { LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__add_rmsnorm__output_fp8<float>(dAq, dAs, dBq, dBs, dRes, dHid, dW, 1e-6f, dQ, dQs, M, 100, K, dWs, wsz, nullptr); },
                      "M or N or K are not aligned.")) { ++fails; printf("fused misaligned N: FAIL\n"); }
   }
+  // ---- decode-sized calls through the reference signatures: the shims bring the split-K scratch themselves (a per-thread,
+  // per-stream cached buffer) and must give the bits of the C API with an explicit workspace
+  {
+    int fd = 0;
+    const int shapes[2][3] = {{16, 2560, 4096}, {5, 2560, 9728}};  // the second needs a larger buffer: the cache grows
+    for (const auto& sh : shapes) {
+      const int m = sh[0], n = sh[1], k = sh[2];
+      llmmm_gemm_cfg qc;
+      if (llmmm_fp8_gemm_query(LLMMM_OUT_FP8Q, m, n, k, &qc) != LLMMM_OK || qc.split_k < 2) { ++fd; printf("expected a split-K shape\n"); }
+      std::vector<float> fx((size_t)m * k), fw((size_t)n * k);
+      for (auto& v : fx) { s = s * 1664525u + 1013904223u; v = ((s >> 8) / 16777216.0f) * 4.f - 2.f; }
+      for (auto& v : fw) { s = s * 1664525u + 1013904223u; v = ((s >> 8) / 16777216.0f) * 0.1f - 0.05f; }
+      float *dx, *dw, *das, *dbs, *dcs0, *dcs1;
+      LLMMM::fp8_t *daq, *dbq, *dc0, *dc1;
+      void*         ws;
+      const size_t  wsz = llmmm_fp8_gemm_workspace(LLMMM_OUT_FP8Q, m, n, k);
+      CHECK(hipMalloc(&dx, fx.size() * 4)); CHECK(hipMalloc(&dw, fw.size() * 4)); CHECK(hipMalloc(&daq, (size_t)m * k)); CHECK(hipMalloc(&dbq, (size_t)n * k));
+      CHECK(hipMalloc(&das, (k / 128) * m * 4)); CHECK(hipMalloc(&dbs, (n / 128) * (k / 128) * 4)); CHECK(hipMalloc(&dc0, (size_t)m * n)); CHECK(hipMalloc(&dc1, (size_t)m * n));
+      CHECK(hipMalloc(&dcs0, (n / 128) * m * 4)); CHECK(hipMalloc(&dcs1, (n / 128) * m * 4)); CHECK(hipMalloc(&ws, wsz));
+      CHECK(hipMemcpy(dx, fx.data(), fx.size() * 4, hipMemcpyHostToDevice));
+      CHECK(hipMemcpy(dw, fw.data(), fw.size() * 4, hipMemcpyHostToDevice));
+      LLMMM::fp8_blockwise_symmetric_quantization<1, 128, true>(dx, daq, das, m, k, nullptr);
+      LLMMM::fp8_blockwise_symmetric_quantization<128, 128, false>(dw, dbq, dbs, n, k, nullptr);
+      LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(daq, das, dbq, dbs, dc0, dcs0, m, n, k, nullptr);
+      if (llmmm_fp8_gemm(LLMMM_OUT_FP8Q, daq, das, dbq, dbs, dc1, dcs1, m, n, k, ws, wsz, nullptr) != LLMMM_OK) ++fd;
+      CHECK(hipDeviceSynchronize());
+      std::vector<unsigned char> h0((size_t)m * n), h1((size_t)m * n);
+      std::vector<float>         s0((n / 128) * m), s1((n / 128) * m);
+      CHECK(hipMemcpy(h0.data(), dc0, h0.size(), hipMemcpyDeviceToHost)); CHECK(hipMemcpy(h1.data(), dc1, h1.size(), hipMemcpyDeviceToHost));
+      CHECK(hipMemcpy(s0.data(), dcs0, s0.size() * 4, hipMemcpyDeviceToHost)); CHECK(hipMemcpy(s1.data(), dcs1, s1.size() * 4, hipMemcpyDeviceToHost));
+      if (memcmp(h0.data(), h1.data(), h0.size()) != 0 || memcmp(s0.data(), s1.data(), s0.size() * 4) != 0) ++fd;
+      bool any = false;
+      for (unsigned char c : h0) any |= (c & 0x7f) != 0;
+      if (!any) ++fd;
+    }
+    printf("decode shapes through the reference signatures (cached split-K workspace): %s\n", fd ? "FAIL" : "ok");
+    fails += fd;
+  }
   printf(fails ? "DROPIN FAIL (%d)\n" : "DROPIN OK\n", fails);
   return fails ? 1 : 0;
 }
