@@ -63,6 +63,8 @@ extern "C" {
 #define LLMMM_TILE_256x128 2
 #define LLMMM_TILE_128x128 3
 #define LLMMM_TILE_64x128 4 /* FP16/BF16 GEMM only: small problems */
+#define LLMMM_TILE_128x160 5 /* FP8 GEMM only, N % 160 == 0, fp32 / bf16 / residual-add outputs (no 1x128-grouped epilogue):
+                              * 2560-column outputs in 16 tiles per row -- one tile per CU at M = 2048 */
 #define LLMMM_TILE_SKINNY 8 /* M <= 128 weight-streaming kernel */
 
 /* Weight layout of the FP8 GEMM's B operand (llmmm_gemm_cfg.b_layout). */

@@ -28,7 +28,7 @@ class APlanesRmsnorm(ctypes.Structure):
     _fields_ = [("planes", ctypes.c_void_p), ("splits", ctypes.c_int), ("hidden_dtype", ctypes.c_int), ("residual", ctypes.c_void_p),
                 ("hidden_out", ctypes.c_void_p), ("norm_weight", ctypes.c_void_p), ("eps", ctypes.c_float)]
 PROBE_FP8 = 2
-TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_64x128, TILE_SKINNY = -1, 0, 1, 2, 3, 4, 8
+TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_64x128, TILE_128x160, TILE_SKINNY = -1, 0, 1, 2, 3, 4, 5, 8
 
 
 class GemmCfg(ctypes.Structure):

@@ -45,12 +45,15 @@ __device__ __forceinline__ f32x4 mfma_fp8_k128(i32x8 x, i32x8 y)
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(x, y, z, 0, 0, 0, 0, 0, 0);
 }
 
-// WM = rows of a wave's sub-tile (64 or 32); its columns are always 128, one quantisation group.
+// WM = rows of a wave's sub-tile (64 or 32); its columns are 128, one quantisation group -- or, in the 160-column tile
+// (BN = 160: 2560-column outputs in 16 tiles per row, one per CU at M = 2048), 160, which straddle two weight-scale blocks.
 template <int BM, int BN, int WM>
 struct Fp8Tile {
   static constexpr int MF      = WM / 16;  // 16-row fragments per wave
+  static constexpr int WN      = BN % 128 == 0 ? 128 : BN;  // columns of a wave
+  static constexpr int NF      = WN / 16;                   // 16-column fragments per wave
   static constexpr int WAVES_M = BM / WM;
-  static constexpr int WAVES_N = BN / 128;
+  static constexpr int WAVES_N = BN / WN;
   static constexpr int NW      = WAVES_M * WAVES_N;
   static constexpr int NT      = NW * 64;
   static constexpr int A_BYTES = BM * 128;
@@ -116,8 +119,10 @@ __device__ __forceinline__ void fp8_issue_loads(unsigned lds_stage, const uint8_
   }
 }
 // The slice scales of the lane's four 16-row fragments and of the wave's column group.
-template <int MF>
-__device__ __forceinline__ void fp8_issue_scales(float (&sa)[MF], float& sb, const float* As_slice, unsigned row_off, const float* Bs_elem, unsigned zero)
+// (TWO: a 160-column wave also takes the scale of the next weight block, Bs_elem2.)
+template <int MF, bool TWO = false>
+__device__ __forceinline__ void fp8_issue_scales(float (&sa)[MF], float& sb, const float* As_slice, unsigned row_off, const float* Bs_elem, unsigned zero,
+                                                 float* sb2 = nullptr, const float* Bs_elem2 = nullptr)
 {
   fp8_load_f32<0>(sa[0], As_slice, row_off);
   fp8_load_f32<64>(sa[1], As_slice, row_off);
@@ -126,6 +131,7 @@ __device__ __forceinline__ void fp8_issue_scales(float (&sa)[MF], float& sb, con
     fp8_load_f32<192>(sa[3], As_slice, row_off);
   }
   fp8_load_f32<0>(sb, Bs_elem, zero);
+  if constexpr (TWO) fp8_load_f32<0>(*sb2, Bs_elem2, zero);
 }
 
 // 32 bytes of one row: chunk 2g at rd0 and chunk 2g+1 at rd1 (= rd0 ^ 16); `imm` selects the
@@ -148,6 +154,7 @@ struct Fp8Next {
   const uint8_t* Bg;
   const float*   As_slice;   // As + kb_next * M
   const float*   Bs_elem;    // &Bs[nb, kb_next]
+  const float*   Bs_elem2;   // 160-column waves: &Bs[nb + 1, kb_next]
   const char*    sc_ptr;     // deep pipeline only: this lane's scale of the slice being requested (see fp8_scale_load_lds)
 };
 
@@ -163,14 +170,17 @@ __device__ __forceinline__ void fp8_scale_load_lds(const char* lane_ptr, unsigne
 // With LOAD, the next stage's loads go out two or more per fragment step during the first four
 // steps (spread, so that no wave sits in the memory pipeline's issue queue while its matrix
 // work waits, and early enough to land within the slice), its scales during the fifth.
+// 160-column waves (NF = 10): fragments nf < nfb lie in the first weight-scale block and take s, the others s2.
 template <int BM, int BN, int WM, bool BNT, bool LOAD, bool SCALE_LDS = false>
 __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int a_rd0, int a_rd1, int b_rd0, int b_rd1,
-                                                  const float (&s)[WM / 16], f32x4 (&acc)[8][WM / 16], const Fp8Next& nx, unsigned lane_off,
+                                                  const float (&s)[WM / 16], f32x4 (&acc)[Fp8Tile<BM, BN, WM>::NF][WM / 16], const Fp8Next& nx, unsigned lane_off,
                                                   unsigned b_lane_off, unsigned row_off, unsigned zero, int K, size_t b_hi, int wave, float (&sa_next)[WM / 16],
-                                                  float& sb_next)
+                                                  float& sb_next, const float (&s2)[WM / 16], int nfb, float& sb2_next)
 {
   constexpr int MF = WM / 16;
   typedef Fp8Tile<BM, BN, WM> TC;
+  constexpr int  NF  = TC::NF;
+  constexpr bool TWO = NF != 8;
   constexpr int           NL   = TC::A_LOADS + TC::B_LOADS;
   constexpr int           LPG  = (NL + 3) / 4;
   const char LLMMM_LDS*   ldsA = lds;
@@ -181,9 +191,9 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int
 #pragma unroll
   for (int mf = 0; mf < MF; ++mf) a[mf] = fp8_read_frag(ldsA, a_rd0, a_rd1, mf * 2048);
 #pragma unroll
-  for (int nf = 0; nf < 8; ++nf) {
+  for (int nf = 0; nf < NF; ++nf) {
     const int cur = nf & 1;
-    if (nf + 1 < 8) b[cur ^ 1] = fp8_read_frag(ldsB, b_rd0, b_rd1, (nf + 1) * 2048);
+    if (nf + 1 < NF) b[cur ^ 1] = fp8_read_frag(ldsB, b_rd0, b_rd1, (nf + 1) * 2048);
     if constexpr (LOAD) {
       if (nf == 0) fp8_issue_loads<BM, BN, WM, BNT, 0, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
       if (nf == 1) fp8_issue_loads<BM, BN, WM, BNT, LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
@@ -193,7 +203,7 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int
         if constexpr (SCALE_LDS)
           fp8_scale_load_lds(nx.sc_ptr, nx.lds_stage + TC::STAGE + wave * 256);
         else
-          fp8_issue_scales<MF>(sa_next, sb_next, nx.As_slice, row_off, nx.Bs_elem, zero);
+          fp8_issue_scales<MF, TWO>(sa_next, sb_next, nx.As_slice, row_off, nx.Bs_elem, zero, &sb2_next, nx.Bs_elem2);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -201,9 +211,11 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int
     for (int mf = 0; mf < MF; ++mf) p[cur][mf] = mfma_fp8_k128(b[cur], a[mf]);
     if (nf > 0) {
 #pragma unroll
-      for (int mf = 0; mf < MF; ++mf)
+      for (int mf = 0; mf < MF; ++mf) {
+        const float sc = TWO ? (nf - 1 < nfb ? s[mf] : s2[mf]) : s[mf];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[nf - 1][mf][r] = __builtin_fmaf(p[cur ^ 1][mf][r], s[mf], acc[nf - 1][mf][r]);
+        for (int r = 0; r < 4; ++r) acc[nf - 1][mf][r] = __builtin_fmaf(p[cur ^ 1][mf][r], sc, acc[nf - 1][mf][r]);
+      }
       // Pin the promotion here (an empty asm the optimiser cannot move or sink), then ask for
       // MFMA, 4 FMA, MFMA, 4 FMA ...: the FMAs of fragment nf-1 run under the MFMAs of fragment nf.
 #pragma unroll
@@ -217,11 +229,13 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int
     __builtin_amdgcn_sched_barrier(0);
   }
 #pragma unroll
-  for (int mf = 0; mf < MF; ++mf)
+  for (int mf = 0; mf < MF; ++mf) {
+    const float sc = TWO ? (NF - 1 < nfb ? s[mf] : s2[mf]) : s[mf];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) acc[7][mf][r] = __builtin_fmaf(p[1][mf][r], s[mf], acc[7][mf][r]);
+    for (int r = 0; r < 4; ++r) acc[NF - 1][mf][r] = __builtin_fmaf(p[(NF - 1) & 1][mf][r], sc, acc[NF - 1][mf][r]);
+  }
 #pragma unroll
-  for (int mf = 0; mf < MF; ++mf) asm volatile("" : "+v"(acc[7][mf]));
+  for (int mf = 0; mf < MF; ++mf) asm volatile("" : "+v"(acc[NF - 1][mf]));
 }
 
 __device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float d)
@@ -364,6 +378,10 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
 {
   typedef Fp8Tile<BM, BN, WM> TC;
   constexpr int  MF   = TC::MF;
+  constexpr int  NF   = TC::NF;
+  constexpr bool TWO  = NF != 8;  // 160-column waves straddle two weight-scale blocks
+  static_assert(!TWO || (OUT == OUT_F32 || OUT == OUT_BF16 || OUT == OUT_ADD_F32 || OUT == OUT_ADD_BF16 || OUT == OUT_ADD_F16),
+                "the 160-column tile has no 1x128-grouped epilogues");
   constexpr bool BPRE = (BMODE & 1) != 0, BNT = (BMODE & 2) != 0;
   // A launch with at most one workgroup per CU (few tiles: decode-sized or mid-sized M) leaves the workgroups
   // waiting on memory latency, not on the matrix pipe, and the LDS a second workgroup would have used lies idle:
@@ -410,11 +428,11 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   // 32 bytes k = 32g .. 32g+31 (chunks 2g and 2g+1)
   const int g     = lane >> 4;
   const int a_rd0 = kmajor_offset<SWZ_ROWS16>(wm * WM + (lane & 15), 2 * g), a_rd1 = a_rd0 ^ 16;
-  const int b_rd0 = kmajor_offset<SWZ_ROWS16>(wn * 128 + (lane & 15), 2 * g), b_rd1 = b_rd0 ^ 16;
+  const int b_rd0 = kmajor_offset<SWZ_ROWS16>(wn * TC::WN + (lane & 15), 2 * g), b_rd1 = b_rd0 ^ 16;
 
-  f32x4 acc[8][MF];
+  f32x4 acc[NF][MF];
 #pragma unroll
-  for (int nf = 0; nf < 8; ++nf)
+  for (int nf = 0; nf < NF; ++nf)
 #pragma unroll
     for (int mf = 0; mf < MF; ++mf) acc[nf][mf] = f32x4{0.f, 0.f, 0.f, 0.f};
 
@@ -422,10 +440,14 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const int      mrow    = m0 + wm * WM + (lane & 15);
   const unsigned row_off = (unsigned)mrow * 4u;
   const float*   Bsp     = Bs + (size_t)((n0 >> 7) + (SWIGLU ? wn * (N >> 8) : wn)) * KB + kb0;
+  // 160-column waves: columns n0 .. n0+159 lie in weight-scale blocks n0/128 and n0/128 + 1; the first nfb fragments
+  // (16 columns each) belong to the former
+  const float*   Bsp2    = Bsp + (TWO ? KB : 0);
+  const int      nfb     = TWO ? (128 - (n0 & 127)) >> 4 : NF;
   const float*   Asl     = As + (size_t)kb0 * M;
   unsigned       zero    = 0;
   asm volatile("" : "+v"(zero));  // a VGPR holding 0: the per-lane offset of the wave-uniform Bs load
-  float sa_next[MF], sb_next;
+  float sa_next[MF], sb_next, sb2_next = 0.f;
 
   const unsigned lds0 = (unsigned)(size_t)(char LLMMM_LDS*)lds;
   char LLMMM_LDS* const s0 = (char LLMMM_LDS*)lds;
@@ -435,7 +457,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
     static_assert((NST - 2) * PER < 64, "vmcnt is a 6-bit counter");
     // this lane's scale source: a row scale (stride M floats per slice) or the column-group scale (stride 1)
     const bool     row_lane = lane < WM;
-    const char*    sc_ptr   = row_lane ? (const char*)(Asl + (m0 + wm * WM + lane)) : (const char*)Bsp;
+    const char*    sc_ptr   = row_lane ? (const char*)(Asl + (m0 + wm * WM + lane)) : (const char*)(TWO && lane >= 48 ? Bsp2 : Bsp);
     const unsigned sc_step  = row_lane ? (unsigned)M * 4u : 4u;
     // prologue: slices 0 .. NST-2 (a K range shorter than that repeats its last slice into the spare stages)
 #pragma unroll
@@ -453,18 +475,22 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
     wait_vmcnt<(WAIT)>();                                                                                                         \
     __syncthreads();                                                                                                              \
     const float LLMMM_LDS* sc_ = (const float LLMMM_LDS*)((const char LLMMM_LDS*)my_scales + cur);                                \
-    float                  s[MF];                                                                                                 \
-    const float            sb_ = sc_[32];                                                                                         \
-    _Pragma("unroll") for (int mf = 0; mf < MF; ++mf) s[mf] = sc_[mf * 16 + (lane & 15)] * sb_;                                    \
+    float                  s[MF], s2[MF];                                                                                         \
+    const float            sb_ = sc_[32], sb2_ = sc_[48];                                                                         \
+    _Pragma("unroll") for (int mf = 0; mf < MF; ++mf) {                                                                            \
+      const float sa_ = sc_[mf * 16 + (lane & 15)];                                                                               \
+      s[mf] = sa_ * sb_, s2[mf] = sa_ * sb2_;                                                                                     \
+    }                                                                                                                             \
     Fp8Next nx;                                                                                                                   \
     nx.lds_stage = lds0 + (cur == 0 ? (NST - 1) * STAGE_D : cur - STAGE_D);                                                       \
     nx.Ag        = Ag + (size_t)(kc + NST - 1) * 128;                                                                             \
     nx.Bg        = Bg + (size_t)(kc + NST - 1) * B_KSTEP;                                                                         \
     nx.As_slice  = nullptr;                                                                                                       \
     nx.Bs_elem   = nullptr;                                                                                                       \
+    nx.Bs_elem2  = nullptr;                                                                                                       \
     nx.sc_ptr    = sc_next;                                                                                                       \
     fp8_compute_stage<BM, BN, WM, BNT, LOAD, true>(s0 + cur, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, b_lane_off, row_off, zero, K, b_hi, \
-                                                   wave, sa_next, sb_next);                                                       \
+                                                   wave, sa_next, sb_next, s2, nfb, sb2_next);                                    \
     cur = cur + STAGE_D == NST * STAGE_D ? 0 : cur + STAGE_D;                                                                     \
   }
     int kc = 0;
@@ -482,7 +508,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   }
   else {
   fp8_issue_loads<BM, BN, WM, BNT, 0, TC::A_LOADS + TC::B_LOADS>(lds0, Ag, Bg, lane_off, b_lane_off, K, b_hi, wave);
-  fp8_issue_scales<MF>(sa_next, sb_next, Asl, row_off, Bsp, zero);
+  fp8_issue_scales<MF, TWO>(sa_next, sb_next, Asl, row_off, Bsp, zero, &sb2_next, Bsp2);
 
   // One slice: wait for this wave's loads of the slice (all of them were issued at least half a
   // slice ago), meet the other waves, then compute it while the loads of the next one go out.
@@ -493,17 +519,19 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
       asm volatile("" : "+v"(sa_next[0]), "+v"(sa_next[1]), "+v"(sa_next[2]), "+v"(sa_next[MF - 1]), "+v"(sb_next));              \
     else                                                                                                                          \
       asm volatile("" : "+v"(sa_next[0]), "+v"(sa_next[1]), "+v"(sb_next));                                                       \
+    if constexpr (TWO) asm volatile("" : "+v"(sb2_next));                                                                         \
     __syncthreads();                                                                                                              \
-    float s[MF];                                                                                                                  \
-    _Pragma("unroll") for (int mf = 0; mf < MF; ++mf) s[mf] = sa_next[mf] * sb_next;                                               \
+    float s[MF], s2[MF];                                                                                                          \
+    _Pragma("unroll") for (int mf = 0; mf < MF; ++mf) s[mf] = sa_next[mf] * sb_next, s2[mf] = sa_next[mf] * sb2_next;              \
     Fp8Next nx;                                                                                                                   \
     nx.lds_stage = NXT_LDS;                                                                                                       \
     nx.Ag        = Ag + (size_t)((KC) + 1) * 128;                                                                                 \
     nx.Bg        = Bg + (size_t)((KC) + 1) * B_KSTEP;                                                                               \
     nx.As_slice  = Asl + (size_t)((KC) + 1) * M;                                                                                  \
     nx.Bs_elem   = Bsp + (KC) + 1;                                                                                                \
+    nx.Bs_elem2  = Bsp2 + (KC) + 1;                                                                                               \
     fp8_compute_stage<BM, BN, WM, BNT, LOAD>(CUR, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, b_lane_off, row_off, zero, K, b_hi, wave, sa_next, \
-                                    sb_next);                                                                                     \
+                                    sb_next, s2, nfb, sb2_next);                                                                  \
   }
 
   unsigned cur = 0;  // byte offset of the stage being computed: 0 or STAGE
@@ -522,12 +550,60 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   // buffers -- 16-byte chunks XOR-ed with row bits so that neither the writes nor the
   // ds_read_b128 reads conflict -- and stores it back out 16 bytes per lane, whole rows at a time.
   __syncthreads();  // every wave is done reading the last operand stage
-  char LLMMM_LDS* const stg  = s0 + wave * (WM * 256);  // WM rows of up to 256 bytes; fp32 goes 16 rows at a time
+  // WM rows of up to 256 bytes (fp32 goes 16 rows at a time); 160-column waves pad their rows by 16 bytes instead of XOR-ing chunks
+  constexpr int         RS32 = TC::WN * 4 + 16, RS16 = TC::WN * 2 + 16;  // padded row strides of the 160-column staging
+  char LLMMM_LDS* const stg  = s0 + wave * (TWO ? (16 * RS32 > WM * RS16 ? 16 * RS32 : WM * RS16) : WM * 256);
   const int             row0 = m0 + wm * WM;
-  const int             col0 = n0 + wn * 128;
+  const int             col0 = n0 + wn * TC::WN;
   const int             li   = lane & 15;
   if constexpr (OUT == OUT_ROPE_BF16 || OUT == OUT_ROPE_FP8Q) qk_norm_rope_fragments<MF>(acc, op, col0 >> 7, row0, lane);
-  if constexpr (OUT == OUT_F32) {
+  if constexpr (TWO) {
+    // 160-column waves: the same staging with padded rows instead of the chunk XOR (a row is 40 or 20 chunks, not a power
+    // of two), 16-byte chunks dealt to the lanes in row-major order
+    constexpr int CH32 = TC::WN / 4, CH16 = TC::WN / 8;  // 16-byte chunks per row: fp32, 2-byte types
+    if constexpr (OUT == OUT_BF16) {
+      __bf16* C = (__bf16*)Cv;
+      typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+      for (int mf = 0; mf < MF; ++mf) {
+        const int r = mf * 16 + li;
+#pragma unroll
+        for (int nf = 0; nf < NF; ++nf) {
+          bf16x4 o;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) o[q] = (__bf16)acc[nf][mf][q];
+          *(bf16x4 LLMMM_LDS*)(stg + r * RS16 + nf * 32 + 8 * g) = o;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < (WM * CH16) / 64; ++j) {
+        const int   idx = j * 64 + lane, r = idx / CH16, c = idx - r * CH16;
+        const i32x4 v   = *(const i32x4 LLMMM_LDS*)(stg + r * RS16 + c * 16);
+        *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 8) = v;
+      }
+    }
+    else {
+      // fp32 planes / fp32 output, or hidden = T(C + residual)
+#pragma unroll
+      for (int mf = 0; mf < MF; ++mf) {
+#pragma unroll
+        for (int nf = 0; nf < NF; ++nf) *(f32x4 LLMMM_LDS*)(stg + li * RS32 + nf * 64 + 16 * g) = acc[nf][mf];
+#pragma unroll
+        for (int j = 0; j < (16 * CH32) / 64; ++j) {
+          const int    idx = j * 64 + lane, r = idx / CH32, c = idx - r * CH32;
+          const f32x4  v   = *(const f32x4 LLMMM_LDS*)(stg + r * RS32 + c * 16);
+          const size_t at  = (size_t)(row0 + 16 * mf + r) * N + col0 + c * 4;
+          if constexpr (OUT == OUT_F32)
+            *(f32x4*)((float*)Cv + (size_t)sp * M * N + at) = v;
+          else {
+            typedef typename std::conditional<OUT == OUT_ADD_F32, float, typename std::conditional<OUT == OUT_ADD_BF16, __bf16, _Float16>::type>::type T;
+            store_row4<T>((T*)Cv + at, v + load_row4<T>((const T*)op.residual + at));
+          }
+        }
+      }
+    }
+  }
+  else if constexpr (OUT == OUT_F32) {
     float* C = (float*)Cv + (size_t)sp * M * N;
 #pragma unroll
     for (int mf = 0; mf < MF; ++mf) {  // 16 rows x 512 B per round
@@ -865,6 +941,12 @@ static hipError_t dispatch_fp8(int tile, const void* A, const float* As, const v
     case LLMMM_TILE_128x256: return launch_fp8<128, 256, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, op, stream);
     case LLMMM_TILE_256x128: return launch_fp8<256, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, op, stream);
     case LLMMM_TILE_128x128: return launch_fp8<128, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, op, stream);
+    case LLMMM_TILE_128x160:
+      // no 1x128-grouped epilogue: fp32 (also the planes of a split run), bf16 and residual-add outputs only
+      if constexpr (OUT == OUT_F32 || OUT == OUT_BF16 || OUT == OUT_ADD_F32 || OUT == OUT_ADD_BF16 || OUT == OUT_ADD_F16)
+        return launch_fp8<128, 160, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, op, stream);
+      else
+        return hipErrorInvalidValue;
     default: return hipErrorInvalidValue;
   }
 }
