@@ -78,6 +78,56 @@ def _events_ms(fn, steps, warmup, graph=False):
     return e0.elapsed_time(e1) / steps, wall_ms / steps
 
 
+def sample_clock_power(step, seconds=1.2):
+    """Shader clock and socket power while `step` runs back to back for `seconds` (outside any timed region): medians of
+    the driver's sysfs readings (pp_dpm_sclk's active level, hwmon power1_input), None where the files cannot be read.
+    The published MFMA peaks are quoted at 2400 MHz; at the board's power limit a GEMM runs below that clock."""
+    import glob
+    import threading
+    import time
+
+    def read():
+        mhz = watts = None
+        for path in glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"):
+            try:
+                for ln in open(path).read().splitlines():
+                    if "*" in ln:
+                        mhz = float(ln.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+            except (OSError, ValueError, IndexError):
+                pass
+        for path in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") + glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average"):
+            try:
+                watts = int(open(path).read()) / 1e6
+                break
+            except (OSError, ValueError):
+                pass
+        return mhz, watts
+
+    samples, stop = [], threading.Event()
+
+    def poll():
+        while not stop.is_set():
+            samples.append(read())
+            time.sleep(0.1)
+
+    for _ in range(50):
+        step()
+    torch.cuda.synchronize()
+    th = threading.Thread(target=poll)
+    t0 = time.time()
+    th.start()
+    while time.time() - t0 < seconds:
+        for _ in range(100):
+            step()
+        torch.cuda.synchronize()
+    stop.set()
+    th.join()
+    samples = samples[len(samples) // 3:]  # the clock settles within the first few hundred milliseconds
+    mhz = sorted(x[0] for x in samples if x[0] is not None)
+    watts = sorted(x[1] for x in samples if x[1] is not None)
+    return {"sclk_mhz": mhz[len(mhz) // 2] if mhz else None, "power_w": watts[len(watts) // 2] if watts else None, "samples": len(samples)}
+
+
 def fp16_inputs(M, N, K, dtype=torch.float16, seed=2):
     g = torch.Generator(device="cuda").manual_seed(seed)
     A = torch.randn((M, K), generator=g, device="cuda", dtype=torch.float32).to(dtype)
@@ -103,7 +153,7 @@ def fp8_inputs(M, N, K, seed=3, copies=1):
     return Aq, As, weights
 
 
-def bench_fp16(M, N, K, steps, warmup, dtype=torch.float16, b_transposed=False):
+def bench_fp16(M, N, K, steps, warmup, dtype=torch.float16, b_transposed=False, clock=False):
     import llmmm_amd
     A, B = fp16_inputs(M, N, K, dtype)
     if b_transposed:
@@ -111,7 +161,10 @@ def bench_fp16(M, N, K, steps, warmup, dtype=torch.float16, b_transposed=False):
     C = torch.empty((M, N), dtype=dtype, device="cuda")
     ms, wall = _events_ms(lambda: llmmm_amd.fp16_gemm(A, B, C, b_transposed=b_transposed), steps, warmup, graph=True)
     flops = 2.0 * M * N * K
-    return {"ms": ms, "wall_ms": wall, "tflops": flops / ms * 1e-9, "bytes": 2.0 * (M * K + K * N + M * N)}, (A, B, C)
+    r = {"ms": ms, "wall_ms": wall, "tflops": flops / ms * 1e-9, "bytes": 2.0 * (M * K + K * N + M * N)}
+    if clock:
+        r["clock"] = sample_clock_power(lambda: llmmm_amd.fp16_gemm(A, B, C, b_transposed=b_transposed))
+    return r, (A, B, C)
 
 
 def fp8_bytes(M, N, K, out):
@@ -127,7 +180,7 @@ def fp8_bytes(M, N, K, out):
     return b
 
 
-def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0, preshuffled=False):
+def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0, preshuffled=False, clock=False):
     """out in {"f32","bf16","fp8q"}.  With rotate_bytes > 0 the launches cycle through enough
     distinct weight copies to exceed that many bytes, so weights stream from HBM, not from cache.
     preshuffled: the weights are permuted once, outside the timed region, into MFMA operand order."""
@@ -165,8 +218,11 @@ def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0, preshuffled=False):
     flops = 2.0 * M * N * K
     nbytes = fp8_bytes(M, N, K, out)
     tile, split = llmmm_amd.query_config(kind, M, N, K)
-    return {"ms": ms, "wall_ms": wall, "tflops": flops / ms * 1e-9, "gbs": nbytes / ms * 1e-6, "bytes": nbytes, "tile": tile,
-            "split_k": split, "weight_copies": copies}
+    r = {"ms": ms, "wall_ms": wall, "tflops": flops / ms * 1e-9, "gbs": nbytes / ms * 1e-6, "bytes": nbytes, "tile": tile,
+         "split_k": split, "weight_copies": copies}
+    if clock:
+        r["clock"] = sample_clock_power(step)
+    return r
 
 
 def bench_mlp_chain(M, steps, warmup, hidden=2560, inter=9728, rotate_bytes=768 << 20):
@@ -453,7 +509,7 @@ def main():
         return
     if w in ("fp16_gemm_4096", "bf16_gemm_4096"):
         dt = torch.float16 if w.startswith("fp16") else torch.bfloat16
-        r, _ = bench_fp16(M, N, K, args.steps, args.warmup, dt)
+        r, _ = bench_fp16(M, N, K, args.steps, args.warmup, dt, clock=True)
         dtype, peak = ("f16" if dt == torch.float16 else "bf16"), PEAK_TFLOPS["f16"]
         roof = {"bound": "mfma", "achieved": r["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": r["tflops"] / peak, "traffic": None,
                 "kernel": "fp16_gemm_kernel<%s,256,256,row-major B>" % dtype}
@@ -462,7 +518,7 @@ def main():
                            "single kernel, no split-K" % dtype, "M": M, "N": N, "K": K}
     elif w in ("fp8_gemm_fused_4096", "fp8_gemm_bf16_4096"):
         out = "fp8q" if "fused" in w else "bf16"
-        r = bench_fp8(M, N, K, out, args.steps, args.warmup)
+        r = bench_fp8(M, N, K, out, args.steps, args.warmup, clock=True)
         dtype, peak = "fp8", PEAK_TFLOPS["fp8"]
         roof = {"bound": "mfma", "achieved": r["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": r["tflops"] / peak, "traffic": None,
                 "kernel": "fp8_gemm_kernel<256,256,%s>" % out}
@@ -538,7 +594,7 @@ def main():
         name, M = mo.group(1), int(mo.group(3))
         N, K = QWEN3_4B[name]
         out = "swiglu" if mo.group(2) else "fp8q"
-        r = bench_fp8(M, N, K, out, args.steps, args.warmup)
+        r = bench_fp8(M, N, K, out, args.steps, args.warmup, clock=True)
         dtype, peak = "fp8", PEAK_TFLOPS["fp8"]
         roof = {"bound": "mfma", "achieved": r["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": r["tflops"] / peak, "traffic": None,
                 "kernel": "fp8_gemm_kernel tile %d split_k %d, output %s" % (r["tile"], r["split_k"], out)}
@@ -550,6 +606,12 @@ def main():
 
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(w)
     roof["algorithmic_bytes"] = r["bytes"]
+    clk = r.get("clock") if isinstance(r, dict) else None
+    if clk and clk.get("sclk_mhz") and roof["bound"] == "mfma":
+        # the published peak is quoted at 2400 MHz; under the board's power limit the kernel runs at a lower clock
+        roof["sclk_mhz"], roof["power_w"] = clk["sclk_mhz"], clk["power_w"]
+        roof["peak_at_clock"] = roof["peak"] * clk["sclk_mhz"] / 2400.0
+        roof["frac_at_clock"] = roof["achieved"] / roof["peak_at_clock"]
     line = {
         "metric": "TFLOPS (% of MI355X FP8/FP16 MFMA peak) at 4096\u00b3; HBM GB/s at M\u226416 decode",
         "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms"],
@@ -642,7 +704,20 @@ def main():
             ms_, _ = _events_ms(lambda: torch.matmul(A, B, out=C), max(10, args.steps // 2), max(3, args.warmup // 2), graph=True)
             comp["torch_matmul_fp16_%d_tflops" % m] = 2.0 * m * n * k / ms_ * 1e-9
             comp["torch_matmul_fp16_%d_us" % m] = ms_ * 1e3
-        comp["note"] = "hipBLASLt via torch.matmul, same inputs and timing method; reported for comparison only"
+        try:
+            # the vendor library's FP8 GEMM (one scale per tensor, bf16 out: a simpler contract than 1x128 / 128x128 blocks)
+            g8 = torch.Generator(device="cuda").manual_seed(7)
+            a8 = torch.randn((4096, 4096), generator=g8, device="cuda").to(torch.float8_e4m3fn)
+            b8 = torch.randn((4096, 4096), generator=g8, device="cuda").to(torch.float8_e4m3fn).t()  # column-major operand
+            one = torch.ones((), device="cuda")
+            ms_, _ = _events_ms(lambda: torch._scaled_mm(a8, b8, scale_a=one, scale_b=one, out_dtype=torch.bfloat16), max(10, args.steps // 2),
+                                max(3, args.warmup // 2), graph=True)
+            comp["torch_scaled_mm_fp8_tensorwise_4096_tflops"] = 2.0 * 4096 ** 3 / ms_ * 1e-9
+            comp["torch_scaled_mm_fp8_tensorwise_4096_us"] = ms_ * 1e3
+        except Exception as e:  # not every build of the vendor library has the kernel
+            comp["torch_scaled_mm_fp8_tensorwise_4096_tflops"] = None
+            comp["torch_scaled_mm_error"] = str(e)[:160]
+        comp["note"] = "hipBLASLt via torch.matmul / torch._scaled_mm, same timing method; reported for comparison only"
         line["comparison"] = comp
     if not args.no_peaks:
         # the same kernel against what this very part sustains: random-operand MFMA rate / streaming read rate
