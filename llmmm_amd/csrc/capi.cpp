@@ -82,19 +82,30 @@ constexpr int MAX_TILE_SPLIT = 8;
 
 bool tile_dims(int tile, int& bm, int& bn);
 
-// Split-K factor for the MFMA tile kernels: only when the tiles alone leave most of the chip
-// idle; about one workgroup per CU, every split at least two slices long.
+// Split-K factor for the MFMA tile kernels: only when the tiles alone leave most of the chip idle -- at most about one
+// workgroup per CU, every split at least two slices long -- and only when the shorter K loop pays for the fp32 planes'
+// round trip and the second launch.  The estimate (microseconds): a 128 x 128 x 128 slice of a lone workgroup takes
+// about 0.5 us (measured: 2048..19456-column outputs at M = 128..512), larger tiles in proportion; the reduce launch
+// costs about 3 us and S planes are written and read at about 4 TB/s.  (M = 256, N = 6144, K = 2560 in 96 tiles:
+// 14.3 us unsplit, 18.9 us in two splits; M = 256, N = 2560, K = 9728 in 40 tiles: 40 us unsplit, 18.6 us in six.)
 int heuristic_tile_split(int tile, int M, int N, int K)
 {
   int bm, bn;
   if (!tile_dims(tile, bm, bn)) return 1;
   const int tiles = (M / bm) * (N / bn), kb = K / 128;
-  int       s     = NUM_CUS / tiles;
-  if (s > kb / 2) s = kb / 2;
-  if (s > MAX_TILE_SPLIT) s = MAX_TILE_SPLIT;
-  return s < 2 ? 1 : s;
+  int       smax  = NUM_CUS / tiles;
+  if (smax > kb / 2) smax = kb / 2;
+  if (smax > MAX_TILE_SPLIT) smax = MAX_TILE_SPLIT;
+  const double t_slice  = 0.5 * (double)bm * bn / (128.0 * 128.0);
+  const double plane_us = (double)M * N * 4.0 * 2.0 / 4.0e6;  // one plane written and read
+  int          best     = 1;
+  double       best_us  = kb * t_slice;
+  for (int s = 2; s <= smax; ++s) {
+    const double us = ((kb + s - 1) / s) * t_slice + 3.0 + s * plane_us;
+    if (us < best_us) best = s, best_us = us;
+  }
+  return best;
 }
-
 bool tile_dims(int tile, int& bm, int& bn)
 {
   switch (tile) {

@@ -26,6 +26,7 @@ static const SkinnyTune kSkinnyTune[] = {
   {1, 2560, 9728, 10},
   {16, 2560, 9728, 10},
   {64, 2560, 9728, 10},
+  {127, 2560, 9728, 12},
   {1, 6144, 2560, 5},
   {16, 6144, 2560, 5},
   {64, 6144, 2560, 5},
@@ -33,6 +34,7 @@ static const SkinnyTune kSkinnyTune[] = {
   {1, 19456, 2560, 1},
   {16, 19456, 2560, 1},
   {64, 19456, 2560, 3},
+  {127, 19456, 2560, 5},
 };
 
 // FP8 MFMA tile kernels (M % 128 == 0).
@@ -44,6 +46,18 @@ static const TileTune kTileTune[] = {
   {2048, 19456, 2560, 0, 1},
   {128, 2560, 9728, 3, 8},
   {2048, 2560, 9728, 3, 1},
+  {256, 6144, 2560, 3, 1},
+  {512, 6144, 2560, 3, 1},
+  {1024, 6144, 2560, 3, 1},
+  {256, 2560, 4096, 3, 4},
+  {512, 2560, 4096, 3, 3},
+  {1024, 2560, 4096, 3, 1},
+  {256, 19456, 2560, 3, 1},
+  {512, 19456, 2560, 0, 1},
+  {1024, 19456, 2560, 3, 1},
+  {256, 2560, 9728, 3, 6},
+  {512, 2560, 9728, 3, 3},
+  {1024, 2560, 9728, 3, 3},
 };
 
 // FP16/BF16 MFMA tile kernels.

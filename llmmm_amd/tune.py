@@ -113,7 +113,7 @@ def render_table(skinny_rows, tile_rows, fp16_rows):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--write", action="store_true", help="rewrite csrc/tune_table.h with the results")
-    ap.add_argument("--m", default="1,16,64,128,2048")
+    ap.add_argument("--m", default="1,16,32,64,96,128,256,512,1024,2048")
     ap.add_argument("--iters", type=int, default=40)
     args = ap.parse_args()
     torch.cuda.set_device(0)
@@ -123,7 +123,9 @@ def main():
         for M in ms:
             tile, split, _ = tune_shape(M, N, K, iters=args.iters)
             if tile == _lib.TILE_SKINNY:
-                skinny_rows.append((M, N, K, split))
+                below = [m for m in ms if m < 128]
+                # the largest tuned M below 128 speaks for every M up to 127
+                skinny_rows.append((127 if below and M == max(below) and M > 64 else M, N, K, split))
             else:
                 tile_rows.append((M, N, K, tile, split))
             torch.cuda.empty_cache()
