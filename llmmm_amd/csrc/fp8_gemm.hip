@@ -95,14 +95,22 @@ __device__ __forceinline__ void fp8_load_f32(float& dst, const void* sbase, unsi
 // are then 8*NW*K bytes apart as well, so only the per-lane offset (16 * lane instead of
 // row * K + chunk * 16, the wave's own rows folded into the base) and the step from slice to
 // slice (2048 instead of 128 bytes) differ between the two layouts.
-template <int BM, int BN, int WM, bool BNT, int I>
-__device__ __forceinline__ void fp8_issue_load(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned a_off, unsigned b_off, int K, size_t b_hi, int wave)
+//
+// MT (a last tile row with fewer than BM rows of A): the lanes of load i whose row lies beyond the matrix fetch its
+// last row instead, so the per-lane offset differs from load to load -- a_tail[i], relative to the tile's first row.
+template <int BM, int BN, int WM, bool BNT, int I, bool MT = false>
+__device__ __forceinline__ void fp8_issue_load(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned a_off, unsigned b_off, int K, size_t b_hi, int wave,
+                                               const unsigned* a_tail = nullptr)
 {
   typedef Fp8Tile<BM, BN, WM> TC;
   // b_hi: extra byte offset of the tile's upper half of weight rows (0 unless the two halves come from different row ranges)
   const size_t b_skip = I - TC::A_LOADS >= TC::B_LOADS / 2 ? b_hi : 0;
-  if constexpr (I < TC::A_LOADS)
-    fp8_load_lds_16B(Ag + (size_t)(8 * TC::NW * I) * K, a_off, lds_stage + (wave + I * TC::NW) * 1024);
+  if constexpr (I < TC::A_LOADS) {
+    if constexpr (MT)
+      fp8_load_lds_16B(Ag, a_tail[I], lds_stage + (wave + I * TC::NW) * 1024);
+    else
+      fp8_load_lds_16B(Ag + (size_t)(8 * TC::NW * I) * K, a_off, lds_stage + (wave + I * TC::NW) * 1024);
+  }
   else if constexpr (I < TC::A_LOADS + TC::B_LOADS) {
     if constexpr (BNT)
       fp8_load_lds_16B_nt(Bg + (size_t)(8 * TC::NW * (I - TC::A_LOADS)) * K + b_skip, b_off, lds_stage + TC::A_BYTES + (wave + (I - TC::A_LOADS) * TC::NW) * 1024);
@@ -110,12 +118,13 @@ __device__ __forceinline__ void fp8_issue_load(unsigned lds_stage, const uint8_t
       fp8_load_lds_16B(Bg + (size_t)(8 * TC::NW * (I - TC::A_LOADS)) * K + b_skip, b_off, lds_stage + TC::A_BYTES + (wave + (I - TC::A_LOADS) * TC::NW) * 1024);
   }
 }
-template <int BM, int BN, int WM, bool BNT, int FIRST, int COUNT>
-__device__ __forceinline__ void fp8_issue_loads(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned a_off, unsigned b_off, int K, size_t b_hi, int wave)
+template <int BM, int BN, int WM, bool BNT, int FIRST, int COUNT, bool MT = false>
+__device__ __forceinline__ void fp8_issue_loads(unsigned lds_stage, const uint8_t* Ag, const uint8_t* Bg, unsigned a_off, unsigned b_off, int K, size_t b_hi, int wave,
+                                                const unsigned* a_tail = nullptr)
 {
   if constexpr (COUNT > 0) {
-    fp8_issue_load<BM, BN, WM, BNT, FIRST>(lds_stage, Ag, Bg, a_off, b_off, K, b_hi, wave);
-    fp8_issue_loads<BM, BN, WM, BNT, FIRST + 1, COUNT - 1>(lds_stage, Ag, Bg, a_off, b_off, K, b_hi, wave);
+    fp8_issue_load<BM, BN, WM, BNT, FIRST, MT>(lds_stage, Ag, Bg, a_off, b_off, K, b_hi, wave, a_tail);
+    fp8_issue_loads<BM, BN, WM, BNT, FIRST + 1, COUNT - 1, MT>(lds_stage, Ag, Bg, a_off, b_off, K, b_hi, wave, a_tail);
   }
 }
 // The slice scales of the lane's four 16-row fragments and of the wave's column group.
@@ -171,11 +180,11 @@ __device__ __forceinline__ void fp8_scale_load_lds(const char* lane_ptr, unsigne
 // steps (spread, so that no wave sits in the memory pipeline's issue queue while its matrix
 // work waits, and early enough to land within the slice), its scales during the fifth.
 // 160-column waves (NF = 10): fragments nf < nfb lie in the first weight-scale block and take s, the others s2.
-template <int BM, int BN, int WM, bool BNT, bool LOAD, bool SCALE_LDS = false>
+template <int BM, int BN, int WM, bool BNT, bool LOAD, bool SCALE_LDS = false, bool MT = false>
 __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int a_rd0, int a_rd1, int b_rd0, int b_rd1,
                                                   const float (&s)[WM / 16], f32x4 (&acc)[Fp8Tile<BM, BN, WM>::NF][WM / 16], const Fp8Next& nx, unsigned lane_off,
                                                   unsigned b_lane_off, unsigned row_off, unsigned zero, int K, size_t b_hi, int wave, float (&sa_next)[WM / 16],
-                                                  float& sb_next, const float (&s2)[WM / 16], int nfb, float& sb2_next)
+                                                  float& sb_next, const float (&s2)[WM / 16], int nfb, float& sb2_next, const unsigned* a_tail = nullptr)
 {
   constexpr int MF = WM / 16;
   typedef Fp8Tile<BM, BN, WM> TC;
@@ -195,10 +204,10 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int
     const int cur = nf & 1;
     if (nf + 1 < NF) b[cur ^ 1] = fp8_read_frag(ldsB, b_rd0, b_rd1, (nf + 1) * 2048);
     if constexpr (LOAD) {
-      if (nf == 0) fp8_issue_loads<BM, BN, WM, BNT, 0, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
-      if (nf == 1) fp8_issue_loads<BM, BN, WM, BNT, LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
-      if (nf == 2) fp8_issue_loads<BM, BN, WM, BNT, 2 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
-      if (nf == 3) fp8_issue_loads<BM, BN, WM, BNT, 3 * LPG, LPG>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave);
+      if (nf == 0) fp8_issue_loads<BM, BN, WM, BNT, 0, LPG, MT>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave, a_tail);
+      if (nf == 1) fp8_issue_loads<BM, BN, WM, BNT, LPG, LPG, MT>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave, a_tail);
+      if (nf == 2) fp8_issue_loads<BM, BN, WM, BNT, 2 * LPG, LPG, MT>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave, a_tail);
+      if (nf == 3) fp8_issue_loads<BM, BN, WM, BNT, 3 * LPG, LPG, MT>(nx.lds_stage, nx.Ag, nx.Bg, lane_off, b_lane_off, K, b_hi, wave, a_tail);
       if (nf == 4) {
         if constexpr (SCALE_LDS)
           fp8_scale_load_lds(nx.sc_ptr, nx.lds_stage + TC::STAGE + wave * 256);
@@ -389,6 +398,10 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   // scales travelling with the stage.  (With two workgroups per CU the two-stage form is faster: 29 vs 38 us on
   // 2048 x 2560 x 4096 in 128 x 128 tiles.)
   constexpr bool DEEP    = (BMODE & 4) != 0 && WM == 32;
+  // BMODE bit 3 (MT, deep 128 x 128 tiles with the fp32 / bf16 / fp8 outputs only): M is not a multiple of BM; the rows
+  // of the last tile row beyond the matrix are computed from copies of its last row and never stored.
+  constexpr bool MT      = (BMODE & 8) != 0;
+  static_assert(!MT || (DEEP && BM == 128 && BN == 128 && (OUT == OUT_F32 || OUT == OUT_BF16 || OUT == OUT_FP8Q)), "row tails: deep 128 x 128 tiles only");
   constexpr int  STAGE_D = TC::STAGE + TC::NW * 256;                 // operands + 256 bytes of scales per wave
   constexpr int  NST     = !DEEP ? 2 : (4 * STAGE_D <= 160 * 1024 ? 4 : 3);
   __shared__ __attribute__((aligned(1024))) char lds[DEEP ? NST * STAGE_D : 2 * TC::STAGE];
@@ -454,17 +467,20 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
 
   if constexpr (DEEP) {
     constexpr int PER = TC::A_LOADS + TC::B_LOADS + 1;  // vector-memory loads of a wave per slice
+    unsigned a_tail[TC::A_LOADS];  // MT: per-load offsets with the row clamped to the matrix
+#pragma unroll
+    for (int i = 0; i < TC::A_LOADS; ++i) a_tail[i] = MT ? (unsigned)(min(lp.row + 8 * TC::NW * i, M - 1 - m0) * K + lp.chunk * 16) : 0u;
     static_assert((NST - 2) * PER < 64, "vmcnt is a 6-bit counter");
     // this lane's scale source: a row scale (stride M floats per slice) or the column-group scale (stride 1)
     const bool     row_lane = lane < WM;
-    const char*    sc_ptr   = row_lane ? (const char*)(Asl + (m0 + wm * WM + lane)) : (const char*)(TWO && lane >= 48 ? Bsp2 : Bsp);
+    const char*    sc_ptr   = row_lane ? (const char*)(Asl + (MT ? min(m0 + wm * WM + lane, M - 1) : m0 + wm * WM + lane)) : (const char*)(TWO && lane >= 48 ? Bsp2 : Bsp);
     const unsigned sc_step  = row_lane ? (unsigned)M * 4u : 4u;
     // prologue: slices 0 .. NST-2 (a K range shorter than that repeats its last slice into the spare stages)
 #pragma unroll
     for (int u = 0; u < NST - 1; ++u) {
       const int kk = min(u, KBL - 1);
-      fp8_issue_loads<BM, BN, WM, BNT, 0, TC::A_LOADS + TC::B_LOADS>(lds0 + u * STAGE_D, Ag + (size_t)kk * 128, Bg + (size_t)kk * B_KSTEP, lane_off,
-                                                                     b_lane_off, K, b_hi, wave);
+      fp8_issue_loads<BM, BN, WM, BNT, 0, TC::A_LOADS + TC::B_LOADS, MT>(lds0 + u * STAGE_D, Ag + (size_t)kk * 128, Bg + (size_t)kk * B_KSTEP, lane_off,
+                                                                         b_lane_off, K, b_hi, wave, a_tail);
       fp8_scale_load_lds(sc_ptr + (size_t)kk * sc_step, lds0 + u * STAGE_D + TC::STAGE + wave * 256);
     }
     const char* sc_next = sc_ptr + (size_t)(NST - 1) * sc_step;
@@ -489,8 +505,8 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
     nx.Bs_elem   = nullptr;                                                                                                       \
     nx.Bs_elem2  = nullptr;                                                                                                       \
     nx.sc_ptr    = sc_next;                                                                                                       \
-    fp8_compute_stage<BM, BN, WM, BNT, LOAD, true>(s0 + cur, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, b_lane_off, row_off, zero, K, b_hi, \
-                                                   wave, sa_next, sb_next, s2, nfb, sb2_next);                                    \
+    fp8_compute_stage<BM, BN, WM, BNT, LOAD, true, MT>(s0 + cur, a_rd0, a_rd1, b_rd0, b_rd1, s, acc, nx, lane_off, b_lane_off, row_off, zero, K, \
+                                                       b_hi, wave, sa_next, sb_next, s2, nfb, sb2_next, a_tail);                  \
     cur = cur + STAGE_D == NST * STAGE_D ? 0 : cur + STAGE_D;                                                                     \
   }
     int kc = 0;
@@ -613,7 +629,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
       for (int j = 0; j < 8; ++j) {
         const int   r = 2 * j + (lane >> 5), c = lane & 31;
         const f32x4 v = *(const f32x4 LLMMM_LDS*)(stg + r * 512 + ((c ^ ((r & 7) << 1)) << 4));
-        *(f32x4*)(C + (size_t)(row0 + 16 * mf + r) * N + col0 + c * 4) = v;
+        if (!MT || row0 + 16 * mf + r < M) *(f32x4*)(C + (size_t)(row0 + 16 * mf + r) * N + col0 + c * 4) = v;
       }
     }
   }
@@ -653,7 +669,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
     for (int j = 0; j < WM / 4; ++j) {
       const int   r = 4 * j + (lane >> 4), c = lane & 15;
       const i32x4 v = *(const i32x4 LLMMM_LDS*)(stg + r * 256 + ((c ^ (r & 15)) << 4));
-      *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 8) = v;
+      if (!MT || row0 + r < M) *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 8) = v;
     }
   }
   else if constexpr (OUT == OUT_SWIGLU) {
@@ -701,13 +717,13 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
         const f32x4 v = acc[nf][mf];
         *(uint32_t LLMMM_LDS*)(stg + r * 128 + ((nf ^ ((r >> 1) & 7)) << 4) + 4 * g) = pack_e4m3x4_in_range(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
       }
-      if (g == 0) Cs[(size_t)((n0 >> 7) + wn) * M + row0 + r] = scale;
+      if (g == 0 && (!MT || row0 + r < M)) Cs[(size_t)((n0 >> 7) + wn) * M + row0 + r] = scale;
     }
 #pragma unroll
     for (int j = 0; j < WM / 8; ++j) {
       const int   r = 8 * j + (lane >> 3), c = lane & 7;
       const i32x4 v = *(const i32x4 LLMMM_LDS*)(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
-      *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 16) = v;
+      if (!MT || row0 + r < M) *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 16) = v;
     }
   }
 }
@@ -880,6 +896,12 @@ static hipError_t launch_reduce(const float* planes, int S, void* C, float* Cs, 
 template <int BM, int BN, int WM, int OUT>
 static auto pick_kernel(int bmode) -> decltype(&fp8_gemm_kernel<BM, BN, WM, OUT, 0>)
 {
+  if (bmode & 8) {  // a row tail: deep 128 x 128 tiles with the fp32 / bf16 / fp8 outputs
+    if constexpr (BM == 128 && BN == 128 && WM == 32 && (OUT == OUT_F32 || OUT == OUT_BF16 || OUT == OUT_FP8Q))
+      return (bmode & 1) ? fp8_gemm_kernel<BM, BN, WM, OUT, 15> : fp8_gemm_kernel<BM, BN, WM, OUT, 14>;
+    else
+      return nullptr;
+  }
   if constexpr (WM != 32) bmode &= 3;  // only the 32-row-wave tiles have a deep form
   switch (bmode) {
     case 1: return fp8_gemm_kernel<BM, BN, WM, OUT, 1>;
@@ -898,16 +920,18 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
                              int K, int S, float* planes, bool bpre, const Fp8HeadOp& op, hipStream_t stream)
 {
   typedef Fp8Tile<BM, BN, WM> TC;
-  const int tiles_m = M / BM, tiles_n = N / BN;
+  const int tiles_m = (M + BM - 1) / BM, tiles_n = N / BN;
+  if (M % BM != 0 && tiles_m != 1) return hipErrorInvalidValue;  // a row tail: M < BM only (one tile row, the deep form)
   // one tile row: the weights are read once (streamed, deep); at most one workgroup per CU: deep
   const bool one_per_cu = (long)tiles_m * tiles_n * (S < 1 ? 1 : S) <= 256;
-  const int  bmode      = (bpre ? 1 : 0) | (tiles_m == 1 ? 2 | 4 : 0) | (one_per_cu ? 4 : 0);
+  const int  bmode      = (bpre ? 1 : 0) | (tiles_m == 1 ? 2 | 4 : 0) | (one_per_cu ? 4 : 0) | (M % BM != 0 ? 8 : 0);
   if (S <= 1 && planes == nullptr) {
     if constexpr (OUT == OUT_SWIGLU && BN != 256) {
       return hipErrorInvalidValue;  // unsplit SwiGLU needs a 256-wide tile (the host picks one)
     }
     else {
       const auto kernel = pick_kernel<BM, BN, WM, OUT>(bmode);
+      if (kernel == nullptr) return hipErrorInvalidValue;
       hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs,
                          M, N, K, tiles_m, tiles_n, op);
       return hipGetLastError();
@@ -921,6 +945,7 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
   else {
     if (S < 1) S = 1;
     const auto kernel = pick_kernel<BM, BN, WM, OUT_F32>(bmode);
+    if (kernel == nullptr) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, S), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs,
                        (void*)planes, (float*)nullptr, M, N, K, tiles_m, tiles_n, op);
     hipError_t e = hipGetLastError();

@@ -1,0 +1,85 @@
+"""A single tile row of fewer than 128 rows in the 128 x 128 FP8 tiles (64 < M < 128 on shapes whose M = 128 the tune
+table gives to those tiles; any M < 128 when the tile is named).  Rows beyond M are computed from copies of the last
+row and never stored: the result must equal the weight-streaming kernel's bit for bit (both add the same 128-K slices
+in the same order) and nothing may be written behind row M - 1 (guard rows of NaN behind every output).  A sits in front of
+rows of NaN codes: a lane that fetched a row other than its own (clamped) one for a stored output would show up as NaN."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_fp8_gemm_close
+
+pytestmark = pytest.mark.gpu
+T128, SKINNY = 3, 8
+
+
+def _inputs(oracle, M, N, K, seed=0):
+    rng = np.random.default_rng(seed + M + N + K)
+    X = rng.standard_normal((M, K)).astype(np.float32)
+    X[:, ::37] *= 11
+    W = (rng.standard_normal((N, K)) * 0.03).astype(np.float32)
+    Aq, As = oracle.quant_fp8(X, 1, True)
+    Bq, Bs = oracle.quant_fp8(W, 128, False)
+    return Aq, As, Bq, Bs
+
+
+@pytest.mark.parametrize("M,N,K,split,pre", [(96, 256, 512, 1, False), (65, 1280, 1024, 1, True), (127, 512, 2560, 4, False), (1, 256, 256, 1, False),
+                                             (100, 2560, 1280, 2, True), (17, 128, 128, 1, False), (112, 19456, 256, 1, False)])
+def test_tail_rows_match_the_weight_streaming_kernel(lib, oracle, M, N, K, split, pre):
+    Aq, As, Bq, Bs = _inputs(oracle, M, N, K)
+    # A sits in front of rows that decode to NaN (0x7f is the e4m3 NaN code)
+    dA_all = torch.full((M + 8, K), 0x7F, dtype=torch.uint8, device="cuda")
+    dA_all[:M] = torch.from_numpy(Aq).cuda()
+    dA = dA_all[:M]
+    dAs = torch.from_numpy(As).cuda()
+    dB, dBs = torch.from_numpy(Bq).cuda(), torch.from_numpy(Bs).cuda()
+    if pre:
+        dB = lib.preshuffle_weight(dB)
+    ws = torch.full((8 * M * N * 4,), 0xFF, dtype=torch.uint8, device="cuda")
+    kw = dict(workspace=ws, split_k=split, b_preshuffled=pre)
+    guard = 4
+    C = torch.full((M + guard, N), float("nan"), device="cuda")
+    Cr = torch.empty((M, N), device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dA, dAs, dB, dBs, C[:M], M, N, K, tile=T128, **kw)
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dA, dAs, dB, dBs, Cr, M, N, K, tile=SKINNY, **kw)
+    Y = torch.full((M + guard, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(dA, dAs, dB, dBs, Y[:M], M, N, K, tile=T128, **kw)
+    Q = torch.full((M + guard, N), 0x7F, dtype=torch.uint8, device="cuda")
+    Qs = torch.full((N // 128, M), float("nan"), device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(dA, dAs, dB, dBs, Q[:M], Qs, M, N, K, tile=T128, **kw)
+    Qr = torch.empty((M, N), dtype=torch.uint8, device="cuda")
+    Qsr = torch.empty((N // 128, M), device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(dA, dAs, dB, dBs, Qr, Qsr, M, N, K, tile=SKINNY, **kw)
+    torch.cuda.synchronize()
+    assert_fp8_gemm_close(C[:M].cpu().numpy(), oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128), "row tail")
+    assert torch.equal(C[:M].view(torch.int32), Cr.view(torch.int32)), "differs from the weight-streaming kernel"
+    assert torch.isnan(C[M:]).all() and torch.isnan(Y[M:].float()).all() and (Q[M:] == 0x7F).all(), "rows behind M were written"
+    assert torch.equal(Y[:M].view(torch.int16), C[:M].to(torch.bfloat16).view(torch.int16)), "bf16 != RNE(fp32)"
+    assert torch.equal(Q[:M], Qr) and torch.equal(Qs.view(torch.int32), Qsr.view(torch.int32)), "fused quantisation differs"
+
+
+def test_table_routes_64_to_127_rows_like_128(lib):
+    from llmmm_amd import _lib
+    # gate_up and down of Qwen3-4B: M = 128 runs in 128 x 128 tiles, and so do 65 .. 127 rows
+    for n, k in ((19456, 2560), (2560, 9728)):
+        want = lib.query_config(_lib.OUT_FP8Q, 128, n, k)
+        assert want[0] == T128
+        for m in (65, 96, 127):
+            assert lib.query_config(_lib.OUT_FP8Q, m, n, k) == want
+        assert lib.query_config(_lib.OUT_FP8Q, 64, n, k)[0] == SKINNY
+
+
+def test_swiglu_and_planes_entry_points_on_tail_rows(lib, oracle):
+    """gate_up at M = 96 goes through the tiles' fp32 plane and the reduce kernel's SwiGLU; the result must equal M = 16-row
+    blocks of the weight-streaming kernel (same planes, same reduce)."""
+    M, N, K = 96, 19456, 2560
+    Aq, As, Bq, Bs = _inputs(oracle, M, N, K, 3)
+    dA, dAs, dB, dBs = (torch.from_numpy(a).cuda() for a in (Aq, As, Bq, Bs))
+    ws = torch.empty(8 * M * N * 4, dtype=torch.uint8, device="cuda")
+    H = torch.empty((M, N // 2), dtype=torch.uint8, device="cuda")
+    Hs = torch.empty((N // 256, M), device="cuda")
+    Hr, Hsr = torch.empty_like(H), torch.empty_like(Hs)
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(dA, dAs, dB, dBs, H, Hs, M, N, K, workspace=ws)
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(dA, dAs, dB, dBs, Hr, Hsr, M, N, K, workspace=ws, tile=SKINNY, split_k=1)
+    torch.cuda.synchronize()
+    assert torch.equal(H, Hr) and torch.equal(Hs.view(torch.int32), Hsr.view(torch.int32))
