@@ -985,8 +985,6 @@ static hipError_t dispatch_fp8(int tile, const void* A, const float* As, const v
 {
   // the 256 x 256 tile uses eight 64-row waves; the smaller tiles 32-row waves (twice the waves per SIMD)
   switch (tile) {
-    // (with the head op the 256 x 256 tile -- 128 accumulator registers per lane -- spills a dozen registers, all of them
-    // inside the epilogue, after the last MFMA: once per launch and lane, not per slice)
     case LLMMM_TILE_256x256: return launch_fp8<256, 256, 64, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, op, stream);
     case LLMMM_TILE_128x256: return launch_fp8<128, 256, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, op, stream);
     case LLMMM_TILE_256x128: return launch_fp8<256, 128, 32, OUT>(A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, op, stream);
