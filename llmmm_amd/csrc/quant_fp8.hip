@@ -2,7 +2,8 @@
 //
 // Replaces fp8_blockwise_symmetric_quantization<QUANT_M, 128, SCALE_TRANSPOSE>
 // (reference: examples/005.fp8.mm.cu:439-563): per block amax -> s = amax / 448.f ->
-// q = e4m3(s ? x / s : 0) with an IEEE-correct fp32 division, round-to-nearest-even and
+// q = e4m3(s ? x / s : 0), the code of the IEEE-correct fp32 quotient (q_pack_quotients_e4m3x4 below
+// finds it without dividing wherever the rounding is not in doubt), round-to-nearest-even and
 // saturation to +-448; a block of zeros gives s = 0 and q = 0.  Scale layouts:
 //   QUANT_M == 1:   transposed s[(n/128)*M + m]      plain s[m*ceil(N/128) + n/128]
 //   QUANT_M == 128: transposed s[(n/128)*M + m/128]  plain s[(m/128)*ceil(N/128) + n/128]
@@ -24,6 +25,29 @@ __device__ __forceinline__ uint32_t q_pack_e4m3x4(float a, float b, float c, flo
   int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
   v     = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
   return (uint32_t)v;
+}
+
+// e4m3 codes of v[0..3] / s (s != 0, |v[e]| <= 448 s up to rounding), equal bit for bit to converting the correctly
+// rounded fp32 quotients -- without dividing, almost always.  An IEEE fp32 division costs about ten vector instructions
+// per element and made the quantisers ALU-bound (the same element rate from bf16 and from fp32 inputs).  Instead:
+// t = v * rcp(s) lies within 2^-22 (relative) of the exact quotient and of its fp32 rounding; if t (1 - 2^-21) and
+// t (1 + 2^-21), which bracket both, convert to the same code, then -- the conversion being monotone -- so does the
+// correctly rounded quotient.  Otherwise (a quotient within 2^-20 of a rounding boundary of the 3-bit mantissa: about
+// 3 in 10^5 elements), or when s is so small or large that rcp(s) leaves the normal range, the lane divides.
+// No clamp on the fast path: |t| < 448 (1 + 2^-20), and everything below 464 converts to 448.
+__device__ __forceinline__ uint32_t q_pack_quotients_e4m3x4(f32x4 v, float s)
+{
+  const float y  = __builtin_amdgcn_rcpf(s);
+  const float dn = 1.0f - 0x1p-21f, up = 1.0f + 0x1p-21f;
+  f32x4       t;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) t[e] = v[e] * y;
+  int lo = __builtin_amdgcn_cvt_pk_fp8_f32(t[0] * dn, t[1] * dn, 0, false);
+  lo     = __builtin_amdgcn_cvt_pk_fp8_f32(t[2] * dn, t[3] * dn, lo, true);
+  int hi = __builtin_amdgcn_cvt_pk_fp8_f32(t[0] * up, t[1] * up, 0, false);
+  hi     = __builtin_amdgcn_cvt_pk_fp8_f32(t[2] * up, t[3] * up, hi, true);
+  if (lo == hi && s >= 0x1p-100f && s <= 0x1p100f) return (uint32_t)lo;
+  return q_pack_e4m3x4(v[0] / s, v[1] / s, v[2] / s, v[3] / s);
 }
 
 __device__ __forceinline__ float amax4(float m, f32x4 v)
@@ -57,7 +81,7 @@ __global__ void __launch_bounds__(256) quant_1x128_kernel(const float* __restric
     a       = wave_xor_max(a, 16);
     const float s = a / 448.f;
     uint32_t    c = 0;
-    if (s != 0.f) c = q_pack_e4m3x4(v[0] / s, v[1] / s, v[2] / s, v[3] / s);
+    if (s != 0.f) c = q_pack_quotients_e4m3x4(v, s);
     if (live) *(uint32_t*)(q + (size_t)m * N + n) = c;
     if (l32 == 0) {
       if (TRANSPOSE)
@@ -105,7 +129,7 @@ __global__ void __launch_bounds__(256) quant_128x128_kernel(const float* __restr
   for (int r = 0; r < 16; ++r) {
     const int m = mb * 128 + r * 8 + sub;
     uint32_t  c = 0;
-    if (s != 0.f) c = q_pack_e4m3x4(v[r][0] / s, v[r][1] / s, v[r][2] / s, v[r][3] / s);
+    if (s != 0.f) c = q_pack_quotients_e4m3x4(v[r], s);
     if (live && m < M) *(uint32_t*)(q + (size_t)m * N + n) = c;
   }
   if (tid == 0) {
@@ -150,7 +174,7 @@ __device__ __forceinline__ void rmsnorm_quant_chunk(f32x4 v, float r, const floa
   a       = wave_xor_max(a, 16);
   const float s  = a / 448.f;
   uint32_t    cd = 0;
-  if (s != 0.f) cd = q_pack_e4m3x4(y[0] / s, y[1] / s, y[2] / s, y[3] / s);
+  if (s != 0.f) cd = q_pack_quotients_e4m3x4(y, s);
   if (live) {
     *(uint32_t*)(q + (size_t)m * K + 4 * c) = cd;
     if ((lane & 31) == 0) scale[(size_t)(c >> 5) * M + m] = s;
@@ -248,7 +272,7 @@ __global__ void __launch_bounds__(256) rmsnorm_quant_row_kernel(const IN_T* __re
     const int   c  = t + 256 * i;
     const float sc = amax[i] / 448.f;
     uint32_t    cd = 0;
-    if (sc != 0.f) cd = q_pack_e4m3x4(held[i][0] / sc, held[i][1] / sc, held[i][2] / sc, held[i][3] / sc);
+    if (sc != 0.f) cd = q_pack_quotients_e4m3x4(held[i], sc);
     if (c < chunks) {
       *(uint32_t*)(q + (size_t)m * K + 4 * c) = cd;
       if ((t & 31) == 0) scale[(size_t)(c >> 5) * M + m] = sc;
@@ -349,7 +373,7 @@ __global__ void __launch_bounds__(256) planes_add_rmsnorm_quant_kernel(const flo
     const int   c  = t + 256 * i;
     const float sc = amax[i] / 448.f;
     uint32_t    cd = 0;
-    if (sc != 0.f) cd = q_pack_e4m3x4(held[i][0] / sc, held[i][1] / sc, held[i][2] / sc, held[i][3] / sc);
+    if (sc != 0.f) cd = q_pack_quotients_e4m3x4(held[i], sc);
     if (c < chunks) {
       *(uint32_t*)(q + (size_t)m * N + 4 * c) = cd;
       if ((t & 31) == 0) scale[(size_t)(c >> 5) * M + m] = sc;

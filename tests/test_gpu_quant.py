@@ -75,3 +75,50 @@ def test_full_size_activation_and_weight(lib, oracle):
     # size-independent invariant over the whole matrix: |q| <= 448 and every 1x128 block reaches +-448
     dec = q.view(torch.float8_e4m3fn).float().abs().reshape(4096, 32, 128).amax(-1)
     assert (dec == 448).all()
+
+
+def test_quotients_on_rounding_boundaries(lib, oracle):
+    """The quantiser decides most codes from x * rcp(s) and divides only where that cannot settle the rounding.  Rows
+    built to sit on the boundaries: quotients that are exact ties of the 3-bit mantissa (power-of-two scales, so the tie
+    survives the division), and, for arbitrary scales, values up to three fp32 steps either side of every tie."""
+    vals = oracle.e4m3_decode(np.arange(0, 0x7F, dtype=np.uint8)).astype(np.float64)  # every finite code >= 0
+    mids = ((vals[:-1] + vals[1:]) / 2).astype(np.float32)                             # 126 ties, exact in fp32
+    rng = np.random.default_rng(11)
+    rows = []
+
+    def row(v, amax):
+        r = np.zeros(384, np.float32)
+        for gi, sign in enumerate((1.0, -1.0, None)):
+            sg = np.float32(sign) if sign else (rng.integers(0, 2, 126) * 2 - 1).astype(np.float32)
+            r[gi * 128] = amax                      # every 128-column group has the same amax, hence the same scale
+            r[gi * 128 + 1:gi * 128 + 127] = v * sg
+        rows.append(r)
+
+    for k in (-20, -3, 0, 5, 30):                   # s = 2^k exactly
+        row(mids * np.float32(2.0 ** k), np.float32(448.0 * 2.0 ** k))
+    for amax in (300.0, 1.0, 7.3e-4, 5.1e6, 447.99):
+        amax = np.float32(amax)
+        s = np.float32(amax / np.float32(448.0))
+        for step in range(-3, 4):
+            x = (mids.astype(np.float64) * float(s)).astype(np.float32)
+            for _ in range(abs(step)):
+                x = np.nextafter(x, np.float32(np.inf if step > 0 else -np.inf), dtype=np.float32)
+            x[np.abs(x) > amax] = 0
+            row(x, amax)
+    x = np.stack(rows)
+    rq, rs = oracle.quant_fp8(x, 1, True)
+    q, s = _run(lib, x, 1, True, rs.shape)
+    assert (s.view(np.uint32) == rs.view(np.uint32)).all()
+    assert (q == rq).all(), "codes differ at %s" % (np.argwhere(q != rq)[:5],)
+    assert len(np.unique(rq)) > 200                 # the rows do exercise the whole code range
+    q128, s128 = _run(lib, x, 128, False, oracle.quant_fp8(x, 128, False)[1].shape)
+    rq128, rs128 = oracle.quant_fp8(x, 128, False)
+    assert (q128 == rq128).all() and (s128.view(np.uint32) == rs128.view(np.uint32)).all()
+    # the same rows through the RMSNorm-fused quantiser (both of its kernels: K = 384 and a long row)
+    for reps in (1, 32):
+        xx = np.tile(x, (1, reps))
+        w = rng.uniform(0.5, 2.0, xx.shape[1]).astype(np.float32)
+        rq2, rs2 = oracle.rmsnorm_quant(xx, w, 1e-6)
+        q2, s2 = lib.rmsnorm_quantize_activation(torch.from_numpy(xx).cuda(), torch.from_numpy(w).cuda(), 1e-6)
+        torch.cuda.synchronize()
+        assert (q2.cpu().numpy() == rq2).all() and (s2.cpu().numpy().view(np.uint32) == rs2.view(np.uint32)).all()
