@@ -401,15 +401,27 @@ __device__ __forceinline__ void qk_norm_rope_fragments(f32x4 (&acc)[8][MF], cons
 #undef LLMMM_ROPE_ROTATE
 }
 
+// LDS bytes of one workgroup of fp8_gemm_body<BM, BN, WM, *, BMODE>: two operand stages, or the deep pipeline's three or four
+// stages with 256 bytes of scales per wave each.
+template <int BM, int BN, int WM, int BMODE>
+constexpr int fp8_lds_bytes()
+{
+  typedef Fp8Tile<BM, BN, WM> TC;
+  const bool deep    = (BMODE & 4) != 0 && WM == 32;
+  const int  stage_d = TC::STAGE + TC::NW * 256;
+  return !deep ? 2 * TC::STAGE : (4 * stage_d <= 160 * 1024 ? 4 : 3) * stage_d;
+}
+
 // BMODE bit 0 (BPRE): Bt is the pre-shuffled image of the weights (layout.hip) instead of row-major [N, K].
 // BMODE bit 1 (BNT): the weight loads carry the non-temporal hint (one tile row: every weight byte is read once).
 // BMODE bit 2 (DEEP, 32-row-wave tiles only): the launch has at most one workgroup per CU, which then runs a deeper pipeline.
 template <int BM, int BN, int WM, int OUT, int BMODE>
-__global__ void __launch_bounds__((BM / WM) * (BN / 128) * 64)
-fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
-                const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int tiles_m,
-                int tiles_n, Fp8HeadOp op)
+__device__ __forceinline__ void fp8_gemm_body(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
+                                              const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K,
+                                              int tiles_m, int tiles_n, const Fp8HeadOp& op, char LLMMM_LDS* lds, int tile_index, int n_base)
 {
+  // tile_index: this workgroup's tile among the tiles_m x tiles_n tiles of the column range that starts at n_base (0 and
+  // the whole matrix for the plain kernel; SwiGLU counts n_base in gate columns); lds: the workgroup's operand buffers
   typedef Fp8Tile<BM, BN, WM> TC;
   constexpr int  MF   = TC::MF;
   constexpr int  NF   = TC::NF;
@@ -429,7 +441,7 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   static_assert(!MT || (DEEP && BM == 128 && BN == 128 && (OUT == OUT_F32 || OUT == OUT_BF16 || OUT == OUT_FP8Q)), "row tails: deep 128 x 128 tiles only");
   constexpr int  STAGE_D = TC::STAGE + TC::NW * 256;                 // operands + 256 bytes of scales per wave
   constexpr int  NST     = !DEEP ? 2 : (4 * STAGE_D <= 160 * 1024 ? 4 : 3);
-  __shared__ __attribute__((aligned(1024))) char lds[DEEP ? NST * STAGE_D : 2 * TC::STAGE];
+  static_assert(fp8_lds_bytes<BM, BN, WM, BMODE>() == (DEEP ? NST * STAGE_D : 2 * TC::STAGE), "the kernels size the buffers with fp8_lds_bytes");
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -437,12 +449,12 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
   const int wm   = wave % TC::WAVES_M;
   const int wn   = wave / TC::WAVES_M;
   int       tm, tn;
-  tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+  tile_coords(tile_index, tiles_m, tiles_n, tm, tn);
   // SwiGLU output: the tile's two 128-column halves are the gate columns n0 .. n0+127 and the up columns
   // N/2 + n0 .. of the same 128 output columns, so the weight rows of the upper half start N/2 - 128 rows further on
   constexpr bool SWIGLU = OUT == OUT_SWIGLU;
   static_assert(!SWIGLU || BN == 256, "the SwiGLU epilogue pairs the two 128-column halves of a 256-wide tile");
-  const int    m0   = tm * BM, n0 = SWIGLU ? tn * 128 : tn * BN;
+  const int    m0   = tm * BM, n0 = n_base + (SWIGLU ? tn * 128 : tn * BN);
   const size_t b_hi = SWIGLU ? (size_t)((N >> 1) - 128) * K : 0;
   const int    KB   = K >> 7;
   // split-K: gridDim.y workgroups share a tile, each taking a contiguous run of slices and (the
@@ -719,9 +731,9 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
     uint8_t*  C    = (uint8_t*)Cv;
     const int half = N >> 1;
     if (wn == 0)
-      swiglu_finish<MF, 0, true>(acc, other, xmine, C, Cs + (size_t)tn * M, half, row0, n0, lane);
+      swiglu_finish<MF, 0, true>(acc, other, xmine, C, Cs + (size_t)(n0 >> 7) * M, half, row0, n0, lane);
     else
-      swiglu_finish<MF, MH, false>(acc, other, xmine, C, Cs + (size_t)tn * M, half, row0, n0, lane);
+      swiglu_finish<MF, MH, false>(acc, other, xmine, C, Cs + (size_t)(n0 >> 7) * M, half, row0, n0, lane);
   }
   else {
     uint8_t* C = (uint8_t*)Cv;
@@ -751,6 +763,38 @@ fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, con
       if (!MT || row0 + r < M) *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 16) = v;
     }
   }
+}
+
+template <int BM, int BN, int WM, int OUT, int BMODE>
+__global__ void __launch_bounds__((BM / WM) * (BN / 128) * 64)
+fp8_gemm_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
+                const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int tiles_m,
+                int tiles_n, Fp8HeadOp op)
+{
+  __shared__ __attribute__((aligned(1024))) char lds[fp8_lds_bytes<BM, BN, WM, BMODE>()];
+  fp8_gemm_body<BM, BN, WM, OUT, BMODE>(A, As, Bt, Bs, Cv, Cs, M, N, K, tiles_m, tiles_n, op, (char LLMMM_LDS*)lds, blockIdx.x, 0);
+}
+
+// 256 x 256 tiles leave the last round of the chip partly filled when their number is not a multiple of the 256 CUs
+// (M = 2048, N = 19456: 608 tiles, the third round 96 of them).  This launch gives the columns that fill whole rounds to
+// 256 x 256 tiles and the remaining ones to twice as many 128 x 256 tiles (the same eight waves and K loop, half the
+// rows per wave; same results bit for bit): the last round then runs on up to all CUs for half as long.  Workgroups
+// 0 .. tiles_m_big * cols_big - 1 are the large tiles (dispatched first), the rest the small ones of the column range
+// behind them.
+template <int OUT, int BPRE>
+__global__ void __launch_bounds__(512)
+fp8_gemm_hybrid_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt,
+                       const float* __restrict__ Bs, void* __restrict__ Cv, float* __restrict__ Cs, int M, int N, int K, int tiles_m_big,
+                       int cols_big, int cols_small, Fp8HeadOp op)
+{
+  static_assert(fp8_lds_bytes<128, 256, 32, BPRE>() <= fp8_lds_bytes<256, 256, 64, BPRE>(), "the small tiles fit the large tiles' buffers");
+  __shared__ __attribute__((aligned(1024))) char lds[fp8_lds_bytes<256, 256, 64, BPRE>()];
+  const int n_big = tiles_m_big * cols_big;
+  if ((int)blockIdx.x < n_big)
+    fp8_gemm_body<256, 256, 64, OUT, BPRE>(A, As, Bt, Bs, Cv, Cs, M, N, K, tiles_m_big, cols_big, op, (char LLMMM_LDS*)lds, blockIdx.x, 0);
+  else
+    fp8_gemm_body<128, 256, 32, OUT, BPRE>(A, As, Bt, Bs, Cv, Cs, M, N, K, 2 * tiles_m_big, cols_small, op, (char LLMMM_LDS*)lds,
+                                           (int)blockIdx.x - n_big, cols_big * (OUT == OUT_SWIGLU ? 128 : 256));
 }
 
 // Sum of S planes at one position, added in plane order 0 .. S-1.  W planes are in flight at a time; positions
@@ -955,6 +999,25 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
       return hipErrorInvalidValue;  // unsplit SwiGLU needs a 256-wide tile (the host picks one)
     }
     else {
+      if constexpr (BM == 256 && BN == 256 && (OUT == OUT_F32 || OUT == OUT_BF16 || OUT == OUT_FP8Q || OUT == OUT_SWIGLU)) {
+        // more than one round of the chip with a partly filled last one: whole rounds in 256 x 256 tiles, the remaining
+        // columns in 128 x 256 tiles, if those fit one round (fp8_gemm_hybrid_kernel)
+        const long tiles = (long)tiles_m * tiles_n;
+        const long full  = tiles / 256 * 256;
+        if (tiles > 256 && tiles_m > 1 && full % tiles_m == 0) {
+          const int cols_big = (int)(full / tiles_m), cols_small = tiles_n - cols_big;
+          if (cols_small > 0 && (long)cols_small * tiles_m * 2 <= 256) {
+            const dim3 grid(tiles_m * cols_big + 2 * tiles_m * cols_small);
+            if (bpre)
+              hipLaunchKernelGGL((fp8_gemm_hybrid_kernel<OUT, 1>), grid, dim3(512), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs, M,
+                                 N, K, tiles_m, cols_big, cols_small, op);
+            else
+              hipLaunchKernelGGL((fp8_gemm_hybrid_kernel<OUT, 0>), grid, dim3(512), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs, M,
+                                 N, K, tiles_m, cols_big, cols_small, op);
+            return hipGetLastError();
+          }
+        }
+      }
       const auto kernel = pick_kernel<BM, BN, WM, OUT>(bmode);
       if (kernel == nullptr) return hipErrorInvalidValue;
       hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs,
