@@ -999,7 +999,7 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
       return hipErrorInvalidValue;  // unsplit SwiGLU needs a 256-wide tile (the host picks one)
     }
     else {
-      if constexpr (BM == 256 && BN == 256 && (OUT == OUT_F32 || OUT == OUT_BF16 || OUT == OUT_FP8Q || OUT == OUT_SWIGLU)) {
+      if constexpr (BM == 256 && BN == 256) {
         // more than one round of the chip with a partly filled last one: whole rounds in 256 x 256 tiles, the remaining
         // columns in 128 x 256 tiles, if those fit one round (fp8_gemm_hybrid_kernel)
         const long tiles = (long)tiles_m * tiles_n;

@@ -54,7 +54,7 @@ static const TileTune kTileTune[] = {
   {1024, 2560, 4096, 3, 1},
   {256, 19456, 2560, 3, 1},
   {512, 19456, 2560, 0, 1},
-  {1024, 19456, 2560, 3, 1},
+  {1024, 19456, 2560, 0, 1},
   {256, 2560, 9728, 3, 6},
   {512, 2560, 9728, 3, 3},
   {1024, 2560, 9728, 3, 3},

@@ -61,3 +61,34 @@ def test_equals_the_128x128_tiles(lib, oracle, M, N, K, pre, check_oracle):
     lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(dA, dAs, dB, dBs, H1, G1, M, N, K, tile=T128x256, **kw)
     torch.cuda.synchronize()
     assert torch.equal(H0, H1) and torch.equal(G0.view(torch.int32), G1.view(torch.int32)), "SwiGLU output differs from the 128 x 256 tiles"
+
+
+def test_head_and_residual_epilogues_across_the_seam(lib, oracle):
+    """The QKV + per-head norm + RoPE and the residual-add epilogues in the two-shape launch against the 128 x 128 tiles."""
+    g = lambda a: torch.from_numpy(a).cuda()
+    rng = np.random.default_rng(5)
+    # 16 x 24 = 384 tiles of 256 x 256: 256 in large tiles, the last 8 tile columns (16 of 48 heads) in 128 x 256 tiles
+    M, K, n_q, n_kv = 4096, 256, 32, 8
+    N = (n_q + 2 * n_kv) * 128
+    Aq, As, Bq, Bs = _inputs(oracle, M, N, K, 1)
+    qw, kw = rng.uniform(0.5, 1.5, 128).astype(np.float32), rng.uniform(0.5, 1.5, 128).astype(np.float32)
+    ang = rng.uniform(0, 6.28, (64, 64)).astype(np.float32)
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    pos = rng.integers(0, 64, M).astype(np.int32)
+    args = (g(Aq), g(As), g(Bq), g(Bs), g(qw), g(kw), 1e-6, g(cos), g(sin), g(pos), n_q, n_kv, M, N, K)
+    y0 = lib.fp8_gemm_qkv_rope(*args, tile=T256, split_k=1)
+    y3 = lib.fp8_gemm_qkv_rope(*args, tile=T128, split_k=1)
+    q0, s0 = lib.fp8_gemm_qkv_rope(*args, out_fp8=True, tile=T256, split_k=1)
+    q3, s3 = lib.fp8_gemm_qkv_rope(*args, out_fp8=True, tile=T128, split_k=1)
+    torch.cuda.synchronize()
+    assert torch.equal(y0.view(torch.int16), y3.view(torch.int16)) and torch.equal(q0, q3) and torch.equal(s0.view(torch.int32), s3.view(torch.int32))
+    # 32 x 10 = 320 tiles: 256 + 2 tile columns; hidden = bf16(C + residual), then norm + quantiser
+    M, N, K = 8192, 2560, 256
+    Aq, As, Bq, Bs = _inputs(oracle, M, N, K, 2)
+    res = torch.from_numpy(rng.standard_normal((M, N)).astype(np.float32)).cuda().to(torch.bfloat16)
+    w = g(rng.uniform(0.5, 1.5, N).astype(np.float32))
+    h0, h3 = torch.empty_like(res), torch.empty_like(res)
+    qa, sa = lib.fp8_gemm_add_rmsnorm_quant(g(Aq), g(As), g(Bq), g(Bs), res, h0, w, 1e-6, M, N, K, tile=T256, split_k=1)
+    qb, sb = lib.fp8_gemm_add_rmsnorm_quant(g(Aq), g(As), g(Bq), g(Bs), res, h3, w, 1e-6, M, N, K, tile=T128, split_k=1)
+    torch.cuda.synchronize()
+    assert torch.equal(h0.view(torch.int16), h3.view(torch.int16)) and torch.equal(qa, qb) and torch.equal(sa.view(torch.int32), sb.view(torch.int32))
