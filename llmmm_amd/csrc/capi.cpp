@@ -53,7 +53,7 @@ int heuristic_split(int M, int N, int K)
 
 // Tile for the MFMA kernels: fewest "waves" of workgroups over the 256 CUs, weighted by tile
 // area and a mild efficiency penalty for the smaller tiles (less operand reuse per byte of LDS).
-int heuristic_tile(int M, int N, bool fp8 = false)
+int heuristic_tile(int M, int N)
 {
   static const struct {
     int   id, bm, bn, per_cu;
@@ -69,9 +69,9 @@ int heuristic_tile(int M, int N, bool fp8 = false)
     const long  tiles = (long)(M / c.bm) * (N / c.bn);
     const long  slots = (long)NUM_CUS * c.per_cu;
     float       waves = (float)((tiles + slots - 1) / slots);
-    if (fp8 && c.id == LLMMM_TILE_256x256) {
-      // the FP8 launch of 256 x 256 tiles fills a partly empty last round with half-size tiles where it can (the same
-      // conditions as launch_fp8 in fp8_gemm.hip): that round then costs half
+    if (c.id == LLMMM_TILE_256x256) {
+      // a launch of 256 x 256 tiles fills a partly empty last round with half-size tiles where it can (the same
+      // conditions as launch_fp8 / launch_fp16 in the kernel files): that round then costs half
       const long tm = M / 256, tn = N / 256, full = tiles / NUM_CUS * NUM_CUS;
       if (tiles > NUM_CUS && tm > 1 && full % tm == 0 && tn - full / tm > 0 && (tn - full / tm) * tm * 2 <= NUM_CUS) waves -= 0.5f;
     }
@@ -161,7 +161,7 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
   }
   if (cfg->tile < 0) {
     if (M % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
-    cfg->tile = heuristic_tile(M, N, true);
+    cfg->tile = heuristic_tile(M, N);
   }
   if (cfg->tile == LLMMM_TILE_SKINNY) {
     if (cfg->split_k <= 0) cfg->split_k = heuristic_split(M, N, K);

@@ -168,14 +168,15 @@ __device__ __forceinline__ void fp16_mfma8(int half, int part, const typename Mf
     for (int mf = 0; mf < MF; ++mf) acc[4 * half + q][mf] = Mfma32<T>::run(b[q], a[mf], acc[4 * half + q][mf]);
 }
 
+// The kernel's body for tile `tile_index` of the tiles_m x tiles_n tiles of the column range that starts at n_base (0 and
+// the whole matrix for the plain kernel); lds_raw: the workgroup's ring of four stages.
 template <typename T, int BM, int BN, int WM, bool B_NK, bool KTAIL>
-__global__ void __launch_bounds__((BM / WM) * (BN / 128) * 64)
-fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n)
+__device__ __forceinline__ void fp16_gemm_body(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K, int tiles_m,
+                                               int tiles_n, char LLMMM_LDS* lds_raw, int tile_index, int n_base)
 {
   typedef Fp16Tile<T, BM, BN, WM, B_NK> TC;
   typedef typename Mfma32<T>::vec   vec;
   constexpr int                     MF = TC::MF;
-  __shared__ __attribute__((aligned(1024))) char lds_raw[4 * TC::STAGE];  // the ring of four stages
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -183,8 +184,8 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
   const int wm   = wave % TC::WAVES_M;
   const int wn   = wave / TC::WAVES_M;
   int       tm, tn;
-  tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
+  tile_coords(tile_index, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = n_base + tn * BN;
 
   // ---- loader setup: lane -> what the 16 bytes at (1 KB group base + 16*lane) must hold
   Fp16Loader<TC::B_LOADS> ld;
@@ -345,12 +346,57 @@ fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
   }
 }
 
+template <typename T, int BM, int BN, int WM, bool B_NK, bool KTAIL>
+__global__ void __launch_bounds__((BM / WM) * (BN / 128) * 64)
+fp16_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n)
+{
+  __shared__ __attribute__((aligned(1024))) char lds_raw[4 * Fp16Tile<T, BM, BN, WM, B_NK>::STAGE];  // the ring of four stages
+  fp16_gemm_body<T, BM, BN, WM, B_NK, KTAIL>(A, B, C, M, N, K, tiles_m, tiles_n, (char LLMMM_LDS*)lds_raw, blockIdx.x, 0);
+}
+
+// 256 x 256 tiles whose number is not a multiple of the 256 CUs end with a round that keeps part of the chip busy for a
+// whole tile's time (2048 x 19456: 608 tiles, the third round 96 of them).  One launch of both shapes: the columns that fill
+// whole rounds go to 256 x 256 tiles (workgroups 0 .. tiles_m_big * cols_big - 1, dispatched first), the remaining columns
+// to twice as many 128 x 256 tiles -- the same eight waves, ring and K loop, half the rows per wave, the same results.
+template <typename T, bool B_NK, bool KTAIL>
+__global__ void __launch_bounds__(512)
+fp16_gemm_hybrid_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K, int tiles_m_big, int cols_big,
+                        int cols_small)
+{
+  static_assert(Fp16Tile<T, 128, 256, 32, B_NK>::STAGE <= Fp16Tile<T, 256, 256, 64, B_NK>::STAGE, "the small tiles fit the large tiles' ring");
+  __shared__ __attribute__((aligned(1024))) char lds_raw[4 * Fp16Tile<T, 256, 256, 64, B_NK>::STAGE];
+  const int n_big = tiles_m_big * cols_big;
+  if ((int)blockIdx.x < n_big)
+    fp16_gemm_body<T, 256, 256, 64, B_NK, KTAIL>(A, B, C, M, N, K, tiles_m_big, cols_big, (char LLMMM_LDS*)lds_raw, blockIdx.x, 0);
+  else
+    fp16_gemm_body<T, 128, 256, 32, B_NK, KTAIL>(A, B, C, M, N, K, 2 * tiles_m_big, cols_small, (char LLMMM_LDS*)lds_raw, (int)blockIdx.x - n_big,
+                                                 cols_big * 256);
+}
+
 // --------------------------------------------------------------------------------------------- host
 template <typename T, int BM, int BN, int WM, bool B_NK>
 static hipError_t launch_fp16(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t stream)
 {
   typedef Fp16Tile<T, BM, BN, WM, B_NK> TC;
   const int tiles_m = M / BM, tiles_n = N / BN;
+  if constexpr (BM == 256 && BN == 256) {
+    // more than one round of the chip with a partly filled last one: whole rounds in 256 x 256 tiles, the remaining
+    // columns in 128 x 256 tiles, if those fit one round (fp16_gemm_hybrid_kernel)
+    const long tiles = (long)tiles_m * tiles_n, full = tiles / 256 * 256;
+    if (tiles > 256 && tiles_m > 1 && full % tiles_m == 0) {
+      const int cols_big = (int)(full / tiles_m), cols_small = tiles_n - cols_big;
+      if (cols_small > 0 && (long)cols_small * tiles_m * 2 <= 256) {
+        const dim3 grid(tiles_m * cols_big + 2 * tiles_m * cols_small);
+        if (K % TC::BK)
+          hipLaunchKernelGGL((fp16_gemm_hybrid_kernel<T, B_NK, true>), grid, dim3(512), 0, stream, (const T*)A, (const T*)B, (T*)C, M, N, K, tiles_m,
+                             cols_big, cols_small);
+        else
+          hipLaunchKernelGGL((fp16_gemm_hybrid_kernel<T, B_NK, false>), grid, dim3(512), 0, stream, (const T*)A, (const T*)B, (T*)C, M, N, K, tiles_m,
+                             cols_big, cols_small);
+        return hipGetLastError();
+      }
+    }
+  }
   if (K % TC::BK)
     hipLaunchKernelGGL((fp16_gemm_kernel<T, BM, BN, WM, B_NK, true>), dim3(tiles_m * tiles_n), dim3(TC::NT), 0, stream, (const T*)A,
                        (const T*)B, (T*)C, M, N, K, tiles_m, tiles_n);

@@ -92,3 +92,25 @@ def test_head_and_residual_epilogues_across_the_seam(lib, oracle):
     qb, sb = lib.fp8_gemm_add_rmsnorm_quant(g(Aq), g(As), g(Bq), g(Bs), res, h3, w, 1e-6, M, N, K, tile=T128, split_k=1)
     torch.cuda.synchronize()
     assert torch.equal(h0.view(torch.int16), h3.view(torch.int16)) and torch.equal(qa, qb) and torch.equal(sa.view(torch.int32), sb.view(torch.int32))
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K,bt", [(512, 33280, 96, False), (2048, 19456, 64, True), (512, 33024, 80, False)])
+def test_fp16_gemm_two_shape_launch(lib, oracle, dt, M, N, K, bt):
+    """The FP16 / BF16 GEMM takes the same launch form; every tile adds the K steps in the same order, so the result must
+    equal the 128 x 128 tiles' bit for bit (K = 80, 96: the K-tail path as well)."""
+    T = torch.float16 if dt == "f16" else torch.bfloat16
+    rng = np.random.default_rng(M + N + K)
+    A = torch.from_numpy(rng.uniform(-1, 1, (M, K)).astype(np.float32)).cuda().to(T)
+    B = torch.from_numpy(rng.uniform(-1, 1, (K, N)).astype(np.float32)).cuda().to(T)
+    Bx = B.t().contiguous() if bt else B
+    C0 = torch.full((M, N), float("nan"), dtype=T, device="cuda")
+    C3 = torch.empty((M, N), dtype=T, device="cuda")
+    lib.fp16_gemm(A, Bx, C0, b_transposed=bt, tile=T256)
+    lib.fp16_gemm(A, Bx, C3, b_transposed=bt, tile=T128)
+    torch.cuda.synchronize()
+    assert torch.equal(C0.view(torch.int16), C3.view(torch.int16))
+    rows = np.r_[0:16, M - 16:M]
+    ref = oracle.kahan_gemm(A[rows].float().cpu().numpy(), B.float().cpu().numpy())
+    got = C0[rows].float().cpu().numpy()
+    assert np.all(np.abs(got - ref) <= 1e-3 + 1e-2 * np.abs(ref))
