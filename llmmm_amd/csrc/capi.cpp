@@ -157,7 +157,11 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
         cfg->split_k = e.split_k;
         break;
       }
-    if (cfg->tile < 0 && M % 128) cfg->tile = LLMMM_TILE_SKINNY;  // untuned M = 128 goes to a split tile kernel
+    // untuned shapes: the weight-streaming kernel up to 64 rows; above that only while the weight matrix is small -- its
+    // eight 16-row blocks per wave and its fp32 planes grow with M, and from about 20 MB of weights on, one row of 128 x 128
+    // tiles (a row tail for M < 128) is faster (measured at M = 96, us, streaming / tiles: N x K = 4096 x 4096 12.4 / 14.2,
+    // 6144 x 4096 19.9 / 16.0, 4096 x 14336 39.4 / 22.1, 28672 x 4096 66.7 / 27.1)
+    if (cfg->tile < 0) cfg->tile = (M <= 64 || (long)N * K < 20000000L) ? LLMMM_TILE_SKINNY : LLMMM_TILE_128x128;
   }
   if (cfg->tile < 0) {
     if (M % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
@@ -167,7 +171,7 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
     if (cfg->split_k <= 0) cfg->split_k = heuristic_split(M, N, K);
   }
   else if (cfg->split_k <= 0)
-    cfg->split_k = heuristic_tile_split(cfg->tile, M, N, K);
+    cfg->split_k = heuristic_tile_split(cfg->tile, M < 128 ? 128 : M, N, K);
   return LLMMM_OK;
 }
 
@@ -202,7 +206,7 @@ int choose_fp8_out(int out_kind, int M, int N, int K, llmmm_gemm_cfg* cfg)
       if (small_plane && wide_tiles < NUM_CUS / 2) {
         if (!narrow) cfg->tile = LLMMM_TILE_128x128;  // through one fp32 plane, twice the workgroups
       }
-      else if (narrow)
+      else if (narrow && M % 128 == 0)  // (a row tail stays with the 128 x 128 tiles and the plane)
         cfg->tile = (M % 256 == 0 && (long)(M / 256) * (N / 256) >= NUM_CUS) ? LLMMM_TILE_256x256 : LLMMM_TILE_128x256;
     }
   }
@@ -397,6 +401,8 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
   if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
   if (user) {
+    // (a named weight-streaming kernel where the library would have taken tiles: the split is that kernel's own heuristic)
+    if (user->tile == LLMMM_TILE_SKINNY && cfg.tile != LLMMM_TILE_SKINNY && M <= SKINNY_MAX_M) cfg.split_k = heuristic_split(M, N, K);
     if (user->tile != LLMMM_TILE_AUTO) cfg.tile = user->tile;
     if (user->split_k > 0) cfg.split_k = user->split_k;
     if (user->b_layout != LLMMM_FP8_B_ROWS && user->b_layout != LLMMM_FP8_B_PRESHUFFLED)
@@ -580,6 +586,8 @@ static int resolve_plane_cfg(const void*& A, const float*& As, const void* Bt, c
   if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
   if (user) {
+    // (a named weight-streaming kernel where the library would have taken tiles: the split is that kernel's own heuristic)
+    if (user->tile == LLMMM_TILE_SKINNY && cfg.tile != LLMMM_TILE_SKINNY && M <= SKINNY_MAX_M) cfg.split_k = heuristic_split(M, N, K);
     if (user->tile != LLMMM_TILE_AUTO) cfg.tile = user->tile;
     if (user->split_k > 0) cfg.split_k = user->split_k;
     if (user->b_layout != LLMMM_FP8_B_ROWS && user->b_layout != LLMMM_FP8_B_PRESHUFFLED)

@@ -83,3 +83,32 @@ def test_swiglu_and_planes_entry_points_on_tail_rows(lib, oracle):
     lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(dA, dAs, dB, dBs, Hr, Hsr, M, N, K, workspace=ws, tile=SKINNY, split_k=1)
     torch.cuda.synchronize()
     assert torch.equal(H, Hr) and torch.equal(Hs.view(torch.int32), Hsr.view(torch.int32))
+
+
+def test_untuned_shapes_between_64_and_128_rows(lib, oracle):
+    """Shapes the tune table does not know: large weight matrices go to one row of 128 x 128 tiles, small ones stay with the
+    weight-streaming kernel; both against the oracle, the SwiGLU output included."""
+    from llmmm_amd import _lib
+    assert lib.query_config(_lib.OUT_FP8Q, 96, 6144, 4096)[0] == T128      # 25 MB of weights
+    assert lib.query_config(_lib.OUT_FP8Q, 128, 6144, 4096)[0] == T128
+    assert lib.query_config(_lib.OUT_FP8Q, 96, 4096, 4096)[0] == SKINNY    # 17 MB
+    assert lib.query_config(_lib.OUT_FP8Q, 128, 2048, 2048)[0] == SKINNY
+    assert lib.query_config(_lib.OUT_FP8Q, 64, 6144, 4096)[0] == SKINNY
+    M, N, K = 90, 6144, 4096
+    Aq, As, Bq, Bs = _inputs(oracle, M, N, K, 9)
+    dA, dAs, dB, dBs = (torch.from_numpy(a).cuda() for a in (Aq, As, Bq, Bs))
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    C = torch.empty((M, N), device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dA, dAs, dB, dBs, C, M, N, K)
+    H = torch.empty((M, N // 2), dtype=torch.uint8, device="cuda")
+    Hs = torch.empty((N // 256, M), device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(dA, dAs, dB, dBs, H, Hs, M, N, K,
+                                                                                 workspace=lib.make_workspace(_lib.OUT_FP8Q_SWIGLU, M, N, K))
+    Hr, Hsr = torch.empty_like(H), torch.empty_like(Hs)
+    ws = torch.empty(8 * M * N * 4, dtype=torch.uint8, device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__swiglu__C_1x128__output_fp8(dA, dAs, dB, dBs, Hr, Hsr, M, N, K, workspace=ws, tile=SKINNY, split_k=4)
+    torch.cuda.synchronize()
+    assert_fp8_gemm_close(C.cpu().numpy(), ref, "untuned row tail")
+    # the two routes split K differently (fp32 sums in another order): codes may differ by one step where a value sits on a boundary
+    same = (H == Hr).float().mean().item()
+    assert same > 0.999 and torch.allclose(Hs, Hsr, rtol=1e-3)
