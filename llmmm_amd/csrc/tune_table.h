@@ -26,7 +26,6 @@ static const SkinnyTune kSkinnyTune[] = {
   {1, 2560, 9728, 10},
   {16, 2560, 9728, 10},
   {64, 2560, 9728, 10},
-  {127, 2560, 9728, 12},
   {1, 6144, 2560, 5},
   {16, 6144, 2560, 5},
   {64, 6144, 2560, 5},
@@ -34,7 +33,6 @@ static const SkinnyTune kSkinnyTune[] = {
   {1, 19456, 2560, 1},
   {16, 19456, 2560, 1},
   {64, 19456, 2560, 3},
-  {127, 19456, 2560, 5},
 };
 
 // FP8 MFMA tile kernels (M % 128 == 0).
