@@ -478,7 +478,7 @@ def main():
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="fp16_gemm_4096",
-                    help="fp16_gemm_4096 (headline) | fp8_gemm_fused_4096 | fp8_gemm_bf16_4096 | bf16_gemm_4096 | "
+                    help="fp16_gemm_4096 (headline) | fp16_gemm_2048x19456x2560 | fp8_gemm_fused_4096 | fp8_gemm_bf16_4096 | bf16_gemm_4096 | "
                          "decode_<qkv|o|gate_up|down>_m<M>[_pre] (_pre: weights pre-shuffled offline) | prefill_<qkv|o|gate_up|down>_m<M> | "
                          "prefill_gate_up_swiglu_m<M> | fused_<o|down>_add_norm_m<M> | fused_qkv_rope_m<M> | layer_[consumer_]m<M> | copy_1g (counter calibration only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
@@ -516,6 +516,15 @@ def main():
         value, unit = r["tflops"], "TFLOP/s"
         cfg = {"workload": "FP16 GEMM M=N=K=4096 A~N(0,1) B~N(0,0.02) seed 2, fp32 accumulate, %s out, "
                            "single kernel, no split-K" % dtype, "M": M, "N": N, "K": K}
+    elif w == "fp16_gemm_2048x19456x2560":
+        # 608 tiles of 256 x 256: two whole rounds of the chip and 96 tiles -- the launch of two tile shapes
+        M, N, K = 2048, 19456, 2560
+        r, _ = bench_fp16(M, N, K, args.steps, args.warmup, torch.float16, clock=True)
+        dtype, peak = "f16", PEAK_TFLOPS["f16"]
+        roof = {"bound": "mfma", "achieved": r["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": r["tflops"] / peak, "traffic": None,
+                "kernel": "fp16_gemm_hybrid_kernel<f16, row-major B>: 512 tiles of 256 x 256 + 192 of 128 x 256"}
+        value, unit = r["tflops"], "TFLOP/s"
+        cfg = {"workload": "FP16 GEMM M=2048 N=19456 K=2560 (the Qwen3-4B gate_up shape) A~N(0,1) B~N(0,0.02) seed 2, fp16 out", "M": M, "N": N, "K": K}
     elif w in ("fp8_gemm_fused_4096", "fp8_gemm_bf16_4096"):
         out = "fp8q" if "fused" in w else "bf16"
         r = bench_fp8(M, N, K, out, args.steps, args.warmup, clock=True)
