@@ -134,6 +134,19 @@ LLMMM_API size_t llmmm_fp8_gemm_workspace(int out_kind, int M, int N, int K);
 /* The configuration llmmm_fp8_gemm would use for this shape (tune table, then heuristic). */
 LLMMM_API int llmmm_fp8_gemm_query(int out_kind, int M, int N, int K, llmmm_gemm_cfg* cfg);
 
+/* The same GEMM for callers that cannot allocate device memory and have no workspace to pass: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The split-K
+ * planes live in a fixed array of LLMMM_STATIC_WS_BYTES inside the library's device image (every GPU the library runs on
+ * holds its own copy until the process ends); the call allocates and frees nothing and is otherwise
+ * llmmm_fp8_gemm(out_kind, ..., workspace of llmmm_fp8_gemm_workspace(out_kind, M, N, K) bytes), bit for bit.  Shapes
+ * whose planes need more than LLMMM_STATIC_WS_BYTES return LLMMM_ERR_WORKSPACE (never a silently smaller split).  All
+ * calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams, different
+ * threads) race on it -- order them on one stream.  The array's address is looked up on the first call per device
+ * (one runtime query, not capturable): make one call per device before capturing. */
+#define LLMMM_STATIC_WS_BYTES (16u << 20)
+LLMMM_API int llmmm_fp8_gemm_static_ws(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs,
+                                       int M, int N, int K, void* stream);
+
 /* ---- FP8 blockwise quantiser ------------------------------------------------------------
  * Replaces  template<int QUANT_M, int QUANT_N, bool SCALE_TRANSPOSE>
  *           void fp8_blockwise_symmetric_quantization(const float* x, __nv_fp8_e4m3* q,

@@ -28,6 +28,7 @@ class APlanesRmsnorm(ctypes.Structure):
     _fields_ = [("planes", ctypes.c_void_p), ("splits", ctypes.c_int), ("hidden_dtype", ctypes.c_int), ("residual", ctypes.c_void_p),
                 ("hidden_out", ctypes.c_void_p), ("norm_weight", ctypes.c_void_p), ("eps", ctypes.c_float)]
 PROBE_FP8 = 2
+STATIC_WS_BYTES = 16 << 20
 TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_64x128, TILE_128x160, TILE_SKINNY = -1, 0, 1, 2, 3, 4, 5, 8
 
 
@@ -43,6 +44,7 @@ SIGNATURES = {
     "llmmm_fp16_gemm_ex": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _c.POINTER(GemmCfg), _vp]),
     "llmmm_fp8_gemm": (_i, [_i, _vp, _fp, _vp, _fp, _vp, _fp, _i, _i, _i, _vp, _sz, _vp]),
     "llmmm_fp8_gemm_ex": (_i, [_i, _vp, _fp, _vp, _fp, _vp, _fp, _i, _i, _i, _vp, _sz, _c.POINTER(GemmCfg), _vp]),
+    "llmmm_fp8_gemm_static_ws": (_i, [_i, _vp, _fp, _vp, _fp, _vp, _fp, _i, _i, _i, _vp]),
     "llmmm_fp8_gemm_workspace": (_sz, [_i, _i, _i, _i]),
     "llmmm_fp8_gemm_query": (_i, [_i, _i, _i, _i, _c.POINTER(GemmCfg)]),
     "llmmm_quant_fp8": (_i, [_i, _fp, _vp, _fp, _i, _i, _vp]),

@@ -29,6 +29,7 @@ SOURCES = {
     "quant_fp8.hip": [],
     "layout.hip": [],
     "probe.hip": [],
+    "static_ws.hip": [],
     "capi.cpp": ["-x", "hip"],
 }
 

@@ -24,6 +24,20 @@ int fail(int code, const char* fmt, ...)
   return code;
 }
 
+}  // namespace
+
+// The same for the other files of the library (declared in kernels.h).
+int llmmm::report_error(int code, const char* fmt, ...)
+{
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+namespace {
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 constexpr int    MAX_SPLIT_K     = 32;

@@ -98,6 +98,9 @@ hipError_t probe_stream_read_launch(const void* src, size_t bytes, float* sink, 
 hipError_t planes_add_rmsnorm_quant_launch(int hidden_dtype, const float* planes, int S, const void* residual, void* hidden, const float* w,
                                            float eps, void* q, float* scale, int M, int N, hipStream_t stream);
 
+// Leaves the text in the calling thread's llmmm_last_error() and returns `code` (capi.cpp).
+int report_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
 hipError_t fill_u32_launch(uint32_t* p, uint32_t value, size_t n, hipStream_t stream);
 
 }  // namespace llmmm

@@ -1,0 +1,72 @@
+"""llmmm_fp8_gemm_static_ws (the FP8 GEMM whose split-K planes live in a fixed array inside the library, for callers
+that cannot allocate) against llmmm_fp8_gemm with a caller's workspace: bit for bit, on two calls in a row that share
+the array, the second smaller than the first, and against the oracle at the fused-output bar."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_fp8_gemm_close, assert_fused_close, fp8_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _both(raw, out_kind, M, N, K, t, stream):
+    """One call of each entry point on the same device operands; returns the two (C, Cs) pairs as numpy arrays."""
+    from llmmm_amd import _lib
+    need = raw.llmmm_fp8_gemm_workspace(out_kind, M, N, K)
+    assert 0 < need <= _lib.STATIC_WS_BYTES, "the case must split K and fit the built-in array"
+    ws = torch.full((need,), 0xA5, dtype=torch.uint8, device="cuda")
+    dt = {0: torch.float32, 1: torch.bfloat16, 2: torch.uint8}[out_kind]
+    outs = []
+    for static in (False, True):
+        C = torch.full((M, N), 0x55 if dt == torch.uint8 else float("nan"), dtype=dt, device="cuda")
+        Cs = torch.full((N // 128, M), -1.0, dtype=torch.float32, device="cuda")
+        if static:
+            rc = raw.llmmm_fp8_gemm_static_ws(out_kind, _p(t[0]), _p(t[1]), _p(t[2]), _p(t[3]), _p(C), _p(Cs), M, N, K, stream)
+        else:
+            rc = raw.llmmm_fp8_gemm(out_kind, _p(t[0]), _p(t[1]), _p(t[2]), _p(t[3]), _p(C), _p(Cs), M, N, K, _p(ws), need, stream)
+        assert rc == 0, raw.llmmm_last_error().decode()
+        torch.cuda.synchronize()
+        bits = C.view(torch.int16) if dt == torch.bfloat16 else C
+        outs.append((bits.cpu().numpy(), Cs.cpu().numpy()))
+    return outs
+
+
+def test_static_workspace_matches_caller_workspace(oracle):
+    from llmmm_amd import _lib
+    raw = _lib.lib
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # first the larger problem (16 x 6144 x 2560, split 5: 1.9 MB of planes), then a smaller one (1 x 2560 x 4096,
+    # split 8: 80 KB) that finds the first call's partial sums still in the array
+    for M, N, K, seed in ((16, 6144, 2560, 11), (1, 2560, 4096, 12)):
+        Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=seed)
+        t = [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (Aq, As, Bq, Bs)]
+        ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+        for out_kind in (_lib.OUT_FP8Q, _lib.OUT_F32, _lib.OUT_BF16):
+            (c0, s0), (c1, s1) = _both(raw, out_kind, M, N, K, t, stream)
+            what = "%dx%dx%d out %d" % (M, N, K, out_kind)
+            assert (c0.view(np.uint8) == c1.view(np.uint8)).all(), what + ": outputs differ between the two entry points"
+            if out_kind == _lib.OUT_FP8Q:
+                assert (s0.view(np.uint32) == s1.view(np.uint32)).all(), what + ": scales differ between the two entry points"
+                rq, rs = oracle.requant_c_1x128(ref)
+                assert_fused_close(oracle, c1, s1, rq, rs, what)
+            elif out_kind == _lib.OUT_F32:
+                assert_fp8_gemm_close(c1, ref, what)
+            else:
+                assert_fp8_gemm_close(oracle.bf16_bits_to_f32(c1.view(np.uint16)), ref, what)
+
+
+def test_static_workspace_rejects_what_does_not_fit():
+    from llmmm_amd import _lib
+    raw = _lib.lib
+    M, N, K = 1024, 2560, 9728  # the down projection at M = 1024 runs in three splits: 3 x 1024 x 2560 floats = 31 MB
+    assert raw.llmmm_fp8_gemm_workspace(_lib.OUT_FP8Q, M, N, K) > _lib.STATIC_WS_BYTES
+    fake = ctypes.c_void_p(0x1000)
+    rc = raw.llmmm_fp8_gemm_static_ws(_lib.OUT_FP8Q, fake, fake, fake, fake, fake, fake, M, N, K, None)
+    assert rc == _lib.ERR_WORKSPACE and b"built-in array" in raw.llmmm_last_error()
