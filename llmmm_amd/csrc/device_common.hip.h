@@ -156,6 +156,39 @@ __device__ __forceinline__ float wave_xor_max(float v, int mask)
   return fmaxf(v, wave_xor_get(v, mask));
 }
 
+// ---------------------------------------------------------------------------------------------
+// fp32 -> OCP e4m3, four codes per dword, as the reference's __nv_fp8_e4m3(float) gives them (round to nearest even,
+// saturate to +-448, every NaN -> 0x7F; examples/005.fp8.mm.cu:482-485, examples/005.fp8.mm.opt.cu:445-454).
+// v_cvt_pk_fp8_f32 rounds to nearest even and converts everything below 464 to 448, but writes 0xFF for a NaN of
+// either sign and sign | 0x7F for larger magnitudes and infinities (measured).
+// ---------------------------------------------------------------------------------------------
+// Bytes whose low seven bits are all ones (the two NaN codes) lose their sign bit; other bytes are unchanged.
+__device__ __forceinline__ uint32_t e4m3x4_nan_codes_to_7f(uint32_t c)
+{
+  const uint32_t m = ((c & 0x7F7F7F7Fu) + 0x01010101u) & 0x80808080u;
+  return c & ~m;
+}
+// For values that are NaN or lie within +-448 (1 + 2^-20): quotients by a block's own scale, products with
+// 448 / amax.  No clamp is needed then, and the only 0x7F / 0xFF bytes the hardware writes stand for NaN.
+__device__ __forceinline__ uint32_t pack_e4m3x4_in_range(float a, float b, float c, float d)
+{
+  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  v     = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+  return e4m3x4_nan_codes_to_7f((uint32_t)v);
+}
+// For any value: clamped to +-448 first (v_med3_f32 turns a NaN into a bound, so NaN is put back by hand).
+__device__ __forceinline__ uint32_t pack_e4m3x4_sat(float a, float b, float c, float d)
+{
+  const uint32_t nan = (a != a ? 0x000000FFu : 0u) | (b != b ? 0x0000FF00u : 0u) | (c != c ? 0x00FF0000u : 0u) | (d != d ? 0xFF000000u : 0u);
+  a     = __builtin_amdgcn_fmed3f(a, -448.f, 448.f);
+  b     = __builtin_amdgcn_fmed3f(b, -448.f, 448.f);
+  c     = __builtin_amdgcn_fmed3f(c, -448.f, 448.f);
+  d     = __builtin_amdgcn_fmed3f(d, -448.f, 448.f);
+  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  v     = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+  return ((uint32_t)v & ~nan) | (0x7F7F7F7Fu & nan);
+}
+
 // Four consecutive row elements of type float / bf16 / fp16 <-> fp32 (one 16- or 8-byte access).
 template <typename IN_T>
 __device__ __forceinline__ f32x4 load_row4(const IN_T* p);

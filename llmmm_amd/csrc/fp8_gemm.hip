@@ -247,29 +247,6 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int
   for (int mf = 0; mf < MF; ++mf) asm volatile("" : "+v"(acc[NF - 1][mf]));
 }
 
-__device__ __forceinline__ uint32_t pack_e4m3x4(float a, float b, float c, float d)
-{
-  // v_cvt_pk_fp8_f32 rounds to nearest even but turns |x| > 464 into NaN: clamp first, which
-  // gives the saturate-to-finite behaviour of the reference's __nv_fp8_e4m3(float).
-  a     = __builtin_amdgcn_fmed3f(a, -448.f, 448.f);
-  b     = __builtin_amdgcn_fmed3f(b, -448.f, 448.f);
-  c     = __builtin_amdgcn_fmed3f(c, -448.f, 448.f);
-  d     = __builtin_amdgcn_fmed3f(d, -448.f, 448.f);
-  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
-  v     = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
-  return (uint32_t)v;
-}
-
-// The same conversion without the clamp, for values that are known to lie within +-448 * (1 + 2^-22):
-// the fused epilogue's C * (448 / amax), whose magnitude cannot exceed the row's own amax * (448 / amax).
-// Anything below 464 rounds to 448, so the codes are those of pack_e4m3x4; 128 v_med3 per lane are saved.
-__device__ __forceinline__ uint32_t pack_e4m3x4_in_range(float a, float b, float c, float d)
-{
-  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
-  v     = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
-  return (uint32_t)v;
-}
-
 // SwiGLU exchange: the fragments mf = SEND0 .. SEND0 + MF/2 - 1 go to the partner wave through LDS, lane for lane.
 template <int MF, int SEND0>
 __device__ __forceinline__ void swiglu_send(const f32x4 (&acc)[8][MF], char LLMMM_LDS* region, int lane)
@@ -861,7 +838,7 @@ fp8_splitk_reduce_kernel(const float* __restrict__ planes, int S, void* __restri
     }
     else {  // e4m3 codes + 1x128 scales, of C or (SwiGLU) of h, whose rows are N/2 wide
       const int ldc = OUT == OUT_SWIGLU ? (N >> 1) : N;
-      float a = fmaxf(fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1])), fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
+      float a = fmaxf(fmaxf(fmaxf(0.f, __builtin_fabsf(v[0])), __builtin_fabsf(v[1])), fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
       a       = wave_xor_max(a, 1);
       a       = wave_xor_max(a, 2);
       a       = wave_xor_max(a, 4);
@@ -869,7 +846,7 @@ fp8_splitk_reduce_kernel(const float* __restrict__ planes, int S, void* __restri
       a       = wave_xor_max(a, 16);
       const float scale = a / 448.f;
       const float inv   = a > 0.f ? 448.f / a : 0.f;
-      *(uint32_t*)((uint8_t*)Cv + (size_t)m * ldc + n) = pack_e4m3x4(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+      *(uint32_t*)((uint8_t*)Cv + (size_t)m * ldc + n) = pack_e4m3x4_in_range(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
       if (l32 == 0) Cs[(size_t)nb * M + m] = scale;
     }
   }
@@ -939,12 +916,12 @@ fp8_planes_qk_norm_rope_kernel(const float* __restrict__ planes, int S, void* __
       *(bf16x4*)((__bf16*)Cv + (size_t)m * N + n) = o;
     }
     else {
-      float a = fmaxf(fmaxf(__builtin_fabsf(v[0]), __builtin_fabsf(v[1])), fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
+      float a = fmaxf(fmaxf(fmaxf(0.f, __builtin_fabsf(v[0])), __builtin_fabsf(v[1])), fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
 #pragma unroll
       for (int step = 1; step <= 16; step <<= 1) a = wave_xor_max(a, step);
       const float scale = a / 448.f;
       const float inv   = a > 0.f ? 448.f / a : 0.f;
-      *(uint32_t*)((uint8_t*)Cv + (size_t)m * N + n) = pack_e4m3x4(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+      *(uint32_t*)((uint8_t*)Cv + (size_t)m * N + n) = pack_e4m3x4_in_range(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
       if (l32 == 0) Cs[(size_t)head * M + m] = scale;
     }
   }

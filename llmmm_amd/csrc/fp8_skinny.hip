@@ -26,17 +26,6 @@ namespace llmmm {
 
 enum { SK_OUT_F32 = 0, SK_OUT_BF16 = 1, SK_OUT_FP8Q = 2 };
 
-__device__ __forceinline__ uint32_t sk_pack_e4m3x4(float a, float b, float c, float d)
-{
-  a     = __builtin_amdgcn_fmed3f(a, -448.f, 448.f);
-  b     = __builtin_amdgcn_fmed3f(b, -448.f, 448.f);
-  c     = __builtin_amdgcn_fmed3f(c, -448.f, 448.f);
-  d     = __builtin_amdgcn_fmed3f(d, -448.f, 448.f);
-  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
-  v     = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
-  return (uint32_t)v;
-}
-
 // What one 128-K slice needs besides the weights: the activation rows (straight into the MFMA
 // operand registers) and both scales.  Rows beyond M are clamped to M-1 (a valid address, no
 // divergence); their products are computed and never stored.
@@ -388,12 +377,12 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
       if (c < chunks && live && j >= 0 && j < nsl) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) held[u][e] = (held[u][e] * rn) * wv[u][e];
-        float a = fmaxf(fmaxf(__builtin_fabsf(held[u][0]), __builtin_fabsf(held[u][1])), fmaxf(__builtin_fabsf(held[u][2]), __builtin_fabsf(held[u][3])));
+        float a = fmaxf(fmaxf(fmaxf(0.f, __builtin_fabsf(held[u][0])), __builtin_fabsf(held[u][1])), fmaxf(__builtin_fabsf(held[u][2]), __builtin_fabsf(held[u][3])));
 #pragma unroll
         for (int step = 1; step <= 16; step <<= 1) a = wave_xor_max(a, step);
         const float sc = a / 448.f;
         uint32_t    cd = 0;
-        if (sc != 0.f) cd = sk_pack_e4m3x4(held[u][0] / sc, held[u][1] / sc, held[u][2] / sc, held[u][3] / sc);
+        if (sc != 0.f) cd = pack_e4m3x4_sat(held[u][0] / sc, held[u][1] / sc, held[u][2] / sc, held[u][3] / sc);
         *(uint32_t LLMMM_LDS*)((char LLMMM_LDS*)a_stage + j * 2048 + kmajor_offset<SWZ_ROWS16>(r, (c & 31) >> 2) + (c & 3) * 4) = cd;
         if ((c & 31) == 0) a_scale[j * 16 + r] = sc;
       }
@@ -438,13 +427,13 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
           f32x4     h;
 #pragma unroll
           for (int q = 0; q < 4; ++q) h[q] = silu_mul(gv[u][q], uv[u][q]);
-          float a = fmaxf(fmaxf(__builtin_fabsf(h[0]), __builtin_fabsf(h[1])), fmaxf(__builtin_fabsf(h[2]), __builtin_fabsf(h[3])));
+          float a = fmaxf(fmaxf(fmaxf(0.f, __builtin_fabsf(h[0])), __builtin_fabsf(h[1])), fmaxf(__builtin_fabsf(h[2]), __builtin_fabsf(h[3])));
 #pragma unroll
           for (int step = 1; step <= 16; step <<= 1) a = wave_xor_max(a, step);
           const float scale = a / 448.f;
           const float inv   = a > 0.f ? 448.f / a : 0.f;
           *(uint32_t LLMMM_LDS*)((char LLMMM_LDS*)a_stage + j * 2048 + kmajor_offset<SWZ_ROWS16>(r, l32 >> 2) + (l32 & 3) * 4) =
-            sk_pack_e4m3x4(h[0] * inv, h[1] * inv, h[2] * inv, h[3] * inv);
+            pack_e4m3x4_in_range(h[0] * inv, h[1] * inv, h[2] * inv, h[3] * inv);
           if (l32 == 0) a_scale[j * 16 + r] = scale;
         }
       }
@@ -517,7 +506,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
     uint8_t* C = (uint8_t*)Cv;
 #pragma unroll
     for (int mb = 0; mb < MBLK; ++mb) {
-      float a = fmaxf(fmaxf(__builtin_fabsf(acc[mb][0]), __builtin_fabsf(acc[mb][1])),
+      float a = fmaxf(fmaxf(fmaxf(0.f, __builtin_fabsf(acc[mb][0])), __builtin_fabsf(acc[mb][1])),
                       fmaxf(__builtin_fabsf(acc[mb][2]), __builtin_fabsf(acc[mb][3])));
       a       = wave_xor_max(a, 16);
       a       = wave_xor_max(a, 32);
@@ -534,7 +523,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
       const float inv   = amax > 0.f ? 448.f / amax : 0.f;
       if (m < M) {
         *(uint32_t*)(C + (size_t)m * N + ncol) =
-          sk_pack_e4m3x4(acc[mb][0] * inv, acc[mb][1] * inv, acc[mb][2] * inv, acc[mb][3] * inv);
+          pack_e4m3x4_in_range(acc[mb][0] * inv, acc[mb][1] * inv, acc[mb][2] * inv, acc[mb][3] * inv);
         if (wave == 0 && g == 0) Cs[(size_t)ng * M + m] = scale;
       }
     }

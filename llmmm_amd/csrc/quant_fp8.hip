@@ -16,17 +16,6 @@
 
 namespace llmmm {
 
-__device__ __forceinline__ uint32_t q_pack_e4m3x4(float a, float b, float c, float d)
-{
-  a     = __builtin_amdgcn_fmed3f(a, -448.f, 448.f);
-  b     = __builtin_amdgcn_fmed3f(b, -448.f, 448.f);
-  c     = __builtin_amdgcn_fmed3f(c, -448.f, 448.f);
-  d     = __builtin_amdgcn_fmed3f(d, -448.f, 448.f);
-  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
-  v     = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
-  return (uint32_t)v;
-}
-
 // e4m3 codes of v[0..3] / s (s != 0, |v[e]| <= 448 s up to rounding), equal bit for bit to converting the correctly
 // rounded fp32 quotients -- without dividing, almost always.  An IEEE fp32 division costs about ten vector instructions
 // per element and made the quantisers ALU-bound (the same element rate from bf16 and from fp32 inputs).  Instead:
@@ -35,6 +24,9 @@ __device__ __forceinline__ uint32_t q_pack_e4m3x4(float a, float b, float c, flo
 // correctly rounded quotient.  Otherwise (a quotient within 2^-20 of a rounding boundary of the 3-bit mantissa: about
 // 3 in 10^5 elements), or when s is so small or large that rcp(s) leaves the normal range, the lane divides.
 // No clamp on the fast path: |t| < 448 (1 + 2^-20), and everything below 464 converts to 448.
+// Non-finite values follow the reference's arithmetic: a NaN element gives 0x7F (on the fast path both brackets
+// convert to the hardware's NaN code, which e4m3x4_nan_codes_to_7f turns into 0x7F); an infinite or negative scale
+// (a block that holds an infinity, or nothing but NaN) fails the range test and the lane divides.
 __device__ __forceinline__ uint32_t q_pack_quotients_e4m3x4(f32x4 v, float s)
 {
   const float y  = __builtin_amdgcn_rcpf(s);
@@ -46,9 +38,14 @@ __device__ __forceinline__ uint32_t q_pack_quotients_e4m3x4(f32x4 v, float s)
   lo     = __builtin_amdgcn_cvt_pk_fp8_f32(t[2] * dn, t[3] * dn, lo, true);
   int hi = __builtin_amdgcn_cvt_pk_fp8_f32(t[0] * up, t[1] * up, 0, false);
   hi     = __builtin_amdgcn_cvt_pk_fp8_f32(t[2] * up, t[3] * up, hi, true);
-  if (lo == hi && s >= 0x1p-100f && s <= 0x1p100f) return (uint32_t)lo;
-  return q_pack_e4m3x4(v[0] / s, v[1] / s, v[2] / s, v[3] / s);
+  if (lo == hi && s >= 0x1p-100f && s <= 0x1p100f) return e4m3x4_nan_codes_to_7f((uint32_t)lo);
+  return pack_e4m3x4_sat(v[0] / s, v[1] / s, v[2] / s, v[3] / s);
 }
+
+// The reference starts its block maximum from (float)INT_MIN (examples/005.fp8.mm.cu:456) and its comparison never
+// takes a NaN, so a block that holds nothing but NaN keeps that seed: scale INT_MIN / 448, codes 0x7F.  fmaxf drops
+// NaN operands the same way.
+constexpr float QUANT_AMAX_SEED = -2147483648.f;
 
 __device__ __forceinline__ float amax4(float m, f32x4 v)
 {
@@ -73,7 +70,8 @@ __global__ void __launch_bounds__(256) quant_1x128_kernel(const float* __restric
   for (int m = mbeg + sub; m < mend; m += 8) {
     f32x4 v = {0.f, 0.f, 0.f, 0.f};
     if (live) v = __builtin_nontemporal_load((const f32x4*)(x + (size_t)m * N + n));
-    float a = amax4(0.f, v);
+    float a = QUANT_AMAX_SEED;
+    if (live) a = amax4(a, v);
     a       = wave_xor_max(a, 1);
     a       = wave_xor_max(a, 2);
     a       = wave_xor_max(a, 4);
@@ -107,13 +105,15 @@ __global__ void __launch_bounds__(256) quant_128x128_kernel(const float* __restr
   const int nbn  = (N + 127) >> 7;
   const bool live = n < N;
   f32x4     v[16];
-  float     a = 0.f;
+  float     a = QUANT_AMAX_SEED;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int m = mb * 128 + r * 8 + sub;
     v[r]        = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (live && m < M) v[r] = __builtin_nontemporal_load((const f32x4*)(x + (size_t)m * N + n));
-    a = amax4(a, v[r]);
+    if (live && m < M) {
+      v[r] = __builtin_nontemporal_load((const f32x4*)(x + (size_t)m * N + n));
+      a    = amax4(a, v[r]);
+    }
   }
   a = wave_xor_max(a, 1);
   a = wave_xor_max(a, 2);

@@ -386,7 +386,13 @@ ORACLE_API int oracle_fp8_gemm(const uint8_t* A, const float* As, const uint8_t*
  * reciprocal == 0: Cq = e4m3(C / scale)         (examples/005.fp8.mm.cu:759-769)
  * Cs[nb*M + m] = scale (opt.cu:458-461).
  * zero_guard != 0: an all-zero group gives codes 0 and scale 0 (this repository's kernels);
- * zero_guard == 0: the reference's unguarded arithmetic (0 * inf = NaN -> 0x7F). */
+ * zero_guard == 0: the reference's unguarded arithmetic (0 * inf = NaN -> 0x7F).
+ * Non-finite C: a NaN element never enters the maximum.  (In the reference a thread's chain
+ * `max_val > |c| ? max_val : |c|`, opt.cu:413, keeps a NaN only when it is the last value that thread compares, and the
+ * cross-lane `max()` steps behind it, opt.cu:415-416 and :432, drop it again: fmaxf semantics.  Only a group that holds
+ * nothing but NaN differs: NaN scale there, scale 0 here under the zero guard.)  A NaN element's code is 0x7F; an
+ * infinite element gives amax = scale = inf and 448/amax = 0, so finite elements become (signed) zeros and the
+ * infinite ones 0 * inf = NaN -> 0x7F, as in the reference. */
 ORACLE_API void oracle_requant_c_1x128(const float* C, uint8_t* Cq, float* Cs, int M, int N, int reciprocal,
                                        int zero_guard)
 {
@@ -398,7 +404,7 @@ ORACLE_API void oracle_requant_c_1x128(const float* C, uint8_t* Cq, float* Cs, i
       float amax = 0.0f;
       for (int n = n0; n < n1; ++n) {
         float v = fabsf(C[(size_t)m * N + n]);
-        amax    = amax > v ? amax : v;
+        if (v > amax) amax = v; /* a NaN is never taken, see above */
       }
       float scale = amax / 448.0f;
       float inv   = 448.0f / amax;
@@ -406,7 +412,7 @@ ORACLE_API void oracle_requant_c_1x128(const float* C, uint8_t* Cq, float* Cs, i
         float v = C[(size_t)m * N + n];
         float r;
         if (zero_guard && amax == 0.0f)
-          r = 0.0f;
+          r = v * 0.0f; /* zeros stay zeros, a NaN stays a NaN (code 0x7F) */
         else
           r = reciprocal ? v * inv : v / scale;
         Cq[(size_t)m * N + n] = oracle_e4m3_encode(r);

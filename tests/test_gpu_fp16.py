@@ -111,3 +111,30 @@ def test_cfg2_4096_slab_against_kahan_and_linearity(lib, oracle):
     perm = torch.randperm(M, device="cuda", generator=torch.Generator(device="cuda").manual_seed(0))
     Cp = lib.fp16_gemm(tA[perm].contiguous(), tB)
     assert torch.equal(Cp, C[perm]), "row permutation of A must permute the rows of C bit-exactly"
+
+
+@pytest.mark.parametrize("N,K", [(4096, 4096), (6144, 2048), (2048, 12288)])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_reference_test_shapes(lib, oracle, dtype, N, K):
+    """The six cases of the reference's own test (test/fp16_mm_test.cc:96-103: M = 4096, (N, K) as listed, half and
+    bfloat16, inputs ~ U(-5, 5) rounded to T on the host, :14-20 and :38-45) through the reference entry point.  The
+    Kahan oracle checks three 32-row slabs of the product of the rounded inputs; a row permutation covers the rest."""
+    M = 4096
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    g = torch.Generator(device="cuda").manual_seed(N + K)
+    tA = (torch.rand((M, K), generator=g, device="cuda") * 10 - 5).to(tdt)
+    tB = (torch.rand((K, N), generator=g, device="cuda") * 10 - 5).to(tdt)
+    C = torch.full((M, N), float("nan"), dtype=tdt, device="cuda")
+    lib.fp16_mm(tA, tB, C, M, N, K)
+    torch.cuda.synchronize()
+    rows = np.r_[0:32, 2040:2072, 4064:4096]
+    r = torch.from_numpy(rows).cuda()
+    ref = oracle.kahan_gemm(tA[r].float().cpu().numpy(), tB.float().cpu().numpy())
+    got = C[r].float().cpu().numpy()
+    # (bfloat16 keeps 8 significant bits: the result's own rounding, 2^-9 relative, is inside the 1e-2 bar)
+    assert_fp16_close(got, ref, "%s fp16_mm %dx%dx%d" % (dtype, M, N, K))
+    perm = torch.randperm(M, device="cuda", generator=g)
+    Cp = torch.empty_like(C)
+    lib.fp16_mm(tA[perm].contiguous(), tB, Cp, M, N, K)
+    torch.cuda.synchronize()
+    assert torch.equal(Cp, C[perm]), "row permutation of A must permute the rows of C bit-exactly"

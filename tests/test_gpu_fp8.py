@@ -192,27 +192,40 @@ def test_cfg5_decode_shapes(lib, oracle, name, N, K, M):
     _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs), ref, "%s M=%d" % (name, M))
 
 
-def _slab_check(lib, oracle, M, N, K, rows, seed):
-    """Full-size run on GPU-quantised inputs; the oracle checks a row slab, properties the rest."""
+def _slab_check(lib, oracle, M, N, K, rows, seed, dist="cfg3"):
+    """Full-size run on GPU-quantised inputs, all three outputs; the oracle checks a row slab, properties the rest.
+    dist "cfg3": A ~ N(0,1) with 1 % of the K channels x 20, B ~ N(0, 0.02); "reference": both operands
+    u / (|v| + 1) with u, v ~ U(-5, 5), the inputs of the reference's own driver (examples/005.fp8.mm.opt.cu:521-527)."""
     g = torch.Generator(device="cuda").manual_seed(seed)
-    X = torch.randn((M, K), generator=g, device="cuda")
-    X[:, torch.randperm(K, generator=g, device="cuda")[:max(1, -(-K // 100))]] *= 20
-    W = torch.randn((N, K), generator=g, device="cuda") * 0.02
+    if dist == "cfg3":
+        X = torch.randn((M, K), generator=g, device="cuda")
+        X[:, torch.randperm(K, generator=g, device="cuda")[:max(1, -(-K // 100))]] *= 20
+        W = torch.randn((N, K), generator=g, device="cuda") * 0.02
+    else:
+        def u(*shape):
+            return torch.rand(shape, generator=g, device="cuda") * 10 - 5
+        X = u(M, K) / (u(M, K).abs() + 1)
+        W = u(N, K) / (u(N, K).abs() + 1)
     Aq, As = lib.quantize_activation(X)
     Bq, Bs = lib.quantize_weight(W)
     C = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    Cb = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
     Cq = torch.empty((M, N), dtype=torch.uint8, device="cuda")
     Cs = torch.empty((N // 128, M), dtype=torch.float32, device="cuda")
     lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(Aq, As, Bq, Bs, C, M, N, K)
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_bf16(Aq, As, Bq, Bs, Cb, M, N, K)
     lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(Aq, As, Bq, Bs, Cq, Cs, M, N, K)
     torch.cuda.synchronize()
     r = torch.from_numpy(rows).cuda()
     ref = oracle.fp8_gemm(Aq[r].cpu().numpy(), As[:, r].contiguous().cpu().numpy(), Bq.cpu().numpy(), Bs.cpu().numpy(), promote=128)
     assert_fp8_gemm_close(C[r].cpu().numpy(), ref, "slab fp32")
+    assert_fp8_gemm_close(Cb[r].float().cpu().numpy(), ref, "slab bf16")
     rq, rs = oracle.requant_c_1x128(ref)
     assert_fused_close(oracle, Cq[r].cpu().numpy(), Cs[:, r].contiguous().cpu().numpy(), rq, rs, "slab fused")
-    # properties over the whole output: every 1x128 group has a code of magnitude 448 (its amax element),
+    # properties over the whole output: the bf16 output is the fp32 output rounded to nearest even (the same kernel
+    # and split produce both), every 1x128 group has a code of magnitude 448 (its amax element),
     # scales equal amax/448 of the fp32 result, and re-quantising the dequantised output is the identity
+    assert torch.equal(Cb, C.to(torch.bfloat16)), "bf16 output is not RNE(fp32 output)"
     dec = Cq.view(torch.float8_e4m3fn).float()
     assert (dec.abs().reshape(M, N // 128, 128).amax(-1) == 448).all()
     amax = C.abs().reshape(M, N // 128, 128).amax(-1)
@@ -227,7 +240,45 @@ def test_cfg3_cfg4_4096_full_size(lib, oracle):
     _slab_check(lib, oracle, 4096, 4096, 4096, np.r_[0:48, 2040:2088, 4048:4096], seed=3)
 
 
-@pytest.mark.parametrize("name,N,K", [("qkv", 6144, 2560), ("down", 2560, 9728)])
+@pytest.mark.parametrize("name,N,K", [("qkv", 6144, 2560), ("o", 2560, 4096), ("gate_up", 19456, 2560), ("down", 2560, 9728)])
 @pytest.mark.parametrize("M", [128, 2048])
 def test_cfg5_prefill_shapes(lib, oracle, name, N, K, M):
-    _slab_check(lib, oracle, M, N, K, np.r_[0:32, M - 32:M], seed=17)
+    # every Qwen3-4B projection at its stated (N, K): whatever tile, hybrid launch or split the library picks for it
+    _slab_check(lib, oracle, M, N, K, np.r_[0:32, M // 2 - 16:M // 2 + 16, M - 32:M] if M > 128 else np.r_[0:32, M - 32:M], seed=17)
+
+
+def test_reference_driver_shape_4096x7168x2048(lib, oracle):
+    # the one non-square problem the reference's own driver runs (examples/005.fp8.mm.opt.cu:515), with its inputs
+    _slab_check(lib, oracle, 4096, 7168, 2048, np.r_[0:32, 2040:2072, 4064:4096], seed=0, dist="reference")
+
+
+@pytest.mark.parametrize("tile,split", [("256x256", 0), ("128x128", 0), ("128x128", 2), (8, 1), (8, 3)])
+def test_non_finite_operands(lib, oracle, tile, split):
+    """NaN codes in A and in B and an infinite activation scale: the fp32 result is NaN / infinite exactly where the
+    oracle's is, and the fused output is the oracle's re-quantisation of it bit for bit -- NaN elements give code
+    0x7F whatever their sign, an infinite element makes the group's scale infinite and every finite element of the
+    group a signed zero (examples/005.fp8.mm.opt.cu:439-454 evaluated on such values)."""
+    skinny = tile == 8
+    M, N, K = (48 if skinny else 256), 512, 512
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=31)
+    Aq[3, 130] = 0x7F       # row 3: NaN in every column group
+    Aq[5, 7] = 0xFF
+    Bq[200, 300] = 0x7F     # column 200: NaN in every row
+    As[1, 9] = np.inf       # row 9, second slice: infinite partial sums (NaN where that slice's sum is zero)
+    As[2, 11] = -np.inf
+    As[0, 13] = 1e38        # row 13: some sums overflow to infinity, their neighbours in the same 1x128 group stay finite
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    assert np.isnan(ref[3]).all() and np.isnan(ref[:, 200]).all() and np.isinf(ref[9]).any()
+    assert np.isinf(ref[13, :128]).any() and np.isfinite(ref[13, :128]).any()
+    C, Cb, Cq, Cs = _run_all(lib, Aq, As, Bq, Bs, tile=tile if skinny else TILES[tile], split_k=split)
+    what = "tile %s split %d" % (tile, split)
+    assert (np.isnan(C) == np.isnan(ref)).all(), what + ": NaN pattern differs from the oracle's"
+    inf = np.isinf(ref)
+    assert (np.isinf(C) == inf).all() and (np.sign(C[inf]) == np.sign(ref[inf])).all(), what + ": infinities differ"
+    fin = np.isfinite(ref)
+    assert_fp8_gemm_close(np.where(fin, C, 0), np.where(fin, ref, 0), what)
+    assert (Cb == oracle.f32_to_bf16_bits(C))[fin].all()
+    oq, os_ = oracle.requant_c_1x128(C)
+    assert (Cq == oq).all(), what + ": fused codes differ from requant(own fp32) at %s" % np.argwhere(Cq != oq)[:5].tolist()
+    assert (Cs.view(np.uint32) == os_.view(np.uint32)).all()
+    assert (Cq[3] == 0x7F).all() and (Cq[:, 200] == 0x7F).all()

@@ -122,3 +122,36 @@ def test_quotients_on_rounding_boundaries(lib, oracle):
         q2, s2 = lib.rmsnorm_quantize_activation(torch.from_numpy(xx).cuda(), torch.from_numpy(w).cuda(), 1e-6)
         torch.cuda.synchronize()
         assert (q2.cpu().numpy() == rq2).all() and (s2.cpu().numpy().view(np.uint32) == rs2.view(np.uint32)).all()
+
+
+def test_non_finite_values_follow_the_reference(lib, oracle):
+    """NaN and infinities through every quantiser layout, bit for bit against the oracle's restatement of the reference's
+    arithmetic (examples/005.fp8.mm.cu:456, :474-485): a NaN never enters the block maximum and its code is 0x7F
+    whatever its sign; an infinity makes the scale infinite, so finite elements become signed zeros and the infinite
+    ones inf / inf = NaN -> 0x7F; a block that holds nothing but NaN keeps the maximum's seed (float)INT_MIN."""
+    rng = np.random.default_rng(5)
+    x = rng.normal(0, 1, (256, 384)).astype(np.float32)
+    nan = np.array([0x7FC00000, 0xFFC00000, 0x7F800001, 0xFF800001, 0x7FFFFFFF], np.uint32).view(np.float32)
+    x[0, :5] = nan                      # NaNs of both signs, quiet and signalling, among ordinary values
+    x[1, 7] = np.inf                    # an infinite maximum
+    x[1, 9] = -np.inf
+    x[1, 11] = nan[1]
+    x[2, 128:256] = nan[0]              # a 1x128 block of nothing but NaN
+    x[3, 130] = -np.inf
+    x[3, 131] = -3.0
+    x[128:256, 256:384] = nan[1]        # a 128x128 block of nothing but NaN
+    x[130, 0] = 3e38                    # near the largest finite value: scale stays finite
+    x[131, 1] = 1e-45                   # the smallest subnormal beside ordinary values
+    for quant_m, transpose in ((1, True), (1, False), (128, False), (128, True)):
+        rq, rs = oracle.quant_fp8(x, quant_m, transpose)
+        q, s = _run(lib, x, quant_m, transpose, rs.shape)
+        bad = np.argwhere(q != rq)
+        assert bad.size == 0, "quant_m %d transpose %s: codes differ at %s (got %s, oracle %s)" % (
+            quant_m, transpose, bad[:5].tolist(), q[tuple(bad[:5].T)], rq[tuple(bad[:5].T)])
+        if quant_m == 128 and transpose:
+            assert (s[:, :2].view(np.uint32) == rs[:, :2].view(np.uint32)).all()
+        else:
+            assert (s.view(np.uint32) == rs.view(np.uint32)).all()
+    rq, rs = oracle.quant_fp8(x, 1, True)
+    assert rq[0, 0] == 0x7F and rq[0, 1] == 0x7F and rq[1, 7] == 0x7F and rq[1, 9] == 0x7F and rq[1, 0] in (0, 0x80)
+    assert rs[1, 2] < 0 and (rq[2, 128:256] == 0x7F).all()
