@@ -84,7 +84,7 @@ typedef struct llmmm_gemm_cfg {
   int tile;
   int split_k;
   int b_layout; /* FP8 only: LLMMM_FP8_B_ROWS (0, the default) or LLMMM_FP8_B_PRESHUFFLED; the FP16 GEMM ignores it */
-  int a_layout; /* FP8 only: LLMMM_FP8_A_QUANTISED (0, the default) or LLMMM_FP8_A_SWIGLU_F32 */
+  int a_layout; /* FP8 only: LLMMM_FP8_A_QUANTISED (0, the default), LLMMM_FP8_A_SWIGLU_F32 or LLMMM_FP8_A_PLANES_RMSNORM */
 } llmmm_gemm_cfg;
 
 /* ---- FP16 / BF16 GEMM -------------------------------------------------------------------
@@ -222,7 +222,7 @@ LLMMM_API size_t llmmm_fp8_swiglu_a_workspace(int M, int N, int K);
  * cfg.a_layout = LLMMM_FP8_A_PLANES_RMSNORM and a llmmm_a_planes_rmsnorm in place of A (As ignored; K of that call = N of
  * the planes), and runs on
  *   h = sum of the planes in split order + residual;  hidden_out = hidden_dtype(h);  A = quantise_1x128(rmsnorm(hidden_out) * w)
- * -- exactly the hidden state, codes and scales llmmm_fp8_gemm_add_rmsnorm_quant delivers, bit for bit.  For M <= 4 and
+ * -- exactly the hidden state, codes and scales llmmm_fp8_gemm_add_rmsnorm_quant delivers, bit for bit.  For M <= 2 and
  * K <= 3072 every workgroup of the weight-streaming kernel makes the operand itself while its first weights are in flight
  * (no reduce kernel, no norm kernel: one launch per projection), provided hidden_out is a buffer of its own, not the
  * residual, and there are at most 10 planes.  Otherwise the library runs the fused reduce + norm + quantise kernel into the

@@ -411,7 +411,9 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
   if (!A || (!As && !a_made) || !Bt || !Bs || !C) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
   if (a_swiglu && swiglu) return fail(LLMMM_ERR_INVALID_ARGUMENT, "SwiGLU on both the A operand and the output");
   if ((out_kind == LLMMM_OUT_FP8Q || swiglu) && !Cs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "C_scale_transposed is required for fp8 output");
-  if (!aligned16(A) || !aligned16(Bt) || !aligned16(C)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+  // (with a_layout = PLANES_RMSNORM, A is a host structure: prepare_a checks the device pointers inside it)
+  const bool a_host = user && user->a_layout == LLMMM_FP8_A_PLANES_RMSNORM;
+  if ((!a_host && !aligned16(A)) || !aligned16(Bt) || !aligned16(C)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
   if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
   if (user) {
@@ -569,14 +571,23 @@ int llmmm_probe_hbm_read(const void* src, size_t bytes, float* sink, int workgro
   return LLMMM_OK;
 }
 
-size_t llmmm_fp8_gemm_add_rmsnorm_quant_workspace(int M, int N, int K)
+// Workspace of the entry points whose epilogue runs either inside an unsplit tile kernel (no planes) or in a second
+// kernel behind fp32 planes: the same decision as resolve_plane_cfg takes for a call without cfg.  A single tile row of
+// fewer than 128 rows (64 < M < 128 in 128 x 128 tiles) has no epilogue of its own and always goes through one plane.
+static size_t plane_route_workspace(int M, int N, int K, bool wide_ok)
 {
   if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
   llmmm_gemm_cfg cfg;
   if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
-  if (cfg.tile != LLMMM_TILE_SKINNY && cfg.split_k <= 1) return 0;  // residual added inside the tile kernel
-  return (size_t)(cfg.split_k < 1 ? 1 : cfg.split_k) * M * N * sizeof(float);
+  if (wide_ok) prefer_wide_tile(&cfg, M, N);
+  int split = cfg.split_k < 1 ? 1 : cfg.split_k;
+  if (split > max_split_for(K)) split = max_split_for(K);
+  int bm = 0, bn = 0;
+  if (cfg.tile != LLMMM_TILE_SKINNY && tile_dims(cfg.tile, bm, bn) && M % bm == 0 && split == 1) return 0;  // epilogue inside the tile kernel
+  return (size_t)split * M * N * sizeof(float);
 }
+
+size_t llmmm_fp8_gemm_add_rmsnorm_quant_workspace(int M, int N, int K) { return plane_route_workspace(M, N, K, true); }
 
 // Kernel and split for the entry points whose epilogue lives in a second kernel behind fp32 planes, chosen and
 // validated as llmmm_fp8_gemm_ex does.  split == 0 on return: a tile kernel without split, which `allow_direct`
@@ -596,7 +607,8 @@ static int resolve_plane_cfg(const void*& A, const float*& As, const void* Bt, c
   if (wide_ok) prefer_wide_tile(&cfg, M, N);
   const bool a_made = user && user->a_layout != LLMMM_FP8_A_QUANTISED;
   if (!A || (!As && !a_made) || !Bt || !Bs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
-  if (!aligned16(A) || !aligned16(Bt)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+  const bool a_host = user && user->a_layout == LLMMM_FP8_A_PLANES_RMSNORM;  // a host structure, checked by prepare_a
+  if ((!a_host && !aligned16(A)) || !aligned16(Bt)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
   if ((long)M * K >= (1L << 31) || (long)N * K >= (1L << 31) || (long)M * N >= (1L << 31))
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
   if (user) {
@@ -736,14 +748,7 @@ int llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As, const void*
   return LLMMM_OK;
 }
 
-size_t llmmm_fp8_gemm_qkv_rope_workspace(int M, int N, int K)
-{
-  if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
-  llmmm_gemm_cfg cfg;
-  if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
-  if (cfg.tile != LLMMM_TILE_SKINNY && cfg.split_k <= 1) return 0;  // epilogue inside the tile kernel
-  return (size_t)(cfg.split_k < 1 ? 1 : cfg.split_k) * M * N * sizeof(float);
-}
+size_t llmmm_fp8_gemm_qkv_rope_workspace(int M, int N, int K) { return plane_route_workspace(M, N, K, false); }
 
 int llmmm_fp8_gemm_qkv_rope(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* out, float* out_scale,
                             const float* q_norm_weight, const float* k_norm_weight, float eps, const float* cos_table, const float* sin_table,

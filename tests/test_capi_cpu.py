@@ -332,3 +332,63 @@ def test_probe_validation_without_device():
     assert lib.llmmm_probe_mfma_flops(0, 256, 10) == 256 * 8 * 10 * 16 * 16384.0
     assert lib.llmmm_probe_mfma_flops(_lib.PROBE_FP8, 256, 10) == 256 * 8 * 10 * 8 * 65536.0
     assert lib.llmmm_probe_mfma_flops(9, 256, 10) == 0.0
+
+
+def _no_gpu_here():
+    import torch
+    return not torch.cuda.is_available()
+
+
+@pytest.mark.skipif(not _no_gpu_here(), reason="passes validation with made-up pointers: only where no device can be reached")
+@pytest.mark.parametrize("N,K", [(2560, 4096), (19456, 2560), (10240, 2048), (6144, 2560), (4096, 14336)])
+@pytest.mark.parametrize("M", [1, 16, 65, 96, 127, 128, 256, 2048])
+def test_queried_workspace_is_accepted_by_the_fused_entry_points(M, N, K):
+    """The size a *_workspace query returns must pass the workspace checks of its call, row tails included (64 < M < 128
+    routed to an unsplit 128 x 128 tile has no epilogue of its own and needs one fp32 plane).  Without a device the call
+    gets as far as the launch (LLMMM_ERR_RUNTIME); a workspace complaint would come before that."""
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    eps = ctypes.c_float(1e-6)
+    if N <= 10240:
+        need = lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K)
+        ws = FAKE if need else None
+        rc = lib.llmmm_fp8_gemm_add_rmsnorm_quant(FAKE, FAKE, FAKE, FAKE, _lib.DTYPE_BF16, FAKE, FAKE, FAKE, eps, FAKE, FAKE, M, N, K, ws, need, None, None)
+        assert rc == _lib.ERR_RUNTIME, lib.llmmm_last_error()
+    heads = N // 128
+    if heads >= 3 and (heads - 2) % 1 == 0:
+        nkv = 1 if heads < 12 else 8
+        nq = heads - 2 * nkv
+        need = lib.llmmm_fp8_gemm_qkv_rope_workspace(M, N, K)
+        ws = FAKE if need else None
+        rc = lib.llmmm_fp8_gemm_qkv_rope(_lib.OUT_BF16, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, eps, FAKE, FAKE, 64, FAKE, nq, nkv, M, N, K,
+                                         ws, need, None, None)
+        assert rc == _lib.ERR_RUNTIME, lib.llmmm_last_error()
+
+
+def test_planes_rmsnorm_descriptor_needs_no_16_byte_alignment():
+    """The A argument of cfg.a_layout = PLANES_RMSNORM is a host structure of pointer alignment (8): one at an address
+    that is 8 modulo 16 is as good as any.  The device pointers inside it are still checked."""
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    buf = (ctypes.c_char * (ctypes.sizeof(_lib.APlanesRmsnorm) + 32))()
+    base = ctypes.addressof(buf)
+    addr = base + ((8 - base) % 16)
+    assert addr % 16 == 8
+    d = _lib.APlanesRmsnorm.from_address(addr)
+    d.planes, d.splits, d.hidden_dtype, d.residual, d.hidden_out, d.norm_weight, d.eps = 0x1000, 8, _lib.DTYPE_BF16, 0x2000, 0x3000, 0x4000, 1e-6
+    cfg = _lib.GemmCfg(_lib.TILE_SKINNY, 0, 0, _lib.FP8_A_PLANES_RMSNORM)
+    M, N, K = 1, 6144, 2560
+
+    def call():
+        return lib.llmmm_fp8_gemm_ex(_lib.OUT_F32, ctypes.c_void_p(addr), None, FAKE, FAKE, FAKE, None, M, N, K, None, 0, ctypes.byref(cfg), None)
+
+    d.residual = 0x2004  # a misaligned device pointer inside the descriptor is still refused ...
+    assert call() == _lib.ERR_INVALID_ARGUMENT and b"16-byte aligned" in lib.llmmm_last_error()
+    d.residual = 0x2000
+    d.splits = 0         # ... and so is a bad field, which shows that validation went past the alignment of A itself
+    assert call() == _lib.ERR_INVALID_ARGUMENT and b"splits" in lib.llmmm_last_error()
+    # the fused entry points take the same route
+    d.splits = 99
+    rc = lib.llmmm_fp8_gemm_qkv_rope(_lib.OUT_BF16, ctypes.c_void_p(addr), None, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, ctypes.c_float(1e-6), FAKE, FAKE, 64, FAKE,
+                                     32, 8, M, N, K, FAKE, 1 << 20, ctypes.byref(cfg), None)
+    assert rc == _lib.ERR_INVALID_ARGUMENT and b"splits" in lib.llmmm_last_error()

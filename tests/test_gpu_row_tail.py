@@ -112,3 +112,56 @@ def test_untuned_shapes_between_64_and_128_rows(lib, oracle):
     # the two routes split K differently (fp32 sums in another order): codes may differ by one step where a value sits on a boundary
     same = (H == Hr).float().mean().item()
     assert same > 0.999 and torch.allclose(Hs, Hsr, rtol=1e-3)
+
+
+@pytest.mark.parametrize("M", [65, 96, 127])
+@pytest.mark.parametrize("N,K", [(2560, 9728), (10240, 2048)])
+def test_add_rmsnorm_quant_on_tail_rows_with_the_queried_workspace(lib, oracle, M, N, K):
+    """The residual + RMSNorm + quantiser entry point on a row tail, tuned (down projection: split tiles) and untuned
+    (one unsplit row of 128 x 128 tiles, which has no epilogue of its own and needs one plane), with exactly the
+    workspace its query function asks for: hidden == T(C32 + residual), codes and scales == the oracle's on that."""
+    from llmmm_amd import _lib
+    assert lib.query_config(_lib.OUT_F32, M, N, K)[0] == T128
+    need = _lib.lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K)
+    assert need >= M * N * 4
+    Aq, As, Bq, Bs = _inputs(oracle, M, N, K, 5)
+    rng = np.random.default_rng(M)
+    res = (rng.standard_normal((M, N)) * 2).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, N).astype(np.float32)
+    dA, dAs, dB, dBs = (torch.from_numpy(a).cuda() for a in (Aq, As, Bq, Bs))
+    C = torch.empty((M, N), device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dA, dAs, dB, dBs, C, M, N, K, workspace=lib.make_workspace(_lib.OUT_F32, M, N, K))
+    tres = torch.from_numpy(res).cuda().to(torch.bfloat16)
+    hidden = torch.full((M + 2, N), 7.0, dtype=torch.bfloat16, device="cuda")
+    ws = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")
+    q, s = lib.fp8_gemm_add_rmsnorm_quant(dA, dAs, dB, dBs, tres, hidden[:M], torch.from_numpy(w).cuda(), 1e-6, M, N, K, workspace=ws)
+    torch.cuda.synchronize()
+    want = torch.from_numpy(C.cpu().numpy() + tres.float().cpu().numpy()).to(torch.bfloat16)
+    assert torch.equal(hidden[:M].cpu().view(torch.int16), want.view(torch.int16)) and (hidden[M:] == 7.0).all()
+    rq, rs = oracle.rmsnorm_quant(want.float().numpy(), w, 1e-6)
+    assert np.array_equal(q.cpu().numpy(), rq) and np.array_equal(s.cpu().numpy().view(np.uint32), rs.view(np.uint32))
+
+
+@pytest.mark.parametrize("M", [65, 127])
+@pytest.mark.parametrize("n_q,n_kv,K", [(136, 8, 2560), (48, 8, 2560)])
+def test_qkv_rope_on_tail_rows_with_the_queried_workspace(lib, oracle, M, n_q, n_kv, K):
+    from llmmm_amd import _lib
+    N = (n_q + 2 * n_kv) * 128
+    assert lib.query_config(_lib.OUT_F32, M, N, K)[0] == T128
+    need = _lib.lib.llmmm_fp8_gemm_qkv_rope_workspace(M, N, K)
+    assert need >= M * N * 4
+    Aq, As, Bq, Bs = _inputs(oracle, M, N, K, 7)
+    rng = np.random.default_rng(M + N)
+    qw, kw = (rng.uniform(0.5, 1.5, 128).astype(np.float32) for _ in range(2))
+    ang = np.arange(512, dtype=np.float64)[:, None] * (1e6 ** (-np.arange(64) / 64.0))[None, :]
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    pos = rng.integers(0, 512, M).astype(np.int32)
+    g = lambda a: torch.from_numpy(a).cuda()
+    dA, dAs, dB, dBs = g(Aq), g(As), g(Bq), g(Bs)
+    C = torch.empty((M, N), device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dA, dAs, dB, dBs, C, M, N, K, workspace=lib.make_workspace(_lib.OUT_F32, M, N, K))
+    ws = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")
+    out = lib.fp8_gemm_qkv_rope(dA, dAs, dB, dBs, g(qw), g(kw), 1e-6, g(cos), g(sin), g(pos), n_q, n_kv, M, N, K, workspace=ws)
+    torch.cuda.synchronize()
+    want = oracle.qk_norm_rope(C.cpu().numpy(), qw, kw, 1e-6, cos, sin, pos, n_q, n_kv)
+    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), oracle.f32_to_bf16_bits(want))
