@@ -37,11 +37,17 @@ MEASURED_TRAFFIC_BYTES = {"fp16_gemm_4096": 235.0e6, "fp8_gemm_fused_4096": 119.
 QWEN3_4B = {"qkv": (6144, 2560), "o": (2560, 4096), "gate_up": (19456, 2560), "down": (2560, 9728)}
 
 
+TIMED_BATCHES = 7      # batches of `steps` launches timed one after the other; the median is reported
+SETTLE_S = 0.06        # untimed replays of a captured graph before the timed ones (the clocks drop during capture)
+LAST_SPREAD = {}       # min / max over the timed batches of the most recent _events_ms call, ms per step
+
+
 def _events_ms(fn, steps, warmup, graph=False):
-    """Average duration of one call of fn, HIP events on torch's current stream (the stream
-    every launch below is enqueued on).  With graph=True (every GEMM workload) the `steps` launches
-    are captured into one HIP graph and replayed once inside the timed region, so that kernels are
-    timed back-to-back on the GPU instead of at the pace of the Python launch loop."""
+    """Duration of one call of fn: the median over TIMED_BATCHES batches of `steps` calls, each batch bracketed by HIP
+    events on torch's current stream (the stream every launch below is enqueued on); the batches are enqueued back to
+    back with no host synchronisation between them, so the GPU never idles inside the timed region.  With graph=True
+    (every GEMM workload) a batch is one replay of a HIP graph of `steps` launches, so that kernels are timed back to
+    back on the GPU instead of at the pace of the Python launch loop."""
     # Untimed pre-heat: the GPU's clocks take tens of milliseconds of sustained load to settle, far
     # longer than a handful of warm-up launches of a ~100 us kernel; time the settled state.
     t_heat = time.perf_counter()
@@ -52,30 +58,34 @@ def _events_ms(fn, steps, warmup, graph=False):
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(TIMED_BATCHES)]
     if graph:
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             for _ in range(steps):
                 fn()
-        for _ in range(3):  # untimed replays: graph upload, and the clocks back up after the idle capture
+        t_settle, n = time.perf_counter(), 0
+        while n < 3 or time.perf_counter() - t_settle < SETTLE_S:  # graph upload, and the clocks back up after the idle capture
             g.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        e0.record()
-        g.replay()
-        e1.record()
-        torch.cuda.synchronize()
+            n += 1
+            if n % 8 == 0:
+                torch.cuda.synchronize()
+        batch = g.replay
     else:
-        t0 = time.perf_counter()
+        def batch():
+            for _ in range(steps):
+                fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for e0, e1 in ev:
         e0.record()
-        for _ in range(steps):
-            fn()
+        batch()
         e1.record()
-        torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    return e0.elapsed_time(e1) / steps, wall_ms / steps
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / TIMED_BATCHES
+    per = sorted(e0.elapsed_time(e1) / steps for e0, e1 in ev)
+    LAST_SPREAD.update(min=per[0], max=per[-1])
+    return per[len(per) // 2], wall_ms / steps
 
 
 def sample_clock_power(step, seconds=1.2):
@@ -161,7 +171,8 @@ def bench_fp16(M, N, K, steps, warmup, dtype=torch.float16, b_transposed=False, 
     C = torch.empty((M, N), dtype=dtype, device="cuda")
     ms, wall = _events_ms(lambda: llmmm_amd.fp16_gemm(A, B, C, b_transposed=b_transposed), steps, warmup, graph=True)
     flops = 2.0 * M * N * K
-    r = {"ms": ms, "wall_ms": wall, "tflops": flops / ms * 1e-9, "bytes": 2.0 * (M * K + K * N + M * N)}
+    r = {"ms": ms, "wall_ms": wall, "tflops": flops / ms * 1e-9, "bytes": 2.0 * (M * K + K * N + M * N), "ms_min": LAST_SPREAD.get("min"),
+         "ms_max": LAST_SPREAD.get("max")}
     if clock:
         r["clock"] = sample_clock_power(lambda: llmmm_amd.fp16_gemm(A, B, C, b_transposed=b_transposed))
     return r, (A, B, C)
@@ -218,8 +229,10 @@ def bench_fp8(M, N, K, out, steps, warmup, rotate_bytes=0, preshuffled=False, cl
     flops = 2.0 * M * N * K
     nbytes = fp8_bytes(M, N, K, out)
     tile, split = llmmm_amd.query_config(kind, M, N, K)
+    kernel = ("fp8_skinny_kernel split_k=%d%s" % (split, " + fp8_splitk_reduce_kernel" if split > 1 else "")) if tile == _lib.TILE_SKINNY else \
+        "fp8_gemm_kernel tile %d split_k %d" % (tile, split)
     r = {"ms": ms, "wall_ms": wall, "tflops": flops / ms * 1e-9, "gbs": nbytes / ms * 1e-6, "bytes": nbytes, "tile": tile,
-         "split_k": split, "weight_copies": copies}
+         "split_k": split, "weight_copies": copies, "kernel": kernel, "ms_min": LAST_SPREAD.get("min"), "ms_max": LAST_SPREAD.get("max")}
     if clock:
         r["clock"] = sample_clock_power(step)
     return r
@@ -457,8 +470,67 @@ def measured_peaks():
     return out
 
 
-def cpu_baseline_fp16(M, N, K, rows):
-    """Oracle Kahan GEMM on the first `rows` rows of the headline workload, all host threads."""
+def bench_read_ceiling(nbytes_per_copy, workgroups, steps, warmup, rotate_bytes=768 << 20):
+    """A bare streaming read (llmmm_probe_hbm_read: nothing computed, nothing written) of as many bytes as one launch of a
+    decode GEMM reads weights, by as many workgroups of the same size, over rotating buffers, timed exactly like the GEMM:
+    the time below which no kernel of that launch shape can get on this part."""
+    from llmmm_amd import _lib
+    nbytes = int(nbytes_per_copy) // 16 * 16
+    copies = max(2, int(np.ceil(rotate_bytes / float(nbytes))))
+    bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(0, 255) for _ in range(copies)]
+    sink = torch.zeros(4, device="cuda")
+    state = {"i": 0}
+
+    def step():
+        b = bufs[state["i"] % copies]
+        state["i"] += 1
+        assert _lib.lib.llmmm_probe_hbm_read(b.data_ptr(), nbytes, sink.data_ptr(), workgroups, torch.cuda.current_stream().cuda_stream) == 0
+
+    ms, _ = _events_ms(step, steps, warmup, graph=True)
+    return ms
+
+
+def bench_targets(steps, warmup, headline=None):
+    """The three figures the metric names, each against its published peak: FP16 GEMM and FP8 fused GEMM at 4096^3 (MFMA),
+    and the four Qwen3-4B projections at M = 1 and 16 with fused C quantisation (HBM; weights rotated over more copies than
+    the caches hold).  The decode rows also carry the time of a bare read of the same weight bytes by the same number of
+    workgroups (read_us) and the fraction of that ceiling the GEMM reaches."""
+    import llmmm_amd
+    from llmmm_amd import _lib
+    t = {}
+    if headline is None:
+        x, _ = bench_fp16(4096, 4096, 4096, steps, warmup)
+        headline = x
+    t["fp16_4096"] = {"us": round(headline["ms"] * 1e3, 2), "tflops": round(headline["tflops"], 1), "frac": round(headline["tflops"] / PEAK_TFLOPS["f16"], 4),
+                      "target": 0.75, "kernel": "fp16_gemm_kernel<f16,256,256>"}
+    x = bench_fp8(4096, 4096, 4096, "fp8q", steps, warmup)
+    t["fp8_fused_4096"] = {"us": round(x["ms"] * 1e3, 2), "tflops": round(x["tflops"], 1), "frac": round(x["tflops"] / PEAK_TFLOPS["fp8"], 4),
+                           "target": 0.70, "kernel": "fp8_gemm_kernel<256,256,fp8q>"}
+    dsteps = max(steps, 200)  # microsecond kernels: enough launches per batch for the event clock
+    for name, (n, k) in QWEN3_4B.items():
+        read_ms = {}
+        for m in (1, 16):
+            for pre in (False, True):
+                x = bench_fp8(m, n, k, "fp8q", dsteps, warmup, rotate_bytes=768 << 20, preshuffled=pre)
+                split = max(1, x["split_k"])
+                wgs = (n // 128) * split
+                if wgs not in read_ms:
+                    read_ms[wgs] = bench_read_ceiling(n * k, wgs, dsteps, warmup)
+                e = {"us": round(x["ms"] * 1e3, 2), "gbs": round(x["gbs"], 1), "frac": round(x["gbs"] / PEAK_HBM_GBS, 4), "target": 0.60,
+                     "kernel": x["kernel"], "read_us": round(read_ms[wgs] * 1e3, 2),
+                     "frac_of_read_ceiling": round(read_ms[wgs] / x["ms"], 4)}
+                t["decode_%s_m%d%s" % (name, m, "_pre" if pre else "")] = e
+            torch.cuda.empty_cache()
+    t["note"] = ("us = median of %d batches; frac = achieved / published peak (2500 TFLOP/s f16, 5000 fp8, 8000 GB/s); decode: algorithmic bytes of the "
+                 "fused-quant GEMM / us, _pre = weights pre-shuffled offline; read_us = bare read of the same weight bytes by the same workgroup count" % TIMED_BATCHES)
+    return t
+
+
+def cpu_baseline(M, N, K, rows):
+    """The CPU oracle on this host's cores, bounded samples of the GPU workloads: the Kahan GEMM (the headline's
+    reference, a port of test/kahan.cu:16-26) on the first `rows` rows of the FP16 workload, and beside it the
+    double-accumulate loop (test/kahan.cu:48-55) and the blockwise FP8 GEMM + fused re-quantisation
+    (examples/005.fp8.mm.cu:885-902, examples/005.fp8.mm.opt.cu:401-462) on a 256-row slab of the 4096^3 FP8 workload."""
     import oracle
     rng = np.random.default_rng(2)
     A = rng.standard_normal((rows, K), dtype=np.float32).astype(np.float16).astype(np.float32)
@@ -467,9 +539,30 @@ def cpu_baseline_fp16(M, N, K, rows):
     t0 = time.perf_counter()
     oracle.kahan_gemm(A, B)
     dt = time.perf_counter() - t0
-    return {"value": 2.0 * rows * N * K / dt * 1e-12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
-            "sample": "oracle Kahan fp32 GEMM (port of test/kahan.cu:16-26) on the first %d of %d rows of the same "
-                      "M=N=K=4096 fp16 workload, %.1f s" % (rows, M, dt)}
+    out = {"value": 2.0 * rows * N * K / dt * 1e-12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+           "sample": "oracle Kahan fp32 GEMM (port of test/kahan.cu:16-26) on the first %d of %d rows of the same "
+                     "M=N=K=4096 fp16 workload, %.1f s" % (rows, M, dt)}
+    drows = min(rows, 1024)
+    t0 = time.perf_counter()
+    oracle.double_gemm(A[:drows], B)
+    dt2 = time.perf_counter() - t0
+    srows = 256
+    X = rng.standard_normal((srows, K), dtype=np.float32)
+    X[:, rng.choice(K, max(1, -(-K // 100)), replace=False)] *= np.float32(20.0)
+    W = rng.standard_normal((N, K), dtype=np.float32) * np.float32(0.02)
+    Aq, As = oracle.quant_fp8(X, 1, True)
+    Bq, Bs = oracle.quant_fp8(W, 128, False)
+    t0 = time.perf_counter()
+    oracle.requant_c_1x128(oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128))
+    dt3 = time.perf_counter() - t0
+    out["others"] = [
+        {"name": "double_accumulate_gemm", "value": 2.0 * drows * N * K / dt2 * 1e-12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+         "sample": "oracle double-accumulate GEMM (port of test/kahan.cu:48-55) on the first %d rows of the same workload, %.1f s" % (drows, dt2)},
+        {"name": "fp8_blockwise_gemm_fused_quant", "value": 2.0 * srows * N * K / dt3 * 1e-12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+         "sample": "oracle FP8 blockwise GEMM (per-128 promotion) + 1x128 re-quantisation of C on a %d-row slab of the M=N=K=4096 FP8 workload "
+                   "(A ~ N(0,1) with 1%% outlier channels, B ~ N(0,0.02)), %.1f s" % (srows, dt3)},
+    ]
+    return out
 
 
 def main():
@@ -484,6 +577,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measured-peak probes")
+    ap.add_argument("--no-targets", action="store_true", help="skip the compact table of the metric's three figures")
     ap.add_argument("--cpu-rows", type=int, default=4096)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -624,13 +718,15 @@ def main():
     line = {
         "metric": "TFLOPS (% of MI355X FP8/FP16 MFMA peak) at 4096\u00b3; HBM GB/s at M\u226416 decode",
         "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms"],
-        "wall_ms_per_step": r["wall_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
+        "wall_ms_per_step": r["wall_ms"], "timing": "median of %d batches of `steps` launches (one HIP-graph replay each), events per batch; min %.5f max %.5f ms per step"
+        % (TIMED_BATCHES, r.get("ms_min") or r["ms"], r.get("ms_max") or r["ms"]), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
         "data": "synthetic", "config": cfg, "roofline": roof,
     }
 
     if not args.no_shapes:
         shapes = []
         s2, w2 = max(10, args.steps // 2), max(3, args.warmup // 2)
+        sd = max(2 * s2, 100)  # launches per batch for the microsecond-scale kernels (M <= 128)
         if w != "fp16_gemm_4096":
             x, _ = bench_fp16(4096, 4096, 4096, s2, w2)
             shapes.append({"name": "fp16_gemm_4096", "ms": x["ms"], "tflops": x["tflops"], "frac_of_fp16_peak": x["tflops"] / PEAK_TFLOPS["f16"]})
@@ -645,7 +741,7 @@ def main():
             shapes.append({"name": "fp8_gemm_4096_" + out, "ms": x["ms"], "tflops": x["tflops"], "frac_of_fp8_peak": x["tflops"] / PEAK_TFLOPS["fp8"]})
         for name, (n, k) in QWEN3_4B.items():
             for m, pre in ((1, False), (1, True), (16, False), (16, True), (128, False), (128, True), (2048, False), (2048, True)):
-                x = bench_fp8(m, n, k, "fp8q", s2 * 2 if m <= 16 else s2, w2, rotate_bytes=(768 << 20) if m <= 128 else 0, preshuffled=pre)
+                x = bench_fp8(m, n, k, "fp8q", sd if m <= 128 else s2, w2, rotate_bytes=(768 << 20) if m <= 128 else 0, preshuffled=pre)
                 e = {"name": "qwen3_4b_%s_m%d%s" % (name, m, "_preshuffled" if pre else ""), "M": m, "N": n, "K": k, "us": x["ms"] * 1e3, "tflops": x["tflops"],
                      "frac_of_fp8_peak": x["tflops"] / PEAK_TFLOPS["fp8"], "tile": x["tile"], "split_k": x["split_k"]}
                 if m <= 128:
@@ -653,14 +749,14 @@ def main():
                 if m <= 16 and pre:
                     # the same launch on one weight copy: served from the L2 / memory-side cache instead of HBM ("hot" next to the
                     # "cold" figure above, which rotates over more copies than the caches hold)
-                    xh = bench_fp8(m, n, k, "fp8q", s2 * 2, w2, rotate_bytes=0, preshuffled=True)
+                    xh = bench_fp8(m, n, k, "fp8q", sd, w2, rotate_bytes=0, preshuffled=True)
                     e["us_hot_cache"] = xh["ms"] * 1e3
                 shapes.append(e)
                 torch.cuda.empty_cache()
         # the gate_up projection with the SwiGLU activation fused in front of the C quantisation (output N/2 wide)
         n, k = QWEN3_4B["gate_up"]
         for m in (1, 16, 128, 2048):
-            x = bench_fp8(m, n, k, "swiglu", s2 * 2 if m <= 16 else s2, w2, rotate_bytes=(768 << 20) if m <= 128 else 0)
+            x = bench_fp8(m, n, k, "swiglu", sd if m <= 128 else s2, w2, rotate_bytes=(768 << 20) if m <= 128 else 0)
             e = {"name": "qwen3_4b_gate_up_swiglu_m%d" % m, "M": m, "N": n, "K": k, "us": x["ms"] * 1e3, "tflops": x["tflops"],
                  "frac_of_fp8_peak": x["tflops"] / PEAK_TFLOPS["fp8"], "tile": x["tile"], "split_k": x["split_k"]}
             if m <= 128:
@@ -686,20 +782,20 @@ def main():
         # One decoder MLP block as three launches: RMSNorm+quant -> gate_up GEMM with fused SwiGLU output -> down GEMM
         # (bf16 output), weights pre-shuffled and rotated over distinct copies so that they stream from HBM.
         for m in (1, 16):
-            shapes.append(bench_mlp_chain(m, s2, w2))
+            shapes.append(bench_mlp_chain(m, sd, w2))
             torch.cuda.empty_cache()
         # o / down projection + residual add + next RMSNorm + quantisation in one entry point, beside the same work as separate launches
         for name in ("o", "down"):
             for m in (1, 16, 128, 2048):
-                shapes.append(bench_proj_add_norm(name, m, s2 * 2 if m <= 16 else s2, w2))
+                shapes.append(bench_proj_add_norm(name, m, sd if m <= 128 else s2, w2))
                 torch.cuda.empty_cache()
         # QKV projection + per-head RMSNorm + RoPE in one entry point, beside the plain bf16-output GEMM
         for m in (1, 16, 128, 2048):
-            shapes.append(bench_qkv_rope(m, s2 * 2 if m <= 16 else s2, w2))
+            shapes.append(bench_qkv_rope(m, sd if m <= 128 else s2, w2))
             torch.cuda.empty_cache()
         # the GEMM side of a whole decoder layer through the four fused entry points
         for m, cs in ((1, False), (1, True), (2, True), (16, False)):
-            shapes.append(bench_decoder_layer(m, s2, w2, consumer_side=cs))
+            shapes.append(bench_decoder_layer(m, sd, w2, consumer_side=cs))
             torch.cuda.empty_cache()
         line["shapes"] = shapes
 
@@ -745,9 +841,14 @@ def main():
         roof["peak_measured"] = mp["hbm_read_1gib_gbs"] if roof["bound"] == "hbm" else mp[key]
         roof["frac_of_measured"] = roof["achieved"] / roof["peak_measured"]
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline_fp16(4096, 4096, 4096, args.cpu_rows)
+        line["cpu_baseline"] = cpu_baseline(4096, 4096, 4096, args.cpu_rows)
     else:
         line["cpu_baseline"] = None
+    if not args.no_targets:
+        # last key of the line, and inside `roofline` as well: all three figures of the metric in one place
+        tg = bench_targets(max(20, args.steps), max(3, args.warmup), headline=r if w == "fp16_gemm_4096" else None)
+        roof["targets"] = tg
+        line["targets"] = tg
     print(json.dumps(line))
 
 
