@@ -14,11 +14,11 @@
 // reference's rule M % 128 == 0, N % 128 == 0, K % 128 == 0 (examples/005.fp8.mm.cu:2490-2492) and
 // additionally accept 1 <= M <= 128 (decode), which the reference does not cover.  The reference
 // signatures have no workspace argument, so the split-K scratch of the small-M shapes comes from a
-// buffer these shims keep per host thread and stream (detail8::cached_workspace: allocated with
-// hipMalloc on first need, grown when a later call needs more, kept until the process ends).  Calls
+// buffer kept per host thread and stream: the caller's, handed over once with LLMMM::set_fp8_workspace
+// (then nothing here allocates or waits, as in the reference), or else one the shim allocates with
+// hipMalloc on first need, grows when a later call needs more and frees when the thread ends.  Calls
 // on one stream are ordered, so one buffer per stream is race-free; a call that has to allocate must
-// not happen inside a stream capture -- run each shape once before capturing, or use llmmm_fp8_gemm()
-// with a workspace of your own.
+// not happen inside a stream capture -- set a workspace first, or run each shape once before capturing.
 #pragma once
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
@@ -26,6 +26,7 @@
 #include <type_traits>
 #include <string>
 #include <unordered_map>
+#include <stdint.h>
 
 #include "../../../llmmm.h"
 
@@ -44,35 +45,82 @@ inline void throw_on_error(int code)
   throw std::runtime_error(std::string(llmmm_error_string(code)) + ": " + llmmm_last_error());
 }
 
-// Scratch for the split-K planes of a shim call: at least `bytes` (nullptr for 0), private to this host thread and
-// stream.  Growing frees the old buffer first (hipFree waits for the device, so no kernel still uses it).
-inline void* cached_workspace(hipStream_t stream, size_t bytes)
-{
+// Scratch for the split-K planes of a shim call, private to this host thread and stream.  Either the caller's own buffer
+// (LLMMM::set_fp8_workspace: the shim then never allocates, frees or waits) or one the shim allocates on first need, grows
+// when a later call needs more (hipFree waits for the device, so no kernel still uses the old one) and frees when the
+// thread ends.
+struct WorkspaceSlots {
   struct Slot {
-    void*  ptr   = nullptr;
-    size_t bytes = 0;
+    void*  ptr    = nullptr;
+    size_t bytes  = 0;
+    bool   caller = false;  // the caller's buffer: never freed here
   };
-  static thread_local std::unordered_map<hipStream_t, Slot> slots;
-  if (bytes == 0) return nullptr;
-  Slot& s = slots[stream];
-  if (s.bytes < bytes) {
+  std::unordered_map<hipStream_t, Slot> slots;
+  ~WorkspaceSlots()
+  {
+    for (auto& kv : slots)
+      if (kv.second.ptr && !kv.second.caller) (void)hipFree(kv.second.ptr);
+  }
+};
+inline WorkspaceSlots& workspace_slots()
+{
+  static thread_local WorkspaceSlots w;
+  return w;
+}
+
+// The buffer for a call that needs `need` bytes; *have = what the library may use of it.  A caller's buffer that is
+// smaller than `need` is passed on as it is: llmmm_fp8_gemm then splits K less (or not at all), it does not fail.
+inline void* cached_workspace(hipStream_t stream, size_t need, size_t* have)
+{
+  *have = 0;
+  if (need == 0) return nullptr;
+  WorkspaceSlots::Slot& s = workspace_slots().slots[stream];
+  if (s.caller) {
+    *have = s.bytes;
+    return s.ptr;
+  }
+  if (s.bytes < need) {
     size_t want = size_t(1) << 20;
-    while (want < bytes) want <<= 1;
+    while (want < need) want <<= 1;
     if (s.ptr) (void)hipFree(s.ptr);
     s.ptr = nullptr, s.bytes = 0;
     const hipError_t e = hipMalloc(&s.ptr, want);
     if (e != hipSuccess) throw std::runtime_error(std::string("workspace allocation failed: ") + hipGetErrorString(e));
     s.bytes = want;
   }
+  *have = s.bytes;
   return s.ptr;
 }
 
 inline void gemm(int out_kind, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K, hipStream_t stream)
 {
   const size_t need = llmmm_fp8_gemm_workspace(out_kind, M, N, K);  // 0 for shapes that run unsplit (and for invalid ones)
-  throw_on_error(llmmm_fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, cached_workspace(stream, need), need, (void*)stream));
+  size_t       have = 0;
+  void*        ws   = cached_workspace(stream, need, &have);
+  throw_on_error(llmmm_fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, ws, have, (void*)stream));
 }
 }  // namespace detail8
+
+// Hands the launchers of this header a split-K workspace for calls of the calling thread on `stream`: device memory of
+// `bytes` bytes, 16-byte aligned, plain scratch, which must stay valid until it is replaced or withdrawn
+// (set_fp8_workspace(stream, nullptr, 0): back to the shim's own buffer; one it had allocated before is kept and reused).
+// With a workspace set, the reference-signature launchers honour the reference's contract to the letter -- no
+// allocation, no free, no synchronisation (src/mm/fp16/mm.cu:6-42) -- and can be captured into a HIP graph on first use.
+// llmmm_fp8_gemm_workspace(out_kind, M, N, K) gives the size a shape wants; with less, K is split less or not at all.
+// The reference has no such call (its kernels never split K, README.md:22).
+inline void set_fp8_workspace(hipStream_t stream, void* workspace, size_t bytes)
+{
+  auto& slots = detail8::workspace_slots().slots;
+  auto  it    = slots.find(stream);
+  if (workspace && bytes) {
+    if (reinterpret_cast<uintptr_t>(workspace) & 15u) throw std::runtime_error("invalid argument: workspace must be 16-byte aligned");
+    if (it != slots.end() && it->second.ptr && !it->second.caller) (void)hipFree(it->second.ptr);  // the shim's own buffer gives way
+    detail8::WorkspaceSlots::Slot& s = slots[stream];
+    s.ptr = workspace, s.bytes = bytes, s.caller = true;
+  }
+  else if (it != slots.end() && it->second.caller)
+    slots.erase(it);
+}
 
 template <int QUANT_M, int QUANT_N, bool SCALE_TRANSPOSE>
 void fp8_blockwise_symmetric_quantization(const float* x, fp8_t* q, float* scale, int M, int N, hipStream_t stream)

@@ -8,7 +8,10 @@
 #include <hip/hip_runtime.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
+
+#include <vector>
 
 namespace {
 
@@ -26,6 +29,18 @@ int fail(int code, const char* fmt, ...)
 
 }  // namespace
 
+int llmmm::num_cus()
+{
+  static const int n = [] {
+    int            dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) return prop.multiProcessorCount;
+    (void)hipGetLastError();  // no device: not an error of the call that asked
+    return 256;
+  }();
+  return n;
+}
+
 // The same for the other files of the library (declared in kernels.h).
 int llmmm::report_error(int code, const char* fmt, ...)
 {
@@ -41,7 +56,9 @@ namespace {
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 constexpr int    MAX_SPLIT_K     = 32;
-constexpr int    NUM_CUS         = 256;   // MI355X
+// Compute units of the current device (llmmm::num_cus: read from the runtime once; 256, the MI355X, where no device
+// can be asked -- the size queries also work without one).
+#define NUM_CUS (llmmm::num_cus())
 
 constexpr int SKINNY_MAX_M = 128;  // rows the weight-streaming kernel takes
 
@@ -139,6 +156,102 @@ bool tile_dims(int tile, int& bm, int& bn)
   }
 }
 
+// ---- tune tables: entries read at run time from the file LLMMM_TUNE_FILE names (if any) come first, the compiled-in
+// table (tune_table.h) second.  File format, one entry per line, '#' starts a comment:
+//   skinny <m_max> <N> <K> <split_k>          FP8 weight-streaming kernel, applies to M <= m_max
+//   tile   <M> <N> <K> <tile id> <split_k>    FP8 MFMA tile kernels (tile ids: LLMMM_TILE_*; split_k 0 = heuristic)
+//   fp16   <M> <N> <K> <tile id>              FP16 / BF16 GEMM
+// (`python -m llmmm_amd.tune --write-file PATH` writes it.)  The reference only hints at tuning: tune(N, K),
+// src/mm/fp32/impl.h:20-23.
+struct TuneOverride {
+  std::vector<llmmm::SkinnyTune> skinny;
+  std::vector<llmmm::TileTune>   tile, fp16;
+};
+const TuneOverride& tune_override()
+{
+  static const TuneOverride t = [] {
+    TuneOverride o;
+    const char*  path = getenv("LLMMM_TUNE_FILE");
+    if (!path || !*path) return o;
+    FILE* f = fopen(path, "r");
+    if (!f) {
+      fprintf(stderr, "llmmm: LLMMM_TUNE_FILE=%s cannot be read; using the built-in table\n", path);
+      return o;
+    }
+    char line[256];
+    int  lineno = 0;
+    while (fgets(line, sizeof(line), f)) {
+      ++lineno;
+      if (char* h = strchr(line, '#')) *h = 0;
+      char kind[16];
+      int  a, b, c, d, e;
+      const int n = sscanf(line, "%15s %d %d %d %d %d", kind, &a, &b, &c, &d, &e);
+      if (n <= 0) continue;  // blank
+      int bm, bn;
+      if (n == 5 && !strcmp(kind, "skinny") && a >= 1 && a <= SKINNY_MAX_M && b > 0 && c > 0 && d >= 1 && d <= MAX_SPLIT_K)
+        o.skinny.push_back({a, b, c, d});
+      else if (n == 6 && !strcmp(kind, "tile") && a > 0 && b > 0 && c > 0 && tile_dims(d, bm, bn) && d != LLMMM_TILE_64x128 && d != LLMMM_TILE_128x160 && e >= 0 &&
+               e <= MAX_SPLIT_K)
+        o.tile.push_back({a, b, c, d, e});
+      else if (n == 5 && !strcmp(kind, "fp16") && a > 0 && b > 0 && c > 0 && tile_dims(d, bm, bn) && d != LLMMM_TILE_128x160)
+        o.fp16.push_back({a, b, c, d, 1});
+      else
+        fprintf(stderr, "llmmm: %s:%d: not a tune entry, ignored\n", path, lineno);
+    }
+    fclose(f);
+    return o;
+  }();
+  return t;
+}
+
+// FP8 tile kernels: the entry of this exact shape; failing that, for an (N, K) the tables know at other M, the tile of the
+// entry nearest in M (by ratio, less than a factor of two away) whose tile divides this M -- its split count does not carry over (it depends on how many
+// tiles M makes), the heuristic decides that.  false: nothing known about (N, K).
+template <typename Table>
+bool lookup_tile_in(const Table& table, int M, int N, int K, int* tile, int* split, double* best_ratio)
+{
+  bool found = false;
+  for (const auto& e : table) {
+    if (e.N != N || e.K != K) continue;
+    int bm, bn;
+    if (!tile_dims(e.tile, bm, bn) || M % bm || N % bn) continue;
+    const double ratio = e.M > M ? (double)e.M / M : (double)M / e.M;
+    if (ratio < *best_ratio) {
+      *best_ratio = ratio, *tile = e.tile, *split = e.M == M ? e.split_k : 0;
+      found = true;
+    }
+  }
+  return found;
+}
+bool lookup_tile(int M, int N, int K, int* tile, int* split, bool exact_only = false)
+{
+  // (beyond a factor of two in M the tile count changes too much for the tuned tile to say anything: M = 8192 on the
+  // 2560-column projections runs 7 % faster in the heuristic's 256 x 256 tiles than in the 128 x 128 ones tuned at M = 2048)
+  const double limit = exact_only ? 1.0 + 1e-9 : 2.0;
+  double       best  = limit;
+  if (lookup_tile_in(tune_override().tile, M, N, K, tile, split, &best) && best == 1.0) return true;  // an exact entry of the file wins
+  double best2 = best;
+  int    t2 = 0, s2 = 0;
+  if (lookup_tile_in(llmmm::kTileTune, M, N, K, &t2, &s2, &best2) && best2 < best) *tile = t2, *split = s2, best = best2;
+  return best < limit;
+}
+bool lookup_skinny(int M, int N, int K, int* split)
+{
+  for (const auto& e : tune_override().skinny)
+    if (e.N == N && e.K == K && M <= e.m_max) return *split = e.split_k, true;
+  for (const auto& e : llmmm::kSkinnyTune)
+    if (e.N == N && e.K == K && M <= e.m_max) return *split = e.split_k, true;
+  return false;
+}
+bool lookup_fp16_tile(int M, int N, int K, int* tile)
+{
+  for (const auto& e : tune_override().fp16)
+    if (e.M == M && e.N == N && e.K == K) return *tile = e.tile, true;
+  for (const auto& e : llmmm::kFp16TileTune)
+    if (e.M == M && e.N == N && e.K == K) return *tile = e.tile, true;
+  return false;
+}
+
 int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
 {
   if (M <= 0 || N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "M, N and K must be positive (got %d, %d, %d)", M, N, K);
@@ -147,30 +260,20 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
   cfg->split_k  = 0;
   cfg->b_layout = LLMMM_FP8_B_ROWS;
   cfg->a_layout = LLMMM_FP8_A_QUANTISED;
-  if (M % 128 == 0)
-    for (const auto& e : llmmm::kTileTune)
-      if (e.M == M && e.N == N && e.K == K) {
-        cfg->tile    = e.tile;
-        cfg->split_k = e.split_k;
-        break;
-      }
+  if (M % 128 == 0) {
+    int t, sp;
+    if (lookup_tile(M, N, K, &t, &sp, true)) cfg->tile = t, cfg->split_k = sp;
+  }
   // 64 < M < 128: where the table gives M = 128 to 128 x 128 tiles, the same tiles take the shorter matrix too (the
   // rows of the tile beyond M are computed and not stored) -- 96 x 19456 x 2560: 20 us instead of 33 us in the
   // weight-streaming kernel, whose eight 16-row blocks per wave are bound by their LDS reads and fp32 planes
-  if (cfg->tile < 0 && M > 64 && M < 128)
-    for (const auto& e : llmmm::kTileTune)
-      if (e.M == 128 && e.N == N && e.K == K && e.tile == LLMMM_TILE_128x128) {
-        cfg->tile    = e.tile;
-        cfg->split_k = e.split_k;
-        break;
-      }
+  if (cfg->tile < 0 && M > 64 && M < 128) {
+    int t, sp;
+    if (lookup_tile(128, N, K, &t, &sp, true) && t == LLMMM_TILE_128x128) cfg->tile = t, cfg->split_k = sp;
+  }
   if (cfg->tile < 0 && M <= SKINNY_MAX_M) {
-    for (const auto& e : llmmm::kSkinnyTune)
-      if (e.N == N && e.K == K && M <= e.m_max) {
-        cfg->tile    = LLMMM_TILE_SKINNY;
-        cfg->split_k = e.split_k;
-        break;
-      }
+    int sp;
+    if (lookup_skinny(M, N, K, &sp)) cfg->tile = LLMMM_TILE_SKINNY, cfg->split_k = sp;
     // untuned shapes: the weight-streaming kernel up to 64 rows; above that only while the weight matrix is small -- its
     // eight 16-row blocks per wave and its fp32 planes grow with M, and from about 20 MB of weights on, one row of 128 x 128
     // tiles (a row tail for M < 128) is faster (measured at M = 96, us, streaming / tiles: N x K = 4096 x 4096 12.4 / 14.2,
@@ -179,7 +282,12 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
   }
   if (cfg->tile < 0) {
     if (M % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
-    cfg->tile = heuristic_tile(M, N);
+    // an (N, K) that was tuned at other M: the tile of the nearest tuned M; otherwise the heuristic
+    int t, sp;
+    if (lookup_tile(M, N, K, &t, &sp))
+      cfg->tile = t, cfg->split_k = sp;
+    else
+      cfg->tile = heuristic_tile(M, N);
   }
   if (cfg->tile == LLMMM_TILE_SKINNY) {
     if (cfg->split_k <= 0) cfg->split_k = heuristic_split(M, N, K);
@@ -262,11 +370,7 @@ int llmmm_fp16_gemm_ex(int dtype, const void* A, const void* B, void* C, int M, 
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
   int tile = cfg ? cfg->tile : LLMMM_TILE_AUTO;
   if (tile == LLMMM_TILE_AUTO) {
-    for (const auto& e : llmmm::kFp16TileTune)
-      if (e.M == M && e.N == N && e.K == K) {
-        tile = e.tile;
-        break;
-      }
+    if (!lookup_fp16_tile(M, N, K, &tile)) tile = LLMMM_TILE_AUTO;
     if (tile == LLMMM_TILE_AUTO) {
       tile = heuristic_tile(M, N);
       // small problems: 128 x 128 tiles on at most half of the CUs -> twice as many 64 x 128 tiles of four 16-row

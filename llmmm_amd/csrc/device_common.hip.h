@@ -12,7 +12,6 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef int i32x2 __attribute__((ext_vector_type(2)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
@@ -21,26 +20,21 @@ typedef int i32x8 __attribute__((ext_vector_type(8)));
 #define LLMMM_GLOBAL __attribute__((address_space(1)))
 
 // ---------------------------------------------------------------------------------------------
-// K-major operand tiles in LDS.  A tile row holds ROW bytes of the K extent as 16-byte chunks;
-// row r / chunk c lives at  phys_row(r) * ROW + ((c ^ swz(r)) << 4).
+// K-major operand tiles in LDS (FP8): a tile row holds 128 bytes of the K extent as eight 16-byte chunks;
+// row r / chunk c lives at  r * 128 + ((c ^ swz(r)) << 4).
 // ds_read_b128 serves a wavefront in four passes of 16 lanes -- {0-3,12-15,20-23,24-27},
 // {4-11,16-19,28-31} and the same two sets + 32 (measured on gfx950) -- and a pass is
 // conflict-free when its 16 lanes touch 16 different 16-byte slots of the 256-byte bank row.
-// Each placement is matched to the lane -> (row, chunk) pattern of one MFMA operand shape:
-//   SWZ_ROW64:  64-byte rows (32 fp16).  Lanes 0-31 read 32 consecutive rows at one chunk,
-//               lanes 32-63 at another (32x32x16 f16/bf16 operands).  Four consecutive rows
-//               fill a bank row; the chunk is XOR-ed with row bits 2..3, inverted when bit 4
-//               is set, which separates the four row quads of a pass.
-//   SWZ_ROWS16: 128-byte rows (128 fp8).  Lanes 16g..16g+15 read 16 consecutive rows at chunk
-//               2g (+1) (16x16x128 fp8 operands).  The chunk is XOR-ed with row bits 1..3 and,
-//               for rows 4..11 of every 16, with 2, which cancels the chunk difference
-//               between the two halves of a pass.
+// SWZ_ROWS16 is matched to the lane -> (row, chunk) pattern of the 16x16x128 fp8 MFMA operands: lanes 16g..16g+15 read
+// 16 consecutive rows at chunk 2g (+1).  The chunk is XOR-ed with row bits 1..3 and, for rows 4..11 of every 16, with
+// 2, which cancels the chunk difference between the two halves of a pass.
 // ---------------------------------------------------------------------------------------------
-enum { SWZ_ROW64 = 0, SWZ_ROWS16 = 1 };
+enum { SWZ_ROWS16 = 1 };
 
 template <int SWZ>
 struct KMajor {
-  static constexpr int ROW    = SWZ == SWZ_ROW64 ? 64 : 128;  // bytes per tile row
+  static_assert(SWZ == SWZ_ROWS16, "one placement only");
+  static constexpr int ROW    = 128;  // bytes per tile row
   static constexpr int CHUNKS = ROW / 16;
   static constexpr int ROWS_PER_KB = 1024 / ROW;              // tile rows covered by one 1 KB load
 };
@@ -48,7 +42,7 @@ struct KMajor {
 template <int SWZ>
 __device__ __forceinline__ int kmajor_swz(int r)
 {
-  return SWZ == SWZ_ROW64 ? (((r >> 2) & 3) ^ (((r >> 4) & 1) * 3)) : (((r >> 1) & 7) ^ ((((r >> 2) ^ (r >> 3)) & 1) << 1));
+  return ((r >> 1) & 7) ^ ((((r >> 2) ^ (r >> 3)) & 1) << 1);
 }
 template <int SWZ>
 __device__ __forceinline__ int kmajor_offset(int r, int c)
@@ -71,14 +65,8 @@ __device__ __forceinline__ KMajorLane kmajor_lane(int group, int lane)
   return p;
 }
 
-// 16 bytes per lane, global -> LDS without passing through registers.  lds_base must be
-// wave-uniform; lane l's data lands at lds_base + 16*l.
-__device__ __forceinline__ void load_lds_16B(const void* gptr, void LLMMM_LDS* lds_base)
-{
-  __builtin_amdgcn_global_load_lds((const void LLMMM_GLOBAL*)gptr, lds_base, 16, 0, 0);
-}
-
-// The same load written as inline assembly, invisible to the compiler's wait-count bookkeeping.
+// 16 bytes per lane, global -> LDS without passing through registers (lane l's data lands at lds_addr + 16*l), written
+// as inline assembly so that it stays invisible to the compiler's wait-count bookkeeping.
 // While an LDS-direct load that the compiler knows about is in flight, every wait it inserts on
 // its own becomes "all loads done", which defeats a deep software pipeline; kernels that keep
 // many slices in flight issue all their vector-memory loads through these helpers and place the

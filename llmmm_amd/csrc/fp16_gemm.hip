@@ -382,10 +382,11 @@ static hipError_t launch_fp16(const void* A, const void* B, void* C, int M, int 
   if constexpr (BM == 256 && BN == 256) {
     // more than one round of the chip with a partly filled last one: whole rounds in 256 x 256 tiles, the remaining
     // columns in 128 x 256 tiles, if those fit one round (fp16_gemm_hybrid_kernel)
-    const long tiles = (long)tiles_m * tiles_n, full = tiles / 256 * 256;
-    if (tiles > 256 && tiles_m > 1 && full % tiles_m == 0) {
+    const int  cus   = num_cus();
+    const long tiles = (long)tiles_m * tiles_n, full = tiles / cus * cus;
+    if (tiles > cus && tiles_m > 1 && full % tiles_m == 0) {
       const int cols_big = (int)(full / tiles_m), cols_small = tiles_n - cols_big;
-      if (cols_small > 0 && (long)cols_small * tiles_m * 2 <= 256) {
+      if (cols_small > 0 && (long)cols_small * tiles_m * 2 <= cus) {
         const dim3 grid(tiles_m * cols_big + 2 * tiles_m * cols_small);
         if (K % TC::BK)
           hipLaunchKernelGGL((fp16_gemm_hybrid_kernel<T, B_NK, true>), grid, dim3(512), 0, stream, (const T*)A, (const T*)B, (T*)C, M, N, K, tiles_m,

@@ -969,7 +969,8 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
   const int tiles_m = (M + BM - 1) / BM, tiles_n = N / BN;
   if (M % BM != 0 && tiles_m != 1) return hipErrorInvalidValue;  // a row tail: M < BM only (one tile row, the deep form)
   // one tile row: the weights are read once (streamed, deep); at most one workgroup per CU: deep
-  const bool one_per_cu = (long)tiles_m * tiles_n * (S < 1 ? 1 : S) <= 256;
+  const int  cus        = num_cus();
+  const bool one_per_cu = (long)tiles_m * tiles_n * (S < 1 ? 1 : S) <= cus;
   const int  bmode      = (bpre ? 1 : 0) | (tiles_m == 1 ? 2 | 4 : 0) | (one_per_cu ? 4 : 0) | (M % BM != 0 ? 8 : 0);
   if (S <= 1 && planes == nullptr) {
     if constexpr (OUT == OUT_SWIGLU && BN != 256) {
@@ -980,10 +981,10 @@ static hipError_t launch_fp8(const void* A, const float* As, const void* Bt, con
         // more than one round of the chip with a partly filled last one: whole rounds in 256 x 256 tiles, the remaining
         // columns in 128 x 256 tiles, if those fit one round (fp8_gemm_hybrid_kernel)
         const long tiles = (long)tiles_m * tiles_n;
-        const long full  = tiles / 256 * 256;
-        if (tiles > 256 && tiles_m > 1 && full % tiles_m == 0) {
+        const long full  = tiles / cus * cus;
+        if (tiles > cus && tiles_m > 1 && full % tiles_m == 0) {
           const int cols_big = (int)(full / tiles_m), cols_small = tiles_n - cols_big;
-          if (cols_small > 0 && (long)cols_small * tiles_m * 2 <= 256) {
+          if (cols_small > 0 && (long)cols_small * tiles_m * 2 <= cus) {
             const dim3 grid(tiles_m * cols_big + 2 * tiles_m * cols_small);
             if (bpre)
               hipLaunchKernelGGL((fp8_gemm_hybrid_kernel<OUT, 1>), grid, dim3(512), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs, M,

@@ -98,6 +98,10 @@ hipError_t probe_stream_read_launch(const void* src, size_t bytes, float* sink, 
 hipError_t planes_add_rmsnorm_quant_launch(int hidden_dtype, const float* planes, int S, const void* residual, void* hidden, const float* w,
                                            float eps, void* q, float* scale, int M, int N, hipStream_t stream);
 
+// Compute units of the device (hipDeviceProp_t::multiProcessorCount of the device that is current on first use; 256 when
+// there is none): what "a round of the chip" means to the tile heuristics and the two-shape launches.
+int num_cus();
+
 // Leaves the text in the calling thread's llmmm_last_error() and returns `code` (capi.cpp).
 int report_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 

@@ -1,13 +1,15 @@
 """Offline auto-tune driver: measures every candidate configuration of the FP8 GEMM for a list
 of shapes on the GPU at hand and writes ``csrc/tune_table.h`` (compiled into ``libllmmm.so``).
 
-    python -m llmmm_amd.tune [--write] [--shapes qwen3-4b] [--m 1,16,128,2048]
+    python -m llmmm_amd.tune [--write] [--write-file PATH] [--m 1,16,128,2048] [--shape N,K ...]
 
 The reference only hints at such an interface (``tune(N, K)`` in src/mm/fp32/impl.h:20-23, a
 stub that throws).  Candidates: for M <= 128 the split-K factor of the weight-streaming kernel;
 for M % 128 == 0 the MFMA tile (M = 128 tries both).  Timing: HIP events around a HIP graph of back-to-back launches
 that rotate over enough weight copies to defeat the caches (decode shapes) -- the same method
-``bench.py`` uses.  Without ``--write`` the table is only printed.
+``bench.py`` uses.  Without ``--write`` the table is only printed.  ``--write-file PATH`` writes the same
+results as a text file that the library reads at run time when ``LLMMM_TUNE_FILE=PATH`` is set (its entries come
+before the compiled-in table; no rebuild), e.g. for the projection shapes of another model: ``--shape 4096,14336``.
 """
 import argparse
 import os
@@ -110,16 +112,48 @@ def render_table(skinny_rows, tile_rows, fp16_rows):
     return "\n".join(out)
 
 
+def render_file(skinny_rows, tile_rows, fp16_rows):
+    """The run-time form of the table (LLMMM_TUNE_FILE): one entry per line, '#' comments."""
+    out = ["# llmmm tune file: entries override the table compiled into libllmmm.so (set LLMMM_TUNE_FILE to this path)",
+           "# skinny <m_max> <N> <K> <split_k> | tile <M> <N> <K> <tile id> <split_k> | fp16 <M> <N> <K> <tile id>"]
+    out += ["skinny %d %d %d %d" % r for r in skinny_rows]
+    out += ["tile %d %d %d %d %d" % r for r in tile_rows]
+    out += ["fp16 %d %d %d %d" % r[:4] for r in fp16_rows]
+    return "\n".join(out) + "\n"
+
+
+def parse_file(text):
+    """Inverse of render_file: (skinny_rows, tile_rows, fp16_rows); lines that are not entries are skipped, as the library does."""
+    skinny, tile, fp16 = [], [], []
+    for line in text.splitlines():
+        f = line.split("#", 1)[0].split()
+        try:
+            if len(f) == 5 and f[0] == "skinny":
+                skinny.append(tuple(int(x) for x in f[1:]))
+            elif len(f) == 6 and f[0] == "tile":
+                tile.append(tuple(int(x) for x in f[1:]))
+            elif len(f) == 5 and f[0] == "fp16":
+                fp16.append(tuple(int(x) for x in f[1:]) + (1,))
+        except ValueError:
+            pass
+    return skinny, tile, fp16
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--write", action="store_true", help="rewrite csrc/tune_table.h with the results")
     ap.add_argument("--m", default="1,16,32,64,96,128,256,512,1024,2048")
     ap.add_argument("--iters", type=int, default=40)
+    ap.add_argument("--write-file", metavar="PATH", help="write the results as a run-time tune file (LLMMM_TUNE_FILE)")
+    ap.add_argument("--shape", action="append", metavar="N,K", help="tune this weight shape instead of the Qwen3-4B projections (repeatable)")
     args = ap.parse_args()
     torch.cuda.set_device(0)
     ms = [int(x) for x in args.m.split(",")]
-    skinny_rows, tile_rows = [], [(4096, 4096, 4096, _lib.TILE_256x256, 1)]
-    for name, (N, K) in QWEN3_4B.items():
+    shapes = QWEN3_4B
+    if args.shape:
+        shapes = {"%sx%s" % tuple(x.split(",")): tuple(int(v) for v in x.split(",")) for x in args.shape}
+    skinny_rows, tile_rows = [], ([] if args.shape else [(4096, 4096, 4096, _lib.TILE_256x256, 1)])
+    for name, (N, K) in shapes.items():
         for M in ms:
             tile, split, _ = tune_shape(M, N, K, iters=args.iters)
             if tile == _lib.TILE_SKINNY:
@@ -130,10 +164,14 @@ def main():
                 tile_rows.append((M, N, K, tile, split))
             torch.cuda.empty_cache()
     skinny_rows.sort(key=lambda r: (r[1], r[2], r[0]))
-    fp16_rows = [(4096, 4096, 4096, _lib.TILE_256x256, 1), (1024, 1024, 1024, _lib.TILE_64x128, 1)]
+    fp16_rows = [] if args.shape else [(4096, 4096, 4096, _lib.TILE_256x256, 1), (1024, 1024, 1024, _lib.TILE_64x128, 1)]
     text = render_table(skinny_rows, tile_rows, fp16_rows)
     print(text)
-    if args.write:
+    if args.write_file:
+        with open(args.write_file, "w") as f:
+            f.write(render_file(skinny_rows, tile_rows, fp16_rows))
+        print("wrote %s -- use it with LLMMM_TUNE_FILE=%s" % (args.write_file, args.write_file), file=sys.stderr)
+    if args.write and not args.shape:
         with open(os.path.join(HERE, "csrc", "tune_table.h"), "w") as f:
             f.write(text)
         print("wrote csrc/tune_table.h -- rebuild with `python llmmm_amd/build.py`", file=sys.stderr)

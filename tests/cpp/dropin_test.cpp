@@ -226,6 +226,70 @@ int main()
     printf("decode shapes through the reference signatures (cached split-K workspace): %s\n", fd ? "FAIL" : "ok");
     fails += fd;
   }
+  // ---- a caller-supplied workspace: the reference-signature launcher then allocates nothing, so its very first call on a
+  // fresh stream can be captured into a graph; replayed, it gives the bits of the eager C-API call
+  {
+    int fw = 0;
+    const int m = 16, n = 2560, k = 4096;
+    std::vector<float> fx((size_t)m * k), fwt((size_t)n * k);
+    for (auto& v : fx) { s = s * 1664525u + 1013904223u; v = ((s >> 8) / 16777216.0f) * 4.f - 2.f; }
+    for (auto& v : fwt) { s = s * 1664525u + 1013904223u; v = ((s >> 8) / 16777216.0f) * 0.1f - 0.05f; }
+    float *dx, *dw, *das, *dbs, *dcs0, *dcs1;
+    LLMMM::fp8_t *daq, *dbq, *dc0, *dc1;
+    void *ws0, *ws1;
+    const size_t wsz = llmmm_fp8_gemm_workspace(LLMMM_OUT_FP8Q, m, n, k);
+    CHECK(hipMalloc(&dx, fx.size() * 4)); CHECK(hipMalloc(&dw, fwt.size() * 4)); CHECK(hipMalloc(&daq, (size_t)m * k)); CHECK(hipMalloc(&dbq, (size_t)n * k));
+    CHECK(hipMalloc(&das, (k / 128) * m * 4)); CHECK(hipMalloc(&dbs, (n / 128) * (k / 128) * 4)); CHECK(hipMalloc(&dc0, (size_t)m * n)); CHECK(hipMalloc(&dc1, (size_t)m * n));
+    CHECK(hipMalloc(&dcs0, (n / 128) * m * 4)); CHECK(hipMalloc(&dcs1, (n / 128) * m * 4)); CHECK(hipMalloc(&ws0, wsz)); CHECK(hipMalloc(&ws1, wsz));
+    CHECK(hipMemcpy(dx, fx.data(), fx.size() * 4, hipMemcpyHostToDevice));
+    CHECK(hipMemcpy(dw, fwt.data(), fwt.size() * 4, hipMemcpyHostToDevice));
+    CHECK(hipMemset(dc0, 0x55, (size_t)m * n));
+    LLMMM::fp8_blockwise_symmetric_quantization<1, 128, true>(dx, daq, das, m, k, nullptr);
+    LLMMM::fp8_blockwise_symmetric_quantization<128, 128, false>(dw, dbq, dbs, n, k, nullptr);
+    if (llmmm_fp8_gemm(LLMMM_OUT_FP8Q, daq, das, dbq, dbs, dc1, dcs1, m, n, k, ws1, wsz, nullptr) != LLMMM_OK) ++fw;
+    CHECK(hipDeviceSynchronize());
+    hipStream_t st;
+    CHECK(hipStreamCreate(&st));
+    if (!throws_with([&] { LLMMM::set_fp8_workspace(st, (char*)ws0 + 4, wsz - 4); }, "invalid argument: workspace must be 16-byte aligned")) { ++fw; printf("misaligned workspace: FAIL\n"); }
+    LLMMM::set_fp8_workspace(st, ws0, wsz);
+    hipGraph_t     graph;
+    hipGraphExec_t exec;
+    CHECK(hipStreamBeginCapture(st, hipStreamCaptureModeGlobal));
+    LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(daq, das, dbq, dbs, dc0, dcs0, m, n, k, st);  // first call on this stream
+    CHECK(hipStreamEndCapture(st, &graph));
+    CHECK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+    for (int rep = 0; rep < 3; ++rep) {
+      CHECK(hipMemsetAsync(dc0, 0x55, (size_t)m * n, st));
+      CHECK(hipGraphLaunch(exec, st));
+      CHECK(hipStreamSynchronize(st));
+      std::vector<unsigned char> h0((size_t)m * n), h1((size_t)m * n);
+      std::vector<float>         s0((n / 128) * m), s1((n / 128) * m);
+      CHECK(hipMemcpy(h0.data(), dc0, h0.size(), hipMemcpyDeviceToHost)); CHECK(hipMemcpy(h1.data(), dc1, h1.size(), hipMemcpyDeviceToHost));
+      CHECK(hipMemcpy(s0.data(), dcs0, s0.size() * 4, hipMemcpyDeviceToHost)); CHECK(hipMemcpy(s1.data(), dcs1, s1.size() * 4, hipMemcpyDeviceToHost));
+      if (memcmp(h0.data(), h1.data(), h0.size()) != 0 || memcmp(s0.data(), s1.data(), s0.size() * 4) != 0) ++fw;
+    }
+    // a workspace too small for any split: the call still succeeds (unsplit), within the blockwise GEMM's tolerance of the split result
+    LLMMM::set_fp8_workspace(st, ws0, 1024);
+    LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(daq, das, dbq, dbs, dc0, dcs0, m, n, k, st);
+    CHECK(hipStreamSynchronize(st));
+    {
+      std::vector<float> s0((n / 128) * m), s1((n / 128) * m);
+      CHECK(hipMemcpy(s0.data(), dcs0, s0.size() * 4, hipMemcpyDeviceToHost)); CHECK(hipMemcpy(s1.data(), dcs1, s1.size() * 4, hipMemcpyDeviceToHost));
+      for (size_t i = 0; i < s0.size(); ++i)
+        if (!(s0[i] >= s1[i] * (1 - 1e-3f) && s0[i] <= s1[i] * (1 + 1e-3f))) ++fw;
+    }
+    LLMMM::set_fp8_workspace(st, nullptr, 0);  // withdrawn: the shim's own buffer again
+    LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(daq, das, dbq, dbs, dc0, dcs0, m, n, k, st);
+    CHECK(hipStreamSynchronize(st));
+    {
+      std::vector<unsigned char> h0((size_t)m * n), h1((size_t)m * n);
+      CHECK(hipMemcpy(h0.data(), dc0, h0.size(), hipMemcpyDeviceToHost)); CHECK(hipMemcpy(h1.data(), dc1, h1.size(), hipMemcpyDeviceToHost));
+      if (memcmp(h0.data(), h1.data(), h0.size()) != 0) ++fw;
+    }
+    CHECK(hipGraphExecDestroy(exec)); CHECK(hipGraphDestroy(graph)); CHECK(hipStreamDestroy(st));
+    printf("caller-supplied workspace: first call captured into a graph, too-small and withdrawn workspaces: %s\n", fw ? "FAIL" : "ok");
+    fails += fw;
+  }
   printf(fails ? "DROPIN FAIL (%d)\n" : "DROPIN OK\n", fails);
   return fails ? 1 : 0;
 }

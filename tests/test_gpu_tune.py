@@ -1,0 +1,30 @@
+"""The auto-tune driver on the GPU: tune_shape measures its candidates for a small shape and names one that the library
+accepts; what it would write for that shape is a valid table row."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 512, 1024), (128, 512, 1024)])
+def test_tune_shape_returns_a_runnable_candidate(lib, oracle, M, N, K):
+    from llmmm_amd import _lib, tune
+    tile, split, results = tune.tune_shape(M, N, K, iters=5, rotate_bytes=8 << 20, verbose=False)
+    assert (tile, split) in results and len(results) >= 3 and all(v > 0 for v in results.values())
+    assert results[(tile, split)] == min(results.values())
+    if M <= 64:
+        assert tile == _lib.TILE_SKINNY and 1 <= split <= K // 128
+    # the winner runs through the C ABI and meets the oracle
+    import numpy as np
+    from helpers import assert_fused_close, fp8_inputs
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=5)
+    t = [torch.from_numpy(a).cuda() for a in (Aq, As, Bq, Bs)]
+    Cq = torch.empty((M, N), dtype=torch.uint8, device="cuda")
+    Cs = torch.empty((N // 128, M), dtype=torch.float32, device="cuda")
+    ws = torch.empty(max(1, split) * M * N * 4, dtype=torch.uint8, device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(*t, Cq, Cs, M, N, K, workspace=ws, tile=tile, split_k=split)
+    torch.cuda.synchronize()
+    rq, rs = oracle.requant_c_1x128(oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128))
+    assert_fused_close(oracle, Cq.cpu().numpy(), Cs.cpu().numpy(), rq, rs, "tuned candidate")
+    rows = ([(M, N, K, split)], []) if tile == _lib.TILE_SKINNY else ([], [(M, N, K, tile, split)])
+    assert tune.parse_file(tune.render_file(rows[0], rows[1], []))[:2] == rows

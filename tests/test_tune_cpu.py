@@ -1,0 +1,70 @@
+"""The tune tables without a GPU: the header `llmmm_amd.tune --write` renders compiles, the run-time file it writes
+round-trips through its parser, and a library started with LLMMM_TUNE_FILE takes the file's entries before its
+compiled-in table; shapes near a tuned one inherit its tile."""
+import os
+import subprocess
+import sys
+import textwrap
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _rows():
+    skinny = [(16, 4096, 14336, 7), (127, 4096, 14336, 4)]
+    tile = [(2048, 4096, 14336, 0, 1), (256, 2560, 4096, 3, 2)]
+    fp16 = [(2048, 2048, 2048, 3, 1)]
+    return skinny, tile, fp16
+
+
+def test_rendered_header_compiles(tmp_path):
+    from llmmm_amd import tune
+    text = tune.render_table(*_rows())
+    csrc = os.path.join(ROOT, "llmmm_amd", "csrc")
+    (tmp_path / "tune_table.h").write_text(text)
+    (tmp_path / "kernels.h").write_text('#include "%s"\n' % os.path.join(csrc, "kernels.h"))
+    (tmp_path / "use.cpp").write_text('#include "tune_table.h"\nint n() { return (int)(sizeof(llmmm::kSkinnyTune) / sizeof(llmmm::kSkinnyTune[0]) + '
+                                      'sizeof(llmmm::kTileTune) / sizeof(llmmm::kTileTune[0]) + sizeof(llmmm::kFp16TileTune) / sizeof(llmmm::kFp16TileTune[0])); }\n')
+    res = subprocess.run(["hipcc", "-x", "hip", "--offload-arch=gfx950", "-fsyntax-only", "-std=c++17", "-I", str(tmp_path), str(tmp_path / "use.cpp")],
+                         stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert res.returncode == 0, res.stdout
+    # and the committed table is what the renderer makes of its own rows
+    cur = open(os.path.join(csrc, "tune_table.h")).read()
+    assert "static const SkinnyTune kSkinnyTune[]" in cur and "static const TileTune kFp16TileTune[]" in cur
+
+
+def test_tune_file_round_trip_and_override(tmp_path):
+    from llmmm_amd import tune
+    skinny, tile, fp16 = _rows()
+    text = tune.render_file(skinny, tile, fp16)
+    assert tune.parse_file(text) == (skinny, tile, fp16)
+    assert tune.parse_file(text + "nonsense 1 2 3\ntile 1 2\n# comment\n") == (skinny, tile, fp16)
+    path = tmp_path / "tune.txt"
+    path.write_text(text + "tile 128 128 128 99 1\nbogus\n")  # an unknown tile id and a stray word: ignored, with a warning
+    prog = textwrap.dedent("""
+        import ctypes, sys
+        sys.path.insert(0, %r)
+        import llmmm_amd
+        from llmmm_amd import _lib
+        q = lambda *a: llmmm_amd.query_config(_lib.OUT_FP8Q, *a)
+        print(q(8, 4096, 14336), q(100, 4096, 14336), q(2048, 4096, 14336), q(256, 2560, 4096), q(16, 2560, 4096), q(3072, 4096, 14336)[0])
+    """ % ROOT)
+    env = dict(os.environ, LLMMM_TUNE_FILE=str(path))
+    res = subprocess.run([sys.executable, "-c", prog], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=env)
+    assert res.returncode == 0, res.stderr
+    # file entries: split 7 up to M = 16, split 4 up to 127; the 256-row entry of the file replaces the built-in one (split 4 -> 2);
+    # shapes the file does not name keep the built-in choice; M = 3072 inherits the tile tuned at M = 2048
+    assert res.stdout.split("\n")[0] == "(8, 7) (8, 4) (0, 1) (3, 2) (8, 8) 0", res.stdout
+    assert "not a tune entry" in res.stderr
+    res = subprocess.run([sys.executable, "-c", prog], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=dict(os.environ, LLMMM_TUNE_FILE=""))
+    assert res.returncode == 0 and "(3, 4) (8, 8)" in res.stdout, res.stdout + res.stderr
+
+
+def test_shapes_near_a_tuned_one_inherit_its_tile():
+    import llmmm_amd
+    from llmmm_amd import _lib
+    q = lambda *a: llmmm_amd.query_config(_lib.OUT_FP8Q, *a)
+    assert q(2048, 19456, 2560) == (_lib.TILE_256x256, 1)
+    assert q(3072, 19456, 2560)[0] == _lib.TILE_256x256      # 1.5 x the tuned M: the tuned tile, the heuristic's split
+    assert q(1536, 2560, 9728)[0] == _lib.TILE_128x128       # between the entries at 1024 and 2048 (both 128 x 128)
+    assert q(128, 6144, 2560)[0] == _lib.TILE_SKINNY         # M = 128 stays with its weight-streaming entry, not the tile tuned at 256
+    assert q(96, 6144, 2560)[0] == _lib.TILE_SKINNY
