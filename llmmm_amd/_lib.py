@@ -29,7 +29,7 @@ class APlanesRmsnorm(ctypes.Structure):
                 ("hidden_out", ctypes.c_void_p), ("norm_weight", ctypes.c_void_p), ("eps", ctypes.c_float)]
 PROBE_FP8 = 2
 STATIC_WS_BYTES = 16 << 20
-TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_64x128, TILE_128x160, TILE_SKINNY = -1, 0, 1, 2, 3, 4, 5, 8
+TILE_AUTO, TILE_256x256, TILE_128x256, TILE_256x128, TILE_128x128, TILE_64x128, TILE_128x160, TILE_SKINNY, TILE_STRIP = -1, 0, 1, 2, 3, 4, 5, 8, 9
 
 
 class GemmCfg(ctypes.Structure):

@@ -314,11 +314,31 @@ void prefer_wide_tile(llmmm_gemm_cfg* cfg, int M, int N)
   if ((t160 + NUM_CUS - 1) / NUM_CUS < (t128 + NUM_CUS - 1) / NUM_CUS) cfg->tile = LLMMM_TILE_128x160;
 }
 
+// The weight-streaming kernel in column strips (one launch, the K split inside the workgroup) takes what the split-K
+// form of that kernel would otherwise do in two launches, for the outputs it has: no 1x128 groups.
+bool strip_fits(int M, int N, int K) { return M >= 1 && M <= llmmm::STRIP_MAX_M && N % 16 == 0 && K % 128 == 0 && K / 128 >= 8; }
+// Every strip reads all M activation rows over all of K, so next to the weights a launch moves M / 16 of their bytes again
+// from L2 into the CUs, whose load path is what bounds it.  Measured against the split form (bf16 out, us, strips /
+// split + reduce): O 4.0 / 6.2 (M = 1), 4.9 / 6.5 (8), 5.6 / 6.8 (16), 7.7 / 7.3 (32); QKV 5.0 / 6.5, 5.7 / 6.6, 6.8 / 6.8,
+// 9.4 / 7.3; down 6.7 / 8.2, 7.7 / 8.9, 9.4 / 9.1, 13.7 / 9.7.
+void prefer_strip(llmmm_gemm_cfg* cfg, int M, int N, int K)
+{
+  if (cfg->tile == LLMMM_TILE_SKINNY && cfg->split_k > 1 && strip_fits(M, N, K) && (M <= 8 || (M <= 16 && K <= 4096)))
+    cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
+}
+
+// The split the weight-streaming kernel runs this shape in when it is the split-K form after all (tune table, then heuristic).
+int skinny_split_for(int M, int N, int K)
+{
+  int sp;
+  return lookup_skinny(M, N, K, &sp) ? sp : heuristic_split(M, N, K);
+}
+
 int choose_fp8_out(int out_kind, int M, int N, int K, llmmm_gemm_cfg* cfg)
 {
   const int rc = choose_fp8(M, N, K, cfg);
   if (rc) return rc;
-  if (out_kind == LLMMM_OUT_F32 || out_kind == LLMMM_OUT_BF16) prefer_wide_tile(cfg, M, N);
+  if (out_kind == LLMMM_OUT_F32 || out_kind == LLMMM_OUT_BF16) prefer_wide_tile(cfg, M, N), prefer_strip(cfg, M, N, K);
   if (out_kind == LLMMM_OUT_FP8Q_SWIGLU) {
     if (N % 256) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
     if (cfg->tile != LLMMM_TILE_SKINNY && cfg->split_k <= 1) {
@@ -522,7 +542,10 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
     return fail(LLMMM_ERR_INVALID_ARGUMENT, "matrix has 2^31 or more elements");
   if (user) {
     // (a named weight-streaming kernel where the library would have taken tiles: the split is that kernel's own heuristic)
-    if (user->tile == LLMMM_TILE_SKINNY && cfg.tile != LLMMM_TILE_SKINNY && M <= SKINNY_MAX_M) cfg.split_k = heuristic_split(M, N, K);
+    if (user->tile == LLMMM_TILE_SKINNY && cfg.tile == LLMMM_TILE_STRIP)
+      cfg.split_k = skinny_split_for(M, N, K);  // (the split-K form named where the library would have taken strips)
+    else if (user->tile == LLMMM_TILE_SKINNY && cfg.tile != LLMMM_TILE_SKINNY && M <= SKINNY_MAX_M)
+      cfg.split_k = heuristic_split(M, N, K);
     if (user->tile != LLMMM_TILE_AUTO) cfg.tile = user->tile;
     if (user->split_k > 0) cfg.split_k = user->split_k;
     if (user->b_layout != LLMMM_FP8_B_ROWS && user->b_layout != LLMMM_FP8_B_PRESHUFFLED)
@@ -535,7 +558,18 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
   const int rca = prepare_a(user, cfg.tile, A, As, M, K, workspace, workspace_bytes, stream, &prep);
   if (rca) return rca;
   const int agen = prep.agen;
-  if (cfg.tile == LLMMM_TILE_SKINNY) {
+  if (cfg.tile == LLMMM_TILE_STRIP && (agen || (user && user->split_k > 1))) {
+    // generated activations and an explicit split are the split-K form's: a strip the library picked itself gives way, one asked for is refused
+    if (user && user->tile == LLMMM_TILE_STRIP) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel takes quantised activations and does not split K over workgroups");
+    cfg.tile = LLMMM_TILE_SKINNY;
+    if (!(user && user->split_k > 0)) cfg.split_k = skinny_split_for(M, N, K);
+  }
+  if (cfg.tile == LLMMM_TILE_STRIP) {
+    if (out_kind != LLMMM_OUT_F32 && out_kind != LLMMM_OUT_BF16) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel has fp32 and bf16 outputs only (a strip holds an eighth of a 1x128 group)");
+    if (!strip_fits(M, N, K)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel handles M <= %d and K >= 1024", llmmm::STRIP_MAX_M);
+    e = llmmm::fp8_strip_launch(out_kind, cfg.b_layout, A, As, Bt, Bs, C, M, N, K, (hipStream_t)stream);
+  }
+  else if (cfg.tile == LLMMM_TILE_SKINNY) {
     int split = cfg.split_k;
     if (split > max_split_for(K)) split = max_split_for(K);
     if (split < 1) split = 1;
@@ -683,7 +717,8 @@ static size_t plane_route_workspace(int M, int N, int K, bool wide_ok)
   if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
   llmmm_gemm_cfg cfg;
   if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
-  if (wide_ok) prefer_wide_tile(&cfg, M, N);
+  if (wide_ok) prefer_wide_tile(&cfg, M, N), prefer_strip(&cfg, M, N, K);
+  if (cfg.tile == LLMMM_TILE_STRIP) return 0;  // epilogue inside the strip kernel
   int split = cfg.split_k < 1 ? 1 : cfg.split_k;
   if (split > max_split_for(K)) split = max_split_for(K);
   int bm = 0, bn = 0;
@@ -700,6 +735,7 @@ size_t llmmm_fp8_gemm_add_rmsnorm_quant_workspace(int M, int N, int K) { return 
 struct PlaneCfg {
   int  tile = 0, split = 0, b_layout = 0;
   bool  skinny = false;
+  bool  strip  = false;  // the weight-streaming kernel in column strips: one launch, its fp32 result is the one "plane"
   APrep prep;
 };
 static int resolve_plane_cfg(const void*& A, const float*& As, const void* Bt, const float* Bs, int M, int N, int K, void*& workspace,
@@ -709,6 +745,9 @@ static int resolve_plane_cfg(const void*& A, const float*& As, const void* Bt, c
   const int      rc = choose_fp8(M, N, K, &cfg);
   if (rc) return rc;
   if (wide_ok) prefer_wide_tile(&cfg, M, N);
+  // (wide_ok also stands for "no 1x128-grouped epilogue behind the GEMM": the callers that may take column strips.  Not with
+  // activations the kernel has to make itself, nor against an explicit split.)
+  if (wide_ok && !(user && (user->a_layout != LLMMM_FP8_A_QUANTISED || user->split_k > 0 || user->tile != LLMMM_TILE_AUTO))) prefer_strip(&cfg, M, N, K);
   const bool a_made = user && user->a_layout != LLMMM_FP8_A_QUANTISED;
   if (!A || (!As && !a_made) || !Bt || !Bs) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
   const bool a_host = user && user->a_layout == LLMMM_FP8_A_PLANES_RMSNORM;  // a host structure, checked by prepare_a
@@ -726,6 +765,22 @@ static int resolve_plane_cfg(const void*& A, const float*& As, const void* Bt, c
   }
   int bm = 0, bn = 0;
   const bool skinny = cfg.tile == LLMMM_TILE_SKINNY;
+  if (cfg.tile == LLMMM_TILE_STRIP) {
+    if (!wide_ok) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel cannot hold whole heads");
+    if (a_made || (user && user->split_k > 1)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel takes quantised activations and does not split K over workgroups");
+    if (!strip_fits(M, N, K)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel handles M <= %d and K >= 1024", llmmm::STRIP_MAX_M);
+    out->prep = APrep();
+    out->tile = cfg.tile, out->b_layout = cfg.b_layout, out->skinny = false, out->strip = true;
+    if (allow_direct) {
+      out->split = 0;  // the caller's epilogue is the strip kernel's own (residual add): no planes
+      return LLMMM_OK;
+    }
+    const size_t plane1 = (size_t)M * N * sizeof(float);
+    if (!workspace || workspace_bytes < plane1) return fail(LLMMM_ERR_WORKSPACE, "workspace holds %zu bytes, one fp32 plane needs %zu", workspace ? workspace_bytes : (size_t)0, plane1);
+    if (!aligned16(workspace)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+    out->split = 1;
+    return LLMMM_OK;
+  }
   if (skinny) {
     if (M > SKINNY_MAX_M) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the weight-streaming kernel handles M <= %d", SKINNY_MAX_M);
   }
@@ -768,7 +823,9 @@ static int launch_into_planes(const PlaneCfg& pc, const void* A, const float* As
 {
   float*     planes = (float*)workspace;
   hipError_t e;
-  if (pc.skinny && pc.prep.agen == 2)
+  if (pc.strip)
+    e = llmmm::fp8_strip_launch(LLMMM_OUT_F32, pc.b_layout, A, As, Bt, Bs, planes, M, N, K, (hipStream_t)stream);
+  else if (pc.skinny && pc.prep.agen == 2)
     e = llmmm::fp8_skinny_rmsnorm_a_launch(pc.prep.hidden_dtype, pc.b_layout, pc.prep.ag, Bt, Bs, nullptr, M, N, K, pc.split, planes, (hipStream_t)stream);
   else if (pc.skinny && pc.prep.agen == 1)
     e = llmmm::fp8_skinny_swiglu_a_launch(LLMMM_OUT_F32, pc.b_layout, (const float*)A, Bt, Bs, nullptr, nullptr, M, N, K, pc.split, planes, (hipStream_t)stream);
@@ -785,6 +842,7 @@ size_t llmmm_fp8_gemm_planes_bytes(int M, int N, int K)
   if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
   llmmm_gemm_cfg cfg;
   if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
+  prefer_strip(&cfg, M, N, K);  // (one plane then: split_k = 1)
   return (size_t)(cfg.split_k < 1 ? 1 : cfg.split_k) * M * N * sizeof(float);
 }
 
@@ -837,9 +895,10 @@ int llmmm_fp8_gemm_add_rmsnorm_quant(const void* A, const float* As, const void*
   int      rc = resolve_plane_cfg(A, As, Bt, Bs, M, N, K, workspace, workspace_bytes, user, true, &pc, stream);
   if (rc) return rc;
   if (pc.split == 0) {
-    // a tile kernel without split: the residual is added in its epilogue, the norm + quantiser kernel follows on the
+    // a tile kernel without split, or column strips: the residual is added in its epilogue, the norm + quantiser kernel follows on the
     // stored hidden state (the same two operations on the same values as behind planes, without the fp32 round trip)
-    hipError_t e = llmmm::fp8_gemm_add_residual_launch(hidden_dtype, pc.tile, pc.b_layout, A, As, Bt, Bs, residual, hidden_out, M, N, K, (hipStream_t)stream);
+    hipError_t e = pc.strip ? llmmm::fp8_strip_add_residual_launch(hidden_dtype, pc.b_layout, A, As, Bt, Bs, residual, hidden_out, M, N, K, (hipStream_t)stream)
+                            : llmmm::fp8_gemm_add_residual_launch(hidden_dtype, pc.tile, pc.b_layout, A, As, Bt, Bs, residual, hidden_out, M, N, K, (hipStream_t)stream);
     if (e == hipSuccess) e = llmmm::rmsnorm_quant_launch(hidden_dtype, hidden_out, norm_weight, eps, q, q_scale, M, N, (hipStream_t)stream);
     if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "fp8 gemm + add, rmsnorm + quantiser launch: %s", hipGetErrorString(e));
     return LLMMM_OK;

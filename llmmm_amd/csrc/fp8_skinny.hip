@@ -530,6 +530,204 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Column strips: one launch for the shapes whose few 128-column groups make the kernel above split K over several
+// workgroups and leave the sum to a second kernel (the 2560-column projections O and down, QKV).  A workgroup owns 16
+// output columns -- one wave's worth of weight rows -- over ALL of K; its eight waves take eight consecutive ranges of
+// 128-K slices, each with the wave-private ring of the kernel above, and their partial sums meet in LDS, where they are
+// added in wave order 0 .. 7: a fixed order, so results are the same run after run, with no planes, no workspace and no
+// second launch.  N / 16 workgroups (160 for 2560 columns) stream the weights at the rate N / 128 x S workgroups of the
+// split kernel did.  A strip holds an eighth of a 1x128 quantisation group, so this form serves the outputs without
+// such groups: fp32, bf16, and hidden = T(C + residual) for the projections that end a decoder block.
+// The activations come straight from global memory (L2) into the operand registers, slice by slice (M <= 32 rows).
+enum { ST_OUT_F32 = 0, ST_OUT_BF16 = 1, ST_OUT_ADD = 2 };
+
+template <int MBLK, int OUT, int D, bool TAIL, typename HT>
+__global__ void __launch_bounds__(512)
+fp8_strip_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt, const float* __restrict__ Bs,
+                 void* __restrict__ Cv, const HT* __restrict__ residual, int M, int N, int K, int bpre)
+{
+  constexpr int LOADS = SKINNY_LOADS_PER_SLOT_BASE + 3 * MBLK;
+  static_assert((D + (TAIL ? 1 : 0)) * LOADS < 64, "vmcnt is a 6-bit counter");
+  static_assert(D >= 2 && D <= 4, "ring depths in use");
+  __shared__ __attribute__((aligned(1024))) char ring0[8 * 2048];
+  __shared__ __attribute__((aligned(1024))) char ring1[8 * 2048];
+  __shared__ __attribute__((aligned(1024))) char ring2[D > 2 ? 8 * 2048 : 16];
+  __shared__ __attribute__((aligned(1024))) char ring3[D > 3 ? 8 * 2048 : 16];
+  __shared__ __attribute__((aligned(1024))) char tail_slot[TAIL ? 8 * 2048 : 16];
+  __shared__ f32x4 part[8][MBLK][64];  // the waves' partial sums, lane for lane
+
+  const int tid  = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int g    = lane >> 4;
+  const int i    = lane & 15;
+  const int n0   = blockIdx.x * 16;
+  const int KB   = K >> 7;
+  // K is dealt in whole slices: every wave takes q = KB / 8 consecutive slices through its ring (q >= 1: the host checks
+  // KB >= 8), and the KB % 8 slices behind them go one each to the first waves as a "tail" slice, requested before
+  // anything else and consumed last -- so the ring never runs over slices that are not the wave's own.  TAIL = (KB % 8 != 0).
+  const int q    = KB >> 3;
+  const int kb0  = wave * q, kb1 = kb0 + q;
+  const int kbt  = 8 * q + wave;        // the wave's tail slice ...
+  const bool has_tail = kbt < KB;        // ... if there is one (otherwise the last slice is fetched in its place and not used)
+
+  char LLMMM_LDS* const ring[4] = {(char LLMMM_LDS*)ring0 + wave * 2048, (char LLMMM_LDS*)ring1 + wave * 2048,
+                                   (char LLMMM_LDS*)ring2 + wave * 2048, (char LLMMM_LDS*)ring3 + wave * 2048};
+  char LLMMM_LDS* const tail = (char LLMMM_LDS*)tail_slot + wave * 2048;
+  unsigned ring_addr[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) ring_addr[u] = __builtin_amdgcn_readfirstlane((unsigned)(size_t)ring[u]);
+  const unsigned tail_addr = __builtin_amdgcn_readfirstlane((unsigned)(size_t)tail);
+
+  // the strip's 16 weight rows: row-major Bt[N,K], or the pre-shuffled image, whose 2 KB blocks of consecutive slices follow each other
+  const uint8_t*   wrow    = Bt + (size_t)n0 * K;
+  const KMajorLane l0      = kmajor_lane<SWZ_ROWS16>(0, lane);
+  const KMajorLane l1      = kmajor_lane<SWZ_ROWS16>(1, lane);
+  const unsigned   w_off0  = bpre ? (unsigned)lane * 16u : (unsigned)(l0.row * K + l0.chunk * 16);
+  const unsigned   w_off1  = bpre ? 1024u + (unsigned)lane * 16u : (unsigned)(l1.row * K + l1.chunk * 16);
+  const int        w_kstep = bpre ? 2048 : 128;
+  const int        w_rd    = kmajor_offset<SWZ_ROWS16>(i, 2 * g);
+  const float*     bsp     = Bs + (size_t)(n0 >> 7) * KB;
+  const uint8_t*   ap[MBLK];
+  const float*     asp[MBLK];
+#pragma unroll
+  for (int mb = 0; mb < MBLK; ++mb) {
+    const int m = min(mb * 16 + i, M - 1);  // rows beyond M repeat the last row; their sums are never stored
+    ap[mb]      = A + (size_t)m * K + 32 * g;
+    asp[mb]     = As + m;
+  }
+  f32x4 acc[MBLK];
+#pragma unroll
+  for (int mb = 0; mb < MBLK; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // the tail slice first (the oldest loads in flight: landed whenever a ring slot has), then the wave's q slices through
+  // its ring, D in flight (the pipeline of fp8_skinny_kernel)
+  SkinnySlot<MBLK, false> tslot;
+  if constexpr (TAIL) {
+    skinny_fetch<MBLK, false>(tslot, tail_addr, wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kbt, KB - 1), M);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  SkinnySlot<MBLK, false> slot[D];
+#pragma unroll
+  for (int u = 0; u < D; ++u) {
+    skinny_fetch<MBLK, false>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb0 + u, kb1 - 1), M);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  int kb = kb0;
+  for (; kb + D < kb1; kb += D) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      skinny_wait<(D - 1) * LOADS, MBLK, false>(slot[u]);
+      skinny_consume<MBLK, false>(slot[u], ring[u], w_rd, true, acc, nullptr, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      skinny_fetch<MBLK, false>(slot[u], ring_addr[u], wrow, w_kstep, w_off0, w_off1, ap, asp, bsp, min(kb + u + D, kb1 - 1), M);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+#define LLMMM_LAST(u)                                                                 \
+  if constexpr ((u) < D) {                                                            \
+    skinny_wait<(D - 1 - (u)) * LOADS, MBLK, false>(slot[u]);                          \
+    skinny_consume<MBLK, false>(slot[u], ring[u], w_rd, kb + (u) < kb1, acc, nullptr, 0); \
+    __builtin_amdgcn_sched_barrier(0);                                                \
+  }
+  LLMMM_LAST(0) LLMMM_LAST(1) LLMMM_LAST(2) LLMMM_LAST(3)
+#undef LLMMM_LAST
+  if constexpr (TAIL) {
+    skinny_wait<0, MBLK, false>(tslot);  // (long landed; ties its registers to this point)
+    skinny_consume<MBLK, false>(tslot, tail, w_rd, has_tail, acc, nullptr, 0);
+  }
+
+#pragma unroll
+  for (int mb = 0; mb < MBLK; ++mb) part[wave][mb][lane] = acc[mb];
+  __syncthreads();
+  if (wave >= MBLK) return;  // wave mb finishes the 16-row block mb
+  const int mb = wave;
+  f32x4     v  = part[0][mb][lane];
+#pragma unroll
+  for (int w = 1; w < 8; ++w) v += part[w][mb][lane];  // wave order: the same sum whatever the waves' timing
+  const int m = mb * 16 + i, ncol = n0 + 4 * g;  // lane (g, i): row m, columns ncol .. ncol + 3
+  if (m >= M) return;
+  if constexpr (OUT == ST_OUT_F32)
+    *(f32x4*)((float*)Cv + (size_t)m * N + ncol) = v;
+  else if constexpr (OUT == ST_OUT_BF16)
+    store_row4<__bf16>((__bf16*)Cv + (size_t)m * N + ncol, v);
+  else {
+    const f32x4 r = load_row4<HT>(residual + (size_t)m * N + ncol);
+    store_row4<HT>((HT*)Cv + (size_t)m * N + ncol, v + r);  // one fp32 addition per element, then the hidden type's rounding
+  }
+}
+
+// Ring depth: of 4, 3 and 2 the one that runs over the fewest slices beyond the q = K / 128 / 8 of a wave (a pass past
+// the end re-fetches the last slice: wasted loads cost more here than a shallow ring -- down at M = 1, 9 slices per
+// wave: 8.3 us with an 8-deep ring, 6.5 us with a 2-deep one); the deeper ring on ties.
+template <int MBLK, int OUT, typename HT>
+static hipError_t launch_strip(const void* A, const float* As, const void* Bt, const float* Bs, void* C, const void* residual, int M, int N, int K, int bpre,
+                               hipStream_t stream)
+{
+  const int  q = (K / 128) / 8;
+  const dim3 grid(N / 16), block(512);
+  int        best = 2, waste = 1 << 30;
+  for (int d = 4; d >= 2; --d) {
+    const int w = (q + d - 1) / d * d - q;
+    if (w < waste) best = d, waste = w;
+  }
+  const bool tail = (K / 128) % 8 != 0;
+#define LLMMM_GO(D)                                                                                                                                         \
+  if (tail)                                                                                                                                                 \
+    hipLaunchKernelGGL((fp8_strip_kernel<MBLK, OUT, D, true, HT>), grid, block, 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, (const HT*)residual, \
+                       M, N, K, bpre);                                                                                                                      \
+  else                                                                                                                                                      \
+    hipLaunchKernelGGL((fp8_strip_kernel<MBLK, OUT, D, false, HT>), grid, block, 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, (const HT*)residual, \
+                       M, N, K, bpre)
+  if (best == 4) {
+    LLMMM_GO(4);
+  }
+  else if (best == 3) {
+    LLMMM_GO(3);
+  }
+  else {
+    LLMMM_GO(2);
+  }
+#undef LLMMM_GO
+  return hipGetLastError();
+}
+
+hipError_t fp8_strip_launch(int out_kind, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C, int M, int N, int K,
+                            hipStream_t stream)
+{
+  if (M < 1 || M > STRIP_MAX_M || N % 16 || K % 128 || K / 128 < 8) return hipErrorInvalidValue;
+  const int bpre = b_layout == LLMMM_FP8_B_PRESHUFFLED;
+  if (out_kind == LLMMM_OUT_F32)
+    return M <= 16 ? launch_strip<1, ST_OUT_F32, float>(A, As, Bt, Bs, C, nullptr, M, N, K, bpre, stream)
+                   : launch_strip<2, ST_OUT_F32, float>(A, As, Bt, Bs, C, nullptr, M, N, K, bpre, stream);
+  if (out_kind == LLMMM_OUT_BF16)
+    return M <= 16 ? launch_strip<1, ST_OUT_BF16, float>(A, As, Bt, Bs, C, nullptr, M, N, K, bpre, stream)
+                   : launch_strip<2, ST_OUT_BF16, float>(A, As, Bt, Bs, C, nullptr, M, N, K, bpre, stream);
+  return hipErrorInvalidValue;
+}
+
+template <typename HT>
+static hipError_t strip_add(int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, const void* residual, void* hidden, int M, int N, int K,
+                            hipStream_t stream)
+{
+  const int bpre = b_layout == LLMMM_FP8_B_PRESHUFFLED;
+  return M <= 16 ? launch_strip<1, ST_OUT_ADD, HT>(A, As, Bt, Bs, hidden, residual, M, N, K, bpre, stream)
+                 : launch_strip<2, ST_OUT_ADD, HT>(A, As, Bt, Bs, hidden, residual, M, N, K, bpre, stream);
+}
+
+hipError_t fp8_strip_add_residual_launch(int hidden_dtype, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, const void* residual,
+                                         void* hidden, int M, int N, int K, hipStream_t stream)
+{
+  if (M < 1 || M > STRIP_MAX_M || N % 16 || K % 128 || K / 128 < 8) return hipErrorInvalidValue;
+  switch (hidden_dtype) {
+    case LLMMM_DTYPE_F32: return strip_add<float>(b_layout, A, As, Bt, Bs, residual, hidden, M, N, K, stream);
+    case LLMMM_DTYPE_BF16: return strip_add<__bf16>(b_layout, A, As, Bt, Bs, residual, hidden, M, N, K, stream);
+    case LLMMM_DTYPE_F16: return strip_add<_Float16>(b_layout, A, As, Bt, Bs, residual, hidden, M, N, K, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
 template <int MBLK, int OUT, int D, int ASTG>
 static hipError_t launch_skinny(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
                                 int N, int K, int S, float* partial, int bpre, hipStream_t stream)

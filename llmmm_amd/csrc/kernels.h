@@ -56,6 +56,17 @@ hipError_t fp8_splitk_reduce_launch(int out_kind, const float* planes, int S, vo
 hipError_t fp8_skinny_launch(int out_kind, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
                              float* Cs, int M, int N, int K, int S, float* partial, hipStream_t stream);
 
+// The weight-streaming kernel in column strips: a workgroup owns 16 output columns over all of K, its eight waves split K and
+// add their sums in LDS in wave order -- one launch, no planes, deterministic.  M <= STRIP_MAX_M, N % 16 == 0,
+// K % 128 == 0, K >= 1024; out_kind LLMMM_OUT_F32 or LLMMM_OUT_BF16 (no 1x128-grouped outputs: a strip holds an eighth
+// of a group).  hipErrorInvalidValue outside these limits.
+constexpr int STRIP_MAX_M = 32;
+hipError_t fp8_strip_launch(int out_kind, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C, int M, int N, int K,
+                            hipStream_t stream);
+// The same with hidden = T(C + residual) as its output (T = hidden_dtype, LLMMM_DTYPE_*; hidden may be the residual buffer).
+hipError_t fp8_strip_add_residual_launch(int hidden_dtype, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, const void* residual,
+                                         void* hidden, int M, int N, int K, hipStream_t stream);
+
 // What the weight-streaming kernel needs to make its activations from a hidden state that is still in pieces.
 constexpr int SKINNY_GEN_MAX_PLANES = 10;
 struct SkinnyGenA {

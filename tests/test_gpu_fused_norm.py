@@ -108,7 +108,7 @@ def test_equals_the_separate_calls(lib, oracle):
 
 
 def test_workspace_and_errors(lib):
-    M, N, K = 16, 2560, 4096
+    M, N, K = 48, 2560, 4096  # (up to 16 rows this shape runs in column strips, which need no workspace)
     need = lib._lib.lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K)
     assert need >= M * N * 4 and need % (M * N * 4) == 0
     A = torch.zeros((M, K), dtype=torch.uint8, device="cuda")

@@ -35,7 +35,11 @@ def _run(lib, oracle, M, K, n_q, n_kv, tile, split, norm=True, pre=False, seed=0
         dB = lib.preshuffle_weight(dB)
     ws = torch.full((16 * M * N * 4,), 0xFF, dtype=torch.uint8, device="cuda")
     C = torch.empty((M, N), dtype=torch.float32, device="cuda")
-    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dA, dAs, dB, dBs, C, M, N, K, workspace=ws, tile=tile, split_k=split, b_preshuffled=pre)
+    # the fp32 result of the kernel the fused call runs: with the library's own choice that is the choice for 1x128-grouped
+    # outputs (heads are such groups), not the column strips a plain fp32 output takes at decode sizes
+    from llmmm_amd import _lib
+    plain_tile = lib.query_config(_lib.OUT_FP8Q, M, N, K)[0] if tile == TILES["auto"] and split == 0 else tile
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dA, dAs, dB, dBs, C, M, N, K, workspace=ws, tile=plain_tile, split_k=split, b_preshuffled=pre)
     torch.cuda.synchronize()
     want = oracle.qk_norm_rope(C.cpu().numpy(), qw, kw, 1e-6, cos, sin, pos, n_q, n_kv)
     args = (dA, dAs, dB, dBs, g(qw), g(kw), 1e-6, g(cos), g(sin), g(pos), n_q, n_kv, M, N, K)

@@ -20,8 +20,9 @@ def _both(raw, out_kind, M, N, K, t, stream):
     """One call of each entry point on the same device operands; returns the two (C, Cs) pairs as numpy arrays."""
     from llmmm_amd import _lib
     need = raw.llmmm_fp8_gemm_workspace(out_kind, M, N, K)
-    assert 0 < need <= _lib.STATIC_WS_BYTES, "the case must split K and fit the built-in array"
-    ws = torch.full((need,), 0xA5, dtype=torch.uint8, device="cuda")
+    assert need <= _lib.STATIC_WS_BYTES, "the case must fit the built-in array"
+    assert need > 0 or out_kind != _lib.OUT_FP8Q, "the fused-quant case must split K"  # (fp32 / bf16 may run in column strips: no planes)
+    ws = torch.full((max(need, 16),), 0xA5, dtype=torch.uint8, device="cuda")
     dt = {0: torch.float32, 1: torch.bfloat16, 2: torch.uint8}[out_kind]
     outs = []
     for static in (False, True):
@@ -42,9 +43,9 @@ def test_static_workspace_matches_caller_workspace(oracle):
     from llmmm_amd import _lib
     raw = _lib.lib
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
-    # first the larger problem (16 x 6144 x 2560, split 5: 1.9 MB of planes), then a smaller one (1 x 2560 x 4096,
-    # split 8: 80 KB) that finds the first call's partial sums still in the array
-    for M, N, K, seed in ((16, 6144, 2560, 11), (1, 2560, 4096, 12)):
+    # first the larger problem (64 x 6144 x 2560, split 5: 7.9 MB of planes for every output kind), then a smaller one
+    # (1 x 2560 x 4096, split 8: 80 KB for the fused output) that finds the first call's partial sums still in the array
+    for M, N, K, seed in ((64, 6144, 2560, 11), (1, 2560, 4096, 12)):
         Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=seed)
         t = [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (Aq, As, Bq, Bs)]
         ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
