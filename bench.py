@@ -535,6 +535,68 @@ def bench_targets(steps, warmup, headline=None):
     return t
 
 
+def phase_accounting(kind, M=4096, N=4096, K=4096, launches=40):
+    """Where one launch of the 256 x 256 tile kernel spends its time (llmmm_probe_*_gemm_phases: the product kernel with clock
+    readings at five points of every wave).  Runs `launches` instrumented launches back to back (the clocks settle), reads the
+    stamps of the last one and returns per-phase times over all waves, in microseconds of the 100 MHz clock and in shader cycles."""
+    import llmmm_amd
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    nbytes = lib.llmmm_probe_phases_bytes(M, N)
+    stamps = torch.zeros(nbytes // 8, dtype=torch.int64, device="cuda")
+    if kind == "fp8":
+        Aq, As, weights = fp8_inputs(M, N, K)
+        Bq, Bs = weights[0]
+        C = torch.empty((M, N), dtype=torch.uint8, device="cuda")
+        Cs = torch.empty((N // 128, M), dtype=torch.float32, device="cuda")
+
+        def probe():
+            assert lib.llmmm_probe_fp8_gemm_phases(Aq.data_ptr(), As.data_ptr(), Bq.data_ptr(), Bs.data_ptr(), C.data_ptr(), Cs.data_ptr(), M, N, K,
+                                                   stamps.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream) == 0
+
+        def plain():
+            llmmm_amd.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(Aq, As, Bq, Bs, C, Cs, M, N, K, tile=_lib.TILE_256x256)
+    else:
+        A, B = fp16_inputs(M, N, K)
+        C = torch.empty((M, N), dtype=torch.float16, device="cuda")
+
+        def probe():
+            assert lib.llmmm_probe_fp16_gemm_phases(_lib.DTYPE_F16, A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, stamps.data_ptr(), nbytes,
+                                                    torch.cuda.current_stream().cuda_stream) == 0
+
+        def plain():
+            llmmm_amd.fp16_gemm(A, B, C, tile=_lib.TILE_256x256)
+    ms_plain, _ = _events_ms(plain, launches, 5, graph=True)
+    ms_probe, _ = _events_ms(probe, launches, 5, graph=True)
+    torch.cuda.synchronize()
+    rec = stamps.cpu().numpy().reshape(-1, 12).astype(np.float64)
+    t = rec[:, :10].reshape(-1, 5, 2)  # [wave, point, (100 MHz ticks, shader cycles)]
+    real, cyc = t[:, :, 0], t[:, :, 1]
+    wait_cy = rec[:, 10]
+    t0 = real[:, 0].min()
+    names = ["prologue (entry -> first operands in LDS)", "K loop", "epilogue (amax / convert / staging / stores issued)", "store drain (stores acknowledged)"]
+    out = {"kernel_us_uninstrumented": ms_plain * 1e3, "kernel_us_instrumented": ms_probe * 1e3, "waves": int(t.shape[0]),
+           "first_wave_start_to_last_wave_end_us": (real[:, 4].max() - t0) / 100.0, "wave_start_spread_us": (real[:, 0].max() - t0) / 100.0, "phases": []}
+    for p, name in enumerate(names):
+        d_us = (real[:, p + 1] - real[:, p]) / 100.0
+        d_cy = cyc[:, p + 1] - cyc[:, p]
+        out["phases"].append({"phase": name, "us_median": float(np.median(d_us)), "us_mean": float(d_us.mean()), "us_min": float(d_us.min()), "us_max": float(d_us.max()),
+                              "cycles_median": float(np.median(d_cy))})
+    whole_cy = cyc[:, 4] - cyc[:, 0]
+    whole_us = (real[:, 4] - real[:, 0]) / 100.0
+    out["wave_lifetime_us_median"] = float(np.median(whole_us))
+    out["shader_mhz_from_stamps"] = float(np.median(whole_cy / whole_us))
+    loop_cy = float(np.median(cyc[:, 2] - cyc[:, 1]))
+    slices = K // 128 if kind == "fp8" else K // 32
+    out["k_loop_cycles_per_stage"] = loop_cy / slices
+    # a SIMD holds two waves; per stage each issues 32 MFMAs of 32 cycles (fp8 16x16x128, a 128-K slice) or of 16 cycles (f16 16x16x32, K = 32)
+    out["k_loop_wait_cycles_per_stage"] = float(np.median(wait_cy)) / slices
+    ideal = 2048.0 if kind == "fp8" else 1024.0
+    out["k_loop_ideal_cycles_per_stage"] = ideal
+    out["k_loop_matrix_pipe_share"] = ideal / out["k_loop_cycles_per_stage"]
+    return out
+
+
 def cpu_baseline(M, N, K, rows):
     """The CPU oracle on this host's cores, bounded samples of the GPU workloads: the Kahan GEMM (the headline's
     reference, a port of test/kahan.cu:16-26) on the first `rows` rows of the FP16 workload, and beside it the
@@ -582,7 +644,8 @@ def main():
     ap.add_argument("--workload", default="fp16_gemm_4096",
                     help="fp16_gemm_4096 (headline) | fp16_gemm_2048x19456x2560 | fp8_gemm_fused_4096 | fp8_gemm_bf16_4096 | bf16_gemm_4096 | "
                          "decode_<qkv|o|gate_up|down>_m<M>[_pre] (_pre: weights pre-shuffled offline) | prefill_<qkv|o|gate_up|down>_m<M> | "
-                         "prefill_gate_up_swiglu_m<M> | fused_<o|down>_add_norm_m<M> | fused_qkv_rope_m<M> | layer_[consumer_]m<M> | copy_1g (counter calibration only)")
+                         "prefill_gate_up_swiglu_m<M> | fused_<o|down>_add_norm_m<M> | fused_qkv_rope_m<M> | layer_[consumer_]m<M> | copy_1g (counter calibration only) | "
+                         "phases_fp8_4096 | phases_fp16_4096 (where a launch of the tile kernel spends its time; prints a table)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measured-peak probes")
@@ -609,6 +672,22 @@ def main():
         ms, _ = _events_ms(lambda: dst.copy_(src), args.steps, args.warmup)
         print(json.dumps({"workload": "copy_1g", "read_bytes": 1 << 30, "write_bytes": 1 << 30, "ms_per_step": ms,
                           "gbs": 2.0 * (1 << 30) / ms * 1e-6}))
+        return
+    if w in ("phases_fp8_4096", "phases_fp16_4096"):
+        kind = "fp8" if "fp8" in w else "fp16"
+        r = phase_accounting(kind)
+        print("phase accounting, %s 256 x 256 tile kernel, M = N = K = 4096 (one tile per CU, 8 waves per tile)" % ("FP8 fused-quant" if kind == "fp8" else "FP16"))
+        print("kernel time per launch (HIP events, graph of back-to-back launches): %.2f us; the instrumented build: %.2f us" %
+              (r["kernel_us_uninstrumented"], r["kernel_us_instrumented"]))
+        print("first wave's start to last wave's end: %.2f us; wave starts spread over %.2f us; median wave lifetime %.2f us; shader clock %.0f MHz" %
+              (r["first_wave_start_to_last_wave_end_us"], r["wave_start_spread_us"], r["wave_lifetime_us_median"], r["shader_mhz_from_stamps"]))
+        print("%-62s %9s %9s %9s %9s %12s" % ("phase (per wave, %d waves)" % r["waves"], "median us", "mean us", "min us", "max us", "median cyc"))
+        for p in r["phases"]:
+            print("%-62s %9.2f %9.2f %9.2f %9.2f %12.0f" % (p["phase"], p["us_median"], p["us_mean"], p["us_min"], p["us_max"], p["cycles_median"]))
+        print("K loop: %.0f cycles per stage against %.0f with the matrix pipe always busy (two waves per SIMD, 32 MFMAs each per stage): %.1f %%" %
+              (r["k_loop_cycles_per_stage"], r["k_loop_ideal_cycles_per_stage"], 100 * r["k_loop_matrix_pipe_share"]))
+        print("of which a wave waits %.0f cycles per stage for its loads to land and for the other waves (vmcnt + barrier)" % r["k_loop_wait_cycles_per_stage"])
+        print(json.dumps({"workload": w, **r}))
         return
     if w in ("fp16_gemm_4096", "bf16_gemm_4096"):
         dt = torch.float16 if w.startswith("fp16") else torch.bfloat16

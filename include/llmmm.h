@@ -278,6 +278,19 @@ LLMMM_API int    llmmm_probe_mfma(int kind, const void* operands, float* sink, i
 LLMMM_API double llmmm_probe_mfma_flops(int kind, int workgroups, int iters);
 LLMMM_API int    llmmm_probe_hbm_read(const void* src, size_t bytes, float* sink, int workgroups, void* stream);
 
+/* Where a launch of the 256 x 256 tile kernels spends its time.  These run the product kernels of llmmm_fp8_gemm(LLMMM_OUT_FP8Q)
+ * / llmmm_fp16_gemm at M, N multiples of 256 (row-major operands), built with clock readings at five points of every wave:
+ * 0 kernel entry, 1 first operands in LDS (end of the prologue), 2 end of the K loop, 3 last store issued, 4 stores acknowledged.
+ * stamps: device memory of llmmm_probe_phases_bytes(M, N) bytes; afterwards, as 64-bit words, record (t * 8 + w) * 12 of
+ * workgroup t and wave w (8 per workgroup) holds at [2 p] the constant 100 MHz clock at point p, at [2 p + 1] the shader's
+ * cycle counter, and at [10] the shader cycles the wave spent waiting in the K loop (loads landed + barrier of every stage).
+ * The reference measures its kernels from outside only (ncu.sh); no counterpart. */
+LLMMM_API size_t llmmm_probe_phases_bytes(int M, int N);
+LLMMM_API int    llmmm_probe_fp8_gemm_phases(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K,
+                                             void* stamps, size_t stamps_bytes, void* stream);
+LLMMM_API int    llmmm_probe_fp16_gemm_phases(int dtype, const void* A, const void* B, void* C, int M, int N, int K, void* stamps, size_t stamps_bytes,
+                                              void* stream);
+
 /* ---- misc ------------------------------------------------------------------------------- */
 LLMMM_API const char* llmmm_error_string(int code); /* the reference's exception texts for codes 1 and 2 */
 LLMMM_API const char* llmmm_last_error(void);       /* thread-local detail of the last failure */

@@ -726,6 +726,38 @@ static size_t plane_route_workspace(int M, int N, int K, bool wide_ok)
   return (size_t)split * M * N * sizeof(float);
 }
 
+size_t llmmm_probe_phases_bytes(int M, int N)
+{
+  if (M <= 0 || N <= 0 || M % 256 || N % 256) return 0;
+  return (size_t)(M / 256) * (N / 256) * 8 * llmmm::PHASE_RECORD * sizeof(unsigned long long);
+}
+
+int llmmm_probe_fp8_gemm_phases(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K, void* stamps,
+                                size_t stamps_bytes, void* stream)
+{
+  if (M <= 0 || N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "M, N and K must be positive (got %d, %d, %d)", M, N, K);
+  if (M % 256 || N % 256 || K % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+  if (!A || !As || !Bt || !Bs || !C || !Cs || !stamps) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (!aligned16(A) || !aligned16(Bt) || !aligned16(C) || !aligned16(stamps)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+  if (stamps_bytes < llmmm_probe_phases_bytes(M, N)) return fail(LLMMM_ERR_WORKSPACE, "stamps holds %zu bytes, %zu needed", stamps_bytes, llmmm_probe_phases_bytes(M, N));
+  const hipError_t e = llmmm::fp8_gemm_phases_launch(A, As, Bt, Bs, C, Cs, M, N, K, (unsigned long long*)stamps, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "probe launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
+int llmmm_probe_fp16_gemm_phases(int dtype, const void* A, const void* B, void* C, int M, int N, int K, void* stamps, size_t stamps_bytes, void* stream)
+{
+  if (dtype != LLMMM_DTYPE_F16 && dtype != LLMMM_DTYPE_BF16) return fail(LLMMM_ERR_UNSUPPORTED_TYPE, "T is not supported.");
+  if (M <= 0 || N <= 0 || K <= 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "M, N and K must be positive (got %d, %d, %d)", M, N, K);
+  if (M % 256 || N % 256 || K % 32) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
+  if (!A || !B || !C || !stamps) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  if (!aligned16(A) || !aligned16(B) || !aligned16(C) || !aligned16(stamps)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "pointers must be 16-byte aligned");
+  if (stamps_bytes < llmmm_probe_phases_bytes(M, N)) return fail(LLMMM_ERR_WORKSPACE, "stamps holds %zu bytes, %zu needed", stamps_bytes, llmmm_probe_phases_bytes(M, N));
+  const hipError_t e = llmmm::fp16_gemm_phases_launch(dtype, A, B, C, M, N, K, (unsigned long long*)stamps, (hipStream_t)stream);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "probe launch: %s", hipGetErrorString(e));
+  return LLMMM_OK;
+}
+
 size_t llmmm_fp8_gemm_add_rmsnorm_quant_workspace(int M, int N, int K) { return plane_route_workspace(M, N, K, true); }
 
 // Kernel and split for the entry points whose epilogue lives in a second kernel behind fp32 planes, chosen and

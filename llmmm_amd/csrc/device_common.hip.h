@@ -97,6 +97,19 @@ __device__ __forceinline__ void wait_vmcnt()
   __builtin_amdgcn_s_waitcnt((N & 15) | 0x70 | ((N >> 4) << 14));
 }
 
+// Clock readings for the phase-accounting builds of the tile kernels: the constant 100 MHz counter and the shader's cycle
+// counter (scalar reads; the values are stored with ordinary vector stores at the end of the kernel).
+struct PhaseClock {
+  unsigned long long real, cycles;
+};
+__device__ __forceinline__ PhaseClock phase_clock()
+{
+  PhaseClock c;
+  c.real   = __builtin_amdgcn_s_memrealtime();
+  c.cycles = __builtin_amdgcn_s_memtime();
+  return c;
+}
+
 // Logical tile id -> (tm, tn).  Hardware hands consecutive workgroup ids to the 8 XCDs in turn,
 // so ids congruent mod 8 share an L2: give each XCD a contiguous run of the grouped order
 // (GROUP_M tile rows swept along n), whose members reuse the same few A and B panels.

@@ -170,13 +170,17 @@ __device__ __forceinline__ void fp16_mfma8(int half, int part, const typename Mf
 
 // The kernel's body for tile `tile_index` of the tiles_m x tiles_n tiles of the column range that starts at n_base (0 and
 // the whole matrix for the plain kernel); lds_raw: the workgroup's ring of four stages.
-template <typename T, int BM, int BN, int WM, bool B_NK, bool KTAIL>
+// STAMP: the phase-accounting build -- clock readings at five points of every wave, stored to `stamps` at the end.
+template <typename T, int BM, int BN, int WM, bool B_NK, bool KTAIL, bool STAMP = false>
 __device__ __forceinline__ void fp16_gemm_body(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K, int tiles_m,
-                                               int tiles_n, char LLMMM_LDS* lds_raw, int tile_index, int n_base)
+                                               int tiles_n, char LLMMM_LDS* lds_raw, int tile_index, int n_base, unsigned long long* stamps = nullptr)
 {
   typedef Fp16Tile<T, BM, BN, WM, B_NK> TC;
   typedef typename Mfma32<T>::vec   vec;
   constexpr int                     MF = TC::MF;
+  PhaseClock                        ph[STAMP ? PHASE_POINTS : 1];
+  unsigned long long                wait_cycles = 0;  // STAMP: shader cycles in the K loop's "loads landed + barrier" waits
+  if constexpr (STAMP) ph[0] = phase_clock();
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -259,6 +263,7 @@ __device__ __forceinline__ void fp16_gemm_body(const T* __restrict__ A, const T*
   else
     wait_vmcnt<0>();
   __builtin_amdgcn_s_barrier();
+  if constexpr (STAMP) ph[1] = phase_clock();
   if (3 < KT) LLMMM_ISSUE(3, 3);
 
   vec aX[MF], aY[MF], bL[4], bR[4];  // A fragments of the current / next stage; B fragments of the left / right 64 columns
@@ -278,6 +283,8 @@ __device__ __forceinline__ void fp16_gemm_body(const T* __restrict__ A, const T*
     __builtin_amdgcn_sched_barrier(0);                                                                             \
     /* every LDS read of stage s has been issued; once they are back (lgkmcnt(0), part of each wait below) the */ \
     /* barrier hands ring[u] to the loader and publishes stage s+1 */                                             \
+    unsigned long long tw_ = 0;                                                                                    \
+    if constexpr (STAMP) tw_ = __builtin_amdgcn_s_memtime();                                                       \
     if (STEADY || (s) + 3 < full_stages)                                                                           \
       wait_vmcnt<2 * TC::LOADS>(); /* stages s+2 and s+3 may still be in flight */                                 \
     else if ((s) + 2 < full_stages)                                                                                \
@@ -285,6 +292,7 @@ __device__ __forceinline__ void fp16_gemm_body(const T* __restrict__ A, const T*
     else                                                                                                           \
       wait_vmcnt<0>();                                                                                             \
     __builtin_amdgcn_s_barrier();                                                                                  \
+    if constexpr (STAMP) wait_cycles += __builtin_amdgcn_s_memtime() - tw_;                                        \
     if (STEADY || (s) + 4 < KT) LLMMM_ISSUE((s) + 4, u);                                                           \
     fp16_mfma8<T, MF>(1, 0, aC, bR, acc);                                                                              \
     __builtin_amdgcn_sched_barrier(0);                                                                             \
@@ -311,6 +319,7 @@ __device__ __forceinline__ void fp16_gemm_body(const T* __restrict__ A, const T*
   }
 #undef LLMMM_STAGE
 #undef LLMMM_ISSUE
+  if constexpr (STAMP) ph[2] = phase_clock();
 
   // ---- epilogue: lane (g, li) holds rows m = .. + mf*16 + li, columns nf*16 + 4g + r.
   // Stored straight from this layout, one instruction would write 8 bytes to each of 16 rows,
@@ -344,6 +353,26 @@ __device__ __forceinline__ void fp16_gemm_body(const T* __restrict__ A, const T*
       *(i32x4*)(cbase + (size_t)r * N + ch * 8) = v;
     }
   }
+  if constexpr (STAMP) {
+    ph[3] = phase_clock();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores are acknowledged
+    ph[4] = phase_clock();
+    if (lane == 0) {
+      unsigned long long* o = stamps + ((size_t)tile_index * TC::NW + wave) * PHASE_RECORD;
+#pragma unroll
+      for (int p = 0; p < PHASE_POINTS; ++p) o[2 * p] = ph[p].real, o[2 * p + 1] = ph[p].cycles;
+      o[PHASE_STAMPS] = wait_cycles;
+    }
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(512)
+fp16_gemm_phases_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
+                        unsigned long long* stamps)
+{
+  __shared__ __attribute__((aligned(1024))) char lds_raw[4 * Fp16Tile<T, 256, 256, 64, false>::STAGE];
+  fp16_gemm_body<T, 256, 256, 64, false, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, (char LLMMM_LDS*)lds_raw, blockIdx.x, 0, stamps);
 }
 
 template <typename T, int BM, int BN, int WM, bool B_NK, bool KTAIL>
@@ -420,6 +449,19 @@ static hipError_t dispatch_fp16(int tile, const void* A, const void* B, void* C,
     case LLMMM_TILE_64x128: return launch_fp16<T, 64, 128, 16, B_NK>(A, B, C, M, N, K, stream);  // four 16-row waves: small problems
     default: return hipErrorInvalidValue;
   }
+}
+
+hipError_t fp16_gemm_phases_launch(int dtype, const void* A, const void* B, void* C, int M, int N, int K, unsigned long long* stamps, hipStream_t stream)
+{
+  if (M % 256 || N % 256 || K % 32 || !stamps) return hipErrorInvalidValue;
+  const int tiles_m = M / 256, tiles_n = N / 256;
+  if (dtype == 0)
+    hipLaunchKernelGGL((fp16_gemm_phases_kernel<_Float16>), dim3(tiles_m * tiles_n), dim3(512), 0, stream, (const _Float16*)A, (const _Float16*)B, (_Float16*)C, M,
+                       N, K, tiles_m, tiles_n, stamps);
+  else
+    hipLaunchKernelGGL((fp16_gemm_phases_kernel<__bf16>), dim3(tiles_m * tiles_n), dim3(512), 0, stream, (const __bf16*)A, (const __bf16*)B, (__bf16*)C, M, N, K,
+                       tiles_m, tiles_n, stamps);
+  return hipGetLastError();
 }
 
 hipError_t fp16_gemm_launch(int dtype, int b_layout, int tile, const void* A, const void* B, void* C, int M, int N, int K,

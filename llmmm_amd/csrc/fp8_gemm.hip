@@ -415,6 +415,11 @@ __device__ __forceinline__ void fp8_gemm_body(const uint8_t* __restrict__ A, con
   // BMODE bit 3 (MT, deep 128 x 128 tiles with the fp32 / bf16 / fp8 outputs only): M is not a multiple of BM; the rows
   // of the last tile row beyond the matrix are computed from copies of its last row and never stored.
   constexpr bool MT      = (BMODE & 8) != 0;
+  // BMODE bit 4 (STAMP): the phase-accounting build -- clock readings at five points of every wave, stored to op.stamps at the end
+  constexpr bool STAMP   = (BMODE & 16) != 0;
+  PhaseClock     ph[STAMP ? PHASE_POINTS : 1];
+  unsigned long long wait_cycles = 0;  // STAMP: shader cycles this wave spent in the K loop's "loads landed + barrier" waits (slices 1 ..)
+  if constexpr (STAMP) ph[0] = phase_clock();
   static_assert(!MT || (DEEP && BM == 128 && BN == 128 && (OUT == OUT_F32 || OUT == OUT_BF16 || OUT == OUT_FP8Q)), "row tails: deep 128 x 128 tiles only");
   constexpr int  STAGE_D = TC::STAGE + TC::NW * 256;                 // operands + 256 bytes of scales per wave
   constexpr int  NST     = !DEEP ? 2 : (4 * STAGE_D <= 160 * 1024 ? 4 : 3);
@@ -544,6 +549,8 @@ __device__ __forceinline__ void fp8_gemm_body(const uint8_t* __restrict__ A, con
   // slice ago), meet the other waves, then compute it while the loads of the next one go out.
 #define LLMMM_FP8_SLICE(LOAD, CUR, NXT_LDS, KC)                                                                                   \
   {                                                                                                                               \
+    unsigned long long tw_ = 0;                                                                                                   \
+    if constexpr (STAMP) tw_ = __builtin_amdgcn_s_memtime();                                                                      \
     wait_vmcnt<0>();                                                                                                              \
     if constexpr (MF == 4)                                                                                                        \
       asm volatile("" : "+v"(sa_next[0]), "+v"(sa_next[1]), "+v"(sa_next[2]), "+v"(sa_next[MF - 1]), "+v"(sb_next));              \
@@ -551,6 +558,12 @@ __device__ __forceinline__ void fp8_gemm_body(const uint8_t* __restrict__ A, con
       asm volatile("" : "+v"(sa_next[0]), "+v"(sa_next[1]), "+v"(sb_next));                                                       \
     if constexpr (TWO) asm volatile("" : "+v"(sb2_next));                                                                         \
     __syncthreads();                                                                                                              \
+    if constexpr (STAMP) {                                                                                                        \
+      if ((KC) == 0)                                                                                                              \
+        ph[1] = phase_clock();                                                                                                    \
+      else                                                                                                                        \
+        wait_cycles += __builtin_amdgcn_s_memtime() - tw_;                                                                        \
+    }                                                                                                                             \
     float s[MF], s2[MF];                                                                                                          \
     _Pragma("unroll") for (int mf = 0; mf < MF; ++mf) s[mf] = sa_next[mf] * sb_next, s2[mf] = sa_next[mf] * sb2_next;              \
     Fp8Next nx;                                                                                                                   \
@@ -579,6 +592,7 @@ __device__ __forceinline__ void fp8_gemm_body(const uint8_t* __restrict__ A, con
   // lays its WM x 128 result out row-major in a private 16 KB piece of the (now idle) operand
   // buffers -- 16-byte chunks XOR-ed with row bits so that neither the writes nor the
   // ds_read_b128 reads conflict -- and stores it back out 16 bytes per lane, whole rows at a time.
+  if constexpr (STAMP) ph[2] = phase_clock();
   __syncthreads();  // every wave is done reading the last operand stage
   // WM rows of up to 256 bytes (fp32 goes 16 rows at a time); 160-column waves pad their rows by 16 bytes instead of XOR-ing chunks
   constexpr int         RS32 = TC::WN * 4 + 16, RS16 = TC::WN * 2 + 16;  // padded row strides of the 160-column staging
@@ -738,6 +752,17 @@ __device__ __forceinline__ void fp8_gemm_body(const uint8_t* __restrict__ A, con
       const int   r = 8 * j + (lane >> 3), c = lane & 7;
       const i32x4 v = *(const i32x4 LLMMM_LDS*)(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
       if (!MT || row0 + r < M) *(i32x4*)(C + (size_t)(row0 + r) * N + col0 + c * 16) = v;
+    }
+  }
+  if constexpr (STAMP) {
+    ph[3] = phase_clock();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores are acknowledged
+    ph[4] = phase_clock();
+    if (lane == 0) {
+      unsigned long long* o = op.stamps + ((size_t)tile_index * TC::NW + wave) * PHASE_RECORD;
+#pragma unroll
+      for (int p = 0; p < PHASE_POINTS; ++p) o[2 * p] = ph[p].real, o[2 * p + 1] = ph[p].cycles;
+      o[PHASE_STAMPS] = wait_cycles;
     }
   }
 }
@@ -1051,6 +1076,18 @@ hipError_t fp8_gemm_launch(int out_kind, int tile, int b_layout, const void* A, 
     case OUT_SWIGLU: return dispatch_fp8<OUT_SWIGLU>(tile, A, As, Bt, Bs, C, Cs, M, N, K, S, planes, bpre, Fp8HeadOp{}, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+hipError_t fp8_gemm_phases_launch(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K,
+                                  unsigned long long* stamps, hipStream_t stream)
+{
+  if (M % 256 || N % 256 || K % 128 || !stamps) return hipErrorInvalidValue;
+  Fp8HeadOp op;
+  op.stamps = stamps;
+  const int tiles_m = M / 256, tiles_n = N / 256;
+  hipLaunchKernelGGL((fp8_gemm_kernel<256, 256, 64, OUT_FP8Q, 16>), dim3(tiles_m * tiles_n), dim3(512), 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C,
+                     Cs, M, N, K, tiles_m, tiles_n, op);
+  return hipGetLastError();
 }
 
 hipError_t fp8_gemm_qk_rope_launch(int out_kind, int tile, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C,

@@ -35,6 +35,7 @@ struct Fp8HeadOp {
   int          n_q        = 0;
   int          n_kv       = 0;
   const void*  residual   = nullptr;  // fp8_gemm_add_residual_launch only: [M, N] of the hidden dtype
+  unsigned long long* stamps = nullptr;  // fp8_gemm_phases_launch only: PHASE_STAMPS clock readings per wave (see there)
 };
 // A tile kernel (no split) with the head op in its epilogue; out_kind LLMMM_OUT_BF16 or LLMMM_OUT_FP8Q.
 hipError_t fp8_gemm_qk_rope_launch(int out_kind, int tile, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C,
@@ -49,6 +50,18 @@ hipError_t fp8_gemm_add_residual_launch(int hidden_dtype, int tile, int b_layout
 hipError_t fp8_planes_qk_norm_rope_launch(int out_kind, const float* planes, int S, void* C, float* Cs, const float* qw, const float* kw, float eps,
                                           const float* cos_t, const float* sin_t, int table_rows, const int* pos, int n_q, int n_kv, int M,
                                           hipStream_t stream);
+// Where a launch of the 256 x 256 tile kernels spends its time: the kernel of fp8_gemm_launch(LLMMM_OUT_FP8Q, LLMMM_TILE_256x256,
+// row-major weights) / fp16_gemm_launch(256 x 256 tile, row-major B) built with clock readings at five points of every
+// wave -- entry, first operands in LDS (end of the prologue), end of the K loop, last store issued, stores acknowledged.
+// stamps[(workgroup * 8 + wave) * PHASE_RECORD + 2 * p] = s_memrealtime (a constant 100 MHz clock) at point p and
+// [.. + 2 * p + 1] = s_memtime (shader clock cycles); [.. + PHASE_STAMPS] = the shader cycles the wave spent in the K loop's
+// waits for its loads and for the other waves (the barrier of every stage); [.. + PHASE_STAMPS + 1] unused.  M and N
+// multiples of 256.  The results are the product kernels'.
+constexpr int PHASE_POINTS = 5, PHASE_STAMPS = 2 * PHASE_POINTS, PHASE_RECORD = PHASE_STAMPS + 2;
+hipError_t fp8_gemm_phases_launch(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K,
+                                  unsigned long long* stamps, hipStream_t stream);
+hipError_t fp16_gemm_phases_launch(int dtype, const void* A, const void* B, void* C, int M, int N, int K, unsigned long long* stamps, hipStream_t stream);
+
 hipError_t fp8_splitk_reduce_launch(int out_kind, const float* planes, int S, void* C, float* Cs, int M, int N, hipStream_t stream);
 
 // M <= 128 (row groups of 64); S splits of K.  partial == nullptr (S must be 1): complete result in C / Cs.
