@@ -31,8 +31,8 @@ PREHEAT_S = 0.25  # seconds of untimed launches before the warm-up steps of ever
 # these same workloads, each scaled by the counter's reading for a 1 GiB device copy (FETCH_SIZE x 2.0 KiB,
 # WRITE_SIZE x 1.0 KiB per count).  Counters cannot be read from inside this process, so the figures are
 # carried here; the summaries they come from are kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"fp16_gemm_4096": 235.0e6, "fp8_gemm_fused_4096": 119.2e6, "decode_gate_up_m1": 50.0e6,
-                          "decode_gate_up_m1_pre": 50.0e6}
+MEASURED_TRAFFIC_BYTES = {"fp16_gemm_4096": 235.1e6, "fp8_gemm_fused_4096": 119.2e6, "decode_gate_up_m1": 50.0e6,
+                          "decode_gate_up_m1_pre": 50.0e6, "decode_o_m1_bf16_pre": 10.6e6}
 
 QWEN3_4B = {"qkv": (6144, 2560), "o": (2560, 4096), "gate_up": (19456, 2560), "down": (2560, 9728)}
 
@@ -572,7 +572,7 @@ def phase_accounting(kind, M=4096, N=4096, K=4096, launches=40):
     rec = stamps.cpu().numpy().reshape(-1, 12).astype(np.float64)
     t = rec[:, :10].reshape(-1, 5, 2)  # [wave, point, (100 MHz ticks, shader cycles)]
     real, cyc = t[:, :, 0], t[:, :, 1]
-    wait_cy = rec[:, 10]
+    wait_cy, load_wait_cy = rec[:, 10], rec[:, 11]
     t0 = real[:, 0].min()
     names = ["prologue (entry -> first operands in LDS)", "K loop", "epilogue (amax / convert / staging / stores issued)", "store drain (stores acknowledged)"]
     out = {"kernel_us_uninstrumented": ms_plain * 1e3, "kernel_us_instrumented": ms_probe * 1e3, "waves": int(t.shape[0]),
@@ -591,6 +591,11 @@ def phase_accounting(kind, M=4096, N=4096, K=4096, launches=40):
     out["k_loop_cycles_per_stage"] = loop_cy / slices
     # a SIMD holds two waves; per stage each issues 32 MFMAs of 32 cycles (fp8 16x16x128, a 128-K slice) or of 16 cycles (f16 16x16x32, K = 32)
     out["k_loop_wait_cycles_per_stage"] = float(np.median(wait_cy)) / slices
+    out["k_loop_load_wait_cycles_per_stage"] = float(np.median(load_wait_cy)) / slices
+    # per SIMD (its two waves are records w and w + 4 of a workgroup: waves are dealt to the four SIMDs in turn): the cycles
+    # per stage in which BOTH of its waves sit in a wait cannot be read off the sums, but their minimum bounds it from above
+    w8 = wait_cy.reshape(-1, 8)
+    out["k_loop_wait_cycles_per_stage_less_waiting_wave_of_a_simd"] = float(np.median(np.minimum(w8[:, :4], w8[:, 4:]))) / slices
     ideal = 2048.0 if kind == "fp8" else 1024.0
     out["k_loop_ideal_cycles_per_stage"] = ideal
     out["k_loop_matrix_pipe_share"] = ideal / out["k_loop_cycles_per_stage"]
@@ -643,7 +648,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="fp16_gemm_4096",
                     help="fp16_gemm_4096 (headline) | fp16_gemm_2048x19456x2560 | fp8_gemm_fused_4096 | fp8_gemm_bf16_4096 | bf16_gemm_4096 | "
-                         "decode_<qkv|o|gate_up|down>_m<M>[_pre] (_pre: weights pre-shuffled offline) | prefill_<qkv|o|gate_up|down>_m<M> | "
+                         "decode_<qkv|o|gate_up|down>_m<M>[_bf16][_pre] (_bf16: bf16 output instead of fused C quant; _pre: weights pre-shuffled offline) | "
+                         "fp16_gemm_4096_k<K> | fp8_gemm_fused_4096_k<K> (M = N = 4096 on another K) | prefill_<qkv|o|gate_up|down>_m<M> | "
                          "prefill_gate_up_swiglu_m<M> | fused_<o|down>_add_norm_m<M> | fused_qkv_rope_m<M> | layer_[consumer_]m<M> | copy_1g (counter calibration only) | "
                          "phases_fp8_4096 | phases_fp16_4096 (where a launch of the tile kernel spends its time; prints a table)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
@@ -686,9 +692,16 @@ def main():
             print("%-62s %9.2f %9.2f %9.2f %9.2f %12.0f" % (p["phase"], p["us_median"], p["us_mean"], p["us_min"], p["us_max"], p["cycles_median"]))
         print("K loop: %.0f cycles per stage against %.0f with the matrix pipe always busy (two waves per SIMD, 32 MFMAs each per stage): %.1f %%" %
               (r["k_loop_cycles_per_stage"], r["k_loop_ideal_cycles_per_stage"], 100 * r["k_loop_matrix_pipe_share"]))
-        print("of which a wave waits %.0f cycles per stage for its loads to land and for the other waves (vmcnt + barrier)" % r["k_loop_wait_cycles_per_stage"])
+        print("of which a wave waits %.0f cycles per stage (%.0f for its own loads to land, the rest for the other waves at the barrier);"
+              % (r["k_loop_wait_cycles_per_stage"], r["k_loop_load_wait_cycles_per_stage"]))
+        print("the less-waiting wave of each SIMD's pair: %.0f cycles per stage (an upper bound on the time a SIMD has no wave to issue from)"
+              % r["k_loop_wait_cycles_per_stage_less_waiting_wave_of_a_simd"])
         print(json.dumps({"workload": w, **r}))
         return
+    import re as _re
+    mk = _re.fullmatch(r"(fp16_gemm_4096|fp8_gemm_fused_4096)_k(\d+)", w)
+    if mk:  # the headline kernels on a shorter or longer K (counter runs: what scales with K and what does not)
+        w, K = mk.group(1), int(mk.group(2))
     if w in ("fp16_gemm_4096", "bf16_gemm_4096"):
         dt = torch.float16 if w.startswith("fp16") else torch.bfloat16
         r, _ = bench_fp16(M, N, K, args.steps, args.warmup, dt, clock=True)
@@ -696,8 +709,8 @@ def main():
         roof = {"bound": "mfma", "achieved": r["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": r["tflops"] / peak, "traffic": None,
                 "kernel": "fp16_gemm_kernel<%s,256,256,row-major B>" % dtype}
         value, unit = r["tflops"], "TFLOP/s"
-        cfg = {"workload": "FP16 GEMM M=N=K=4096 A~N(0,1) B~N(0,0.02) seed 2, fp32 accumulate, %s out, "
-                           "single kernel, no split-K" % dtype, "M": M, "N": N, "K": K}
+        cfg = {"workload": "FP16 GEMM %s A~N(0,1) B~N(0,0.02) seed 2, fp32 accumulate, %s out, "
+                           "single kernel, no split-K" % ("M=N=K=4096" if K == 4096 else "M=N=4096 K=%d" % K, dtype), "M": M, "N": N, "K": K}
     elif w == "fp16_gemm_2048x19456x2560":
         # 608 tiles of 256 x 256: two whole rounds of the chip and 96 tiles -- the launch of two tile shapes
         M, N, K = 2048, 19456, 2560
@@ -714,7 +727,8 @@ def main():
         roof = {"bound": "mfma", "achieved": r["tflops"], "peak": peak, "unit": "TFLOP/s", "frac": r["tflops"] / peak, "traffic": None,
                 "kernel": "fp8_gemm_kernel<256,256,%s>" % out}
         value, unit = r["tflops"], "TFLOP/s"
-        cfg = {"workload": "FP8 e4m3 blockwise GEMM M=N=K=4096 (A 1x128, B 128x128 scales), output %s" % out, "M": M, "N": N, "K": K}
+        cfg = {"workload": "FP8 e4m3 blockwise GEMM %s (A 1x128, B 128x128 scales), output %s" % ("M=N=K=4096" if K == 4096 else "M=N=4096 K=%d" % K, out),
+               "M": M, "N": N, "K": K}
     elif w.startswith("layer_"):
         import re
         mo = re.fullmatch(r"layer_(consumer_)?m(\d+)", w)
@@ -762,20 +776,22 @@ def main():
                            % (what, M, N, K, x["weight_copies"], x.get("us_separate_launches", x.get("us_plain_bf16_gemm", 0.0))), "M": M, "N": N, "K": K}
     elif w.startswith("decode_"):
         import re
-        mo = re.fullmatch(r"decode_(qkv|o|gate_up|down)_m(\d+)(_pre)?", w)
+        mo = re.fullmatch(r"decode_(qkv|o|gate_up|down)_m(\d+)(_bf16)?(_pre)?", w)
         if not mo:
             print("unknown workload", w, file=sys.stderr)
             sys.exit(2)
         name, M = mo.group(1), int(mo.group(2))
         N, K = QWEN3_4B[name]
-        pre = mo.group(3) is not None
-        r = bench_fp8(M, N, K, "fp8q", args.steps, args.warmup, rotate_bytes=768 << 20, preshuffled=pre)
+        out = "bf16" if mo.group(3) else "fp8q"
+        pre = mo.group(4) is not None
+        r = bench_fp8(M, N, K, out, args.steps, args.warmup, rotate_bytes=768 << 20, preshuffled=pre)
         dtype = "fp8"
         roof = {"bound": "hbm", "achieved": r["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": r["gbs"] / PEAK_HBM_GBS, "traffic": None,
-                "kernel": "fp8_skinny_kernel split_k=%d" % r["split_k"]}
+                "kernel": r["kernel"]}
         value, unit = r["gbs"], "GB/s"
-        cfg = {"workload": "Qwen3-4B %s projection, FP8 blockwise GEMM + fused C quant, M=%d N=%d K=%d, %s weights rotated over %d "
-                           "copies" % (name, M, N, K, "pre-shuffled" if pre else "row-major", r["weight_copies"]), "M": M, "N": N, "K": K}
+        cfg = {"workload": "Qwen3-4B %s projection, FP8 blockwise GEMM, %s, M=%d N=%d K=%d, %s weights rotated over %d "
+                           "copies" % (name, "bf16 output" if out == "bf16" else "fused C quant", M, N, K, "pre-shuffled" if pre else "row-major", r["weight_copies"]),
+               "M": M, "N": N, "K": K}
     elif w.startswith("prefill_"):
         import re
         mo = re.fullmatch(r"prefill_(qkv|o|gate_up|down)(_swiglu)?_m(\d+)", w)
@@ -795,7 +811,7 @@ def main():
         print("unknown workload", w, file=sys.stderr)
         sys.exit(2)
 
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(w)
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(w) if not mk else None
     roof["algorithmic_bytes"] = r["bytes"]
     clk = r.get("clock") if isinstance(r, dict) else None
     if clk and clk.get("sclk_mhz") and roof["bound"] == "mfma":

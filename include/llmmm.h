@@ -283,7 +283,8 @@ LLMMM_API int    llmmm_probe_hbm_read(const void* src, size_t bytes, float* sink
  * 0 kernel entry, 1 first operands in LDS (end of the prologue), 2 end of the K loop, 3 last store issued, 4 stores acknowledged.
  * stamps: device memory of llmmm_probe_phases_bytes(M, N) bytes; afterwards, as 64-bit words, record (t * 8 + w) * 12 of
  * workgroup t and wave w (8 per workgroup) holds at [2 p] the constant 100 MHz clock at point p, at [2 p + 1] the shader's
- * cycle counter, and at [10] the shader cycles the wave spent waiting in the K loop (loads landed + barrier of every stage).
+ * cycle counter, at [10] the shader cycles the wave spent waiting in the K loop (loads landed + barrier of every stage) and at [11] the part
+ * of those spent waiting for its own loads.
  * The reference measures its kernels from outside only (ncu.sh); no counterpart. */
 LLMMM_API size_t llmmm_probe_phases_bytes(int M, int N);
 LLMMM_API int    llmmm_probe_fp8_gemm_phases(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K,

@@ -179,7 +179,7 @@ __device__ __forceinline__ void fp16_gemm_body(const T* __restrict__ A, const T*
   typedef typename Mfma32<T>::vec   vec;
   constexpr int                     MF = TC::MF;
   PhaseClock                        ph[STAMP ? PHASE_POINTS : 1];
-  unsigned long long                wait_cycles = 0;  // STAMP: shader cycles in the K loop's "loads landed + barrier" waits
+  unsigned long long                wait_cycles = 0, load_wait_cycles = 0;  // STAMP: shader cycles in the K loop's "loads landed + barrier" waits; of which for the loads
   if constexpr (STAMP) ph[0] = phase_clock();
 
   const int tid  = threadIdx.x;
@@ -291,6 +291,7 @@ __device__ __forceinline__ void fp16_gemm_body(const T* __restrict__ A, const T*
       wait_vmcnt<TC::LOADS>();                                                                                     \
     else                                                                                                           \
       wait_vmcnt<0>();                                                                                             \
+    if constexpr (STAMP) load_wait_cycles += __builtin_amdgcn_s_memtime() - tw_;                                   \
     __builtin_amdgcn_s_barrier();                                                                                  \
     if constexpr (STAMP) wait_cycles += __builtin_amdgcn_s_memtime() - tw_;                                        \
     if (STEADY || (s) + 4 < KT) LLMMM_ISSUE((s) + 4, u);                                                           \
@@ -361,7 +362,7 @@ __device__ __forceinline__ void fp16_gemm_body(const T* __restrict__ A, const T*
       unsigned long long* o = stamps + ((size_t)tile_index * TC::NW + wave) * PHASE_RECORD;
 #pragma unroll
       for (int p = 0; p < PHASE_POINTS; ++p) o[2 * p] = ph[p].real, o[2 * p + 1] = ph[p].cycles;
-      o[PHASE_STAMPS] = wait_cycles;
+      o[PHASE_STAMPS] = wait_cycles, o[PHASE_STAMPS + 1] = load_wait_cycles;
     }
   }
 }

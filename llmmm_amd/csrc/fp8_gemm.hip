@@ -419,6 +419,7 @@ __device__ __forceinline__ void fp8_gemm_body(const uint8_t* __restrict__ A, con
   constexpr bool STAMP   = (BMODE & 16) != 0;
   PhaseClock     ph[STAMP ? PHASE_POINTS : 1];
   unsigned long long wait_cycles = 0;  // STAMP: shader cycles this wave spent in the K loop's "loads landed + barrier" waits (slices 1 ..)
+  unsigned long long load_wait_cycles = 0;  // ... of which for its own loads (the rest: for the other waves at the barrier)
   if constexpr (STAMP) ph[0] = phase_clock();
   static_assert(!MT || (DEEP && BM == 128 && BN == 128 && (OUT == OUT_F32 || OUT == OUT_BF16 || OUT == OUT_FP8Q)), "row tails: deep 128 x 128 tiles only");
   constexpr int  STAGE_D = TC::STAGE + TC::NW * 256;                 // operands + 256 bytes of scales per wave
@@ -552,6 +553,8 @@ __device__ __forceinline__ void fp8_gemm_body(const uint8_t* __restrict__ A, con
     unsigned long long tw_ = 0;                                                                                                   \
     if constexpr (STAMP) tw_ = __builtin_amdgcn_s_memtime();                                                                      \
     wait_vmcnt<0>();                                                                                                              \
+    if constexpr (STAMP)                                                                                                          \
+      if ((KC) != 0) load_wait_cycles += __builtin_amdgcn_s_memtime() - tw_;                                                      \
     if constexpr (MF == 4)                                                                                                        \
       asm volatile("" : "+v"(sa_next[0]), "+v"(sa_next[1]), "+v"(sa_next[2]), "+v"(sa_next[MF - 1]), "+v"(sb_next));              \
     else                                                                                                                          \
@@ -762,7 +765,7 @@ __device__ __forceinline__ void fp8_gemm_body(const uint8_t* __restrict__ A, con
       unsigned long long* o = op.stamps + ((size_t)tile_index * TC::NW + wave) * PHASE_RECORD;
 #pragma unroll
       for (int p = 0; p < PHASE_POINTS; ++p) o[2 * p] = ph[p].real, o[2 * p + 1] = ph[p].cycles;
-      o[PHASE_STAMPS] = wait_cycles;
+      o[PHASE_STAMPS] = wait_cycles, o[PHASE_STAMPS + 1] = load_wait_cycles;
     }
   }
 }

@@ -55,7 +55,8 @@ hipError_t fp8_planes_qk_norm_rope_launch(int out_kind, const float* planes, int
 // wave -- entry, first operands in LDS (end of the prologue), end of the K loop, last store issued, stores acknowledged.
 // stamps[(workgroup * 8 + wave) * PHASE_RECORD + 2 * p] = s_memrealtime (a constant 100 MHz clock) at point p and
 // [.. + 2 * p + 1] = s_memtime (shader clock cycles); [.. + PHASE_STAMPS] = the shader cycles the wave spent in the K loop's
-// waits for its loads and for the other waves (the barrier of every stage); [.. + PHASE_STAMPS + 1] unused.  M and N
+// waits for its loads and for the other waves (the barrier of every stage); [.. + PHASE_STAMPS + 1] = the part of that spent
+// waiting for its own loads (and LDS reads).  M and N
 // multiples of 256.  The results are the product kernels'.
 constexpr int PHASE_POINTS = 5, PHASE_STAMPS = 2 * PHASE_POINTS, PHASE_RECORD = PHASE_STAMPS + 2;
 hipError_t fp8_gemm_phases_launch(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K,
