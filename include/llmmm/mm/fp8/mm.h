@@ -103,7 +103,8 @@ inline void gemm(int out_kind, const void* A, const float* As, const void* Bt, c
 
 // Hands the launchers of this header a split-K workspace for calls of the calling thread on `stream`: device memory of
 // `bytes` bytes, 16-byte aligned, plain scratch, which must stay valid until it is replaced or withdrawn
-// (set_fp8_workspace(stream, nullptr, 0): back to the shim's own buffer; one it had allocated before is kept and reused).
+// (set_fp8_workspace(stream, nullptr, 0): back to a buffer of the shim's own, allocated on the next need; one it held
+// before the caller's came was freed when the caller's arrived -- hipFree synchronises, so set the workspace before any capture).
 // With a workspace set, the reference-signature launchers honour the reference's contract to the letter -- no
 // allocation, no free, no synchronisation (src/mm/fp16/mm.cu:6-42) -- and can be captured into a HIP graph on first use.
 // llmmm_fp8_gemm_workspace(out_kind, M, N, K) gives the size a shape wants; with less, K is split less or not at all.

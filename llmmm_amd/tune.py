@@ -23,28 +23,31 @@ QWEN3_4B = {"qkv": (6144, 2560), "o": (2560, 4096), "gate_up": (19456, 2560), "d
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
-def _time_ms(fn, iters, graph):
+def _time_ms(fn, iters, graph, batches=5):
+    """ms per call: the median over `batches` event-bracketed batches of `iters` calls (one graph replay each when graph)."""
     for _ in range(3):
         fn()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     if graph:
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             for _ in range(iters):
                 fn()
-        g.replay()
-        torch.cuda.synchronize()
-        e0.record()
-        g.replay()
-        e1.record()
+        for _ in range(3):
+            g.replay()
+        batch = g.replay
     else:
+        def batch():
+            for _ in range(iters):
+                fn()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(batches)]
+    for e0, e1 in ev:
         e0.record()
-        for _ in range(iters):
-            fn()
+        batch()
         e1.record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / iters
+    return sorted(e0.elapsed_time(e1) for e0, e1 in ev)[batches // 2] / iters
 
 
 def _inputs(M, N, K, copies):
