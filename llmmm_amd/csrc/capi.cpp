@@ -267,9 +267,11 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
   // 64 < M < 128: where the table gives M = 128 to 128 x 128 tiles, the same tiles take the shorter matrix too (the
   // rows of the tile beyond M are computed and not stored) -- 96 x 19456 x 2560: 20 us instead of 33 us in the
   // weight-streaming kernel, whose eight 16-row blocks per wave are bound by their LDS reads and fp32 planes
-  if (cfg->tile < 0 && M > 64 && M < 128) {
+  // (where that entry is unsplit -- enough column groups to fill the chip, i.e. a large weight matrix -- already from 33
+  // rows on: 19456 x 2560 at M = 48 / 64: 15.9 / 16.7 us in tiles, 18.0 / 19.5 us streaming in three splits; at 32: 15.3 / 15.5)
+  if (cfg->tile < 0 && M > 32 && M < 128) {
     int t, sp;
-    if (lookup_tile(128, N, K, &t, &sp, true) && t == LLMMM_TILE_128x128) cfg->tile = t, cfg->split_k = sp;
+    if (lookup_tile(128, N, K, &t, &sp, true) && t == LLMMM_TILE_128x128 && (M > 64 || sp <= 1)) cfg->tile = t, cfg->split_k = sp;
   }
   if (cfg->tile < 0 && M <= SKINNY_MAX_M) {
     int sp;
@@ -278,7 +280,8 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
     // eight 16-row blocks per wave and its fp32 planes grow with M, and from about 20 MB of weights on, one row of 128 x 128
     // tiles (a row tail for M < 128) is faster (measured at M = 96, us, streaming / tiles: N x K = 4096 x 4096 12.4 / 14.2,
     // 6144 x 4096 19.9 / 16.0, 4096 x 14336 39.4 / 22.1, 28672 x 4096 66.7 / 27.1)
-    if (cfg->tile < 0) cfg->tile = (M <= 64 || (long)N * K < 20000000L) ? LLMMM_TILE_SKINNY : LLMMM_TILE_128x128;
+    // (from 40 MB on the tiles win from 33 rows on, as on the tuned 19456 x 2560)
+    if (cfg->tile < 0) cfg->tile = (M <= 32 || (long)N * K < 20000000L || (M <= 64 && (long)N * K < 40000000L)) ? LLMMM_TILE_SKINNY : LLMMM_TILE_128x128;
   }
   if (cfg->tile < 0) {
     if (M % 128) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");

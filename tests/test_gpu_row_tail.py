@@ -66,7 +66,11 @@ def test_table_routes_64_to_127_rows_like_128(lib):
         assert want[0] == T128
         for m in (65, 96, 127):
             assert lib.query_config(_lib.OUT_FP8Q, m, n, k) == want
-        assert lib.query_config(_lib.OUT_FP8Q, 64, n, k)[0] == SKINNY
+    # an unsplit entry (gate_up: enough column groups to fill the chip) already takes 33 .. 64 rows; a split one (down) does not
+    for m in (33, 48, 64):
+        assert lib.query_config(_lib.OUT_FP8Q, m, 19456, 2560) == lib.query_config(_lib.OUT_FP8Q, 128, 19456, 2560)
+    assert lib.query_config(_lib.OUT_FP8Q, 32, 19456, 2560)[0] == SKINNY
+    assert lib.query_config(_lib.OUT_FP8Q, 64, 2560, 9728)[0] == SKINNY
 
 
 def test_swiglu_and_planes_entry_points_on_tail_rows(lib, oracle):
