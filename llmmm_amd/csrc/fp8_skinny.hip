@@ -189,7 +189,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
   const int i    = lane & 15;
   const int ng   = blockIdx.x;
   const int sp   = blockIdx.y;
-  const int m0   = blockIdx.z * (MBLK == 8 ? 128 : 64);  // row groups of 64 (of 128 with MBLK = 8): gridDim.z = number of groups
+  const int m0   = blockIdx.z * (16 * MBLK);  // row groups of 16 * MBLK rows: gridDim.z = number of groups
   const int KB   = K >> 7;
   const int kb0  = sp * KB / S;  // KB * S is small: 32-bit arithmetic (a 64-bit divide costs hundreds of scalar ops)
   const int kb1  = (sp + 1) * KB / S;
@@ -732,7 +732,7 @@ template <int MBLK, int OUT, int D, int ASTG>
 static hipError_t launch_skinny(const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M,
                                 int N, int K, int S, float* partial, int bpre, hipStream_t stream)
 {
-  hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D, ASTG>), dim3(N / 128, S, MBLK == 8 ? (M + 127) / 128 : (M + 63) / 64), dim3(512), 0, stream,
+  hipLaunchKernelGGL((fp8_skinny_kernel<MBLK, OUT, D, ASTG>), dim3(N / 128, S, (M + 16 * MBLK - 1) / (16 * MBLK)), dim3(512), 0, stream,
                      (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, Cs, M, N, K, S, partial, bpre, SkinnyGenA{});
   return hipGetLastError();
 }
@@ -822,6 +822,7 @@ static hipError_t dispatch_skinny(const void* A, const float* As, const void* Bt
     const int need = 2 * 2048 * longest;
     if (slices >= 4 && need <= 65536) LLMMM_GO(2, 4, 65536);
     if (need <= 65536) LLMMM_GO(2, 2, 65536);
+    if (slices >= 4 && need <= 81920) LLMMM_GO(2, 4, 81920);  // 20 slices (K = 2560 unsplit): 80 KB beside a 4-deep ring
     if (slices >= 4) LLMMM_GO(2, 4, 0);
     LLMMM_GO(2, 2, 0);
   }
@@ -833,6 +834,10 @@ static hipError_t dispatch_skinny(const void* A, const float* As, const void* Bt
     const int need = 4 * 2048 * longest;
     if (slices >= 4 && need <= 65536) LLMMM_GO(4, 4, 65536);
     if (need <= 65536) LLMMM_GO(4, 2, 65536);
+    // K ranges too long to stage 64 rows of: row groups of 32 whose rows still fit (every group streams the weights of
+    // its columns again, from L2) -- 128 x 6144 x 2560 unsplit: 10.6 us in four groups, one launch, against 13.3 us in
+    // five splits + reduce and 42 us with the activations fetched per wave and slice
+    if (slices >= 4 && 2 * 2048 * longest <= 81920) LLMMM_GO(2, 4, 81920);
     if (slices >= 4) LLMMM_GO(4, 4, 0);
     LLMMM_GO(4, 2, 0);
   }

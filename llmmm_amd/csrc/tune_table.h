@@ -29,9 +29,10 @@ static const SkinnyTune kSkinnyTune[] = {
   {1, 6144, 2560, 5},
   {16, 6144, 2560, 5},
   {64, 6144, 2560, 5},
-  {128, 6144, 2560, 5},
+  {128, 6144, 2560, 1},
   {1, 19456, 2560, 1},
   {16, 19456, 2560, 1},
+  {32, 19456, 2560, 1},
   {64, 19456, 2560, 3},
 };
 
