@@ -169,6 +169,21 @@ def test_skinny_kernel_against_oracle(lib, oracle, M, split):
     _check_all(oracle, _run_all(lib, Aq, As, Bq, Bs, tile=8, split_k=split), ref, "skinny M=%d S=%d" % (M, split))
 
 
+@pytest.mark.parametrize("M", [17, 32, 33, 64, 65, 100, 128])
+def test_skinny_row_groups_over_an_unsplit_long_k(lib, oracle, M):
+    """K = 2560 unsplit: 20 slices of 32 rows are 80 KB of staged activations, so the rows go in groups of 32 (gridDim.z up to 4),
+    each with its own fused epilogue.  Against the oracle, and bit for bit against one row of 128 x 128 tiles (no split on
+    either side: the same additions in the same order)."""
+    N, K = 512, 2560
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=100 + M)
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    got = _run_all(lib, Aq, As, Bq, Bs, tile=8, split_k=1)
+    _check_all(oracle, got, ref, "skinny row groups M=%d" % M)
+    tiles = _run_all(lib, Aq, As, Bq, Bs, tile=3, split_k=1)  # LLMMM_TILE_128x128
+    for a, b in zip(got[:4], tiles[:4]):
+        assert np.array_equal(np.asarray(a).view(np.uint8), np.asarray(b).view(np.uint8)), "differs from the 128 x 128 tiles"
+
+
 def test_skinny_without_workspace_does_not_split(lib, oracle):
     Aq, As, Bq, Bs = fp8_inputs(oracle, 4, 256, 2560, seed=8)
     ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
