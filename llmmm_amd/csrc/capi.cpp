@@ -115,6 +115,33 @@ int heuristic_tile(int M, int N)
   return best;
 }
 
+// The FP16 / BF16 kernels' tile for shapes the table does not list: the most tiles any CU gets (two 128 x 128 tiles share
+// a CU side by side, but it then takes as long as for both) times the tile's area, over a measured efficiency relative
+// to the 256 x 256 tile (4096^3: 111.6 us in 256 x 256, 127.6 in 128 x 256, 131.9 in 256 x 128, 146.8 in 128 x 128).  Picks
+// the measured best on every shape of the tune driver's list, e.g. 128 x 256 for 2048 x 2560 x 9728 (115 us; 144 in
+// 128 x 128, 182 in 256 x 256) and for 4096 x 2048 x 12288 (184 us; 229 in 256 x 256).
+int heuristic_tile_fp16(int M, int N)
+{
+  static const struct {
+    int   id, bm, bn;
+    float eff;
+  } cand[] = {{LLMMM_TILE_256x256, 256, 256, 1.00f}, {LLMMM_TILE_128x256, 128, 256, 0.875f}, {LLMMM_TILE_256x128, 256, 128, 0.85f}, {LLMMM_TILE_128x128, 128, 128, 0.74f}};
+  int   best      = -1;
+  float best_cost = 0.f;
+  for (const auto& c : cand) {
+    if (M % c.bm || N % c.bn) continue;
+    const long tiles  = (long)(M / c.bm) * (N / c.bn);
+    float      rounds = (float)((tiles + NUM_CUS - 1) / NUM_CUS);
+    if (c.id == LLMMM_TILE_256x256) {  // a partly filled last round runs in half-size tiles where launch_fp16 can arrange it
+      const long tm = M / 256, tn = N / 256, full = tiles / NUM_CUS * NUM_CUS;
+      if (tiles > NUM_CUS && tm > 1 && full % tm == 0 && tn - full / tm > 0 && (tn - full / tm) * tm * 2 <= NUM_CUS) rounds -= 0.5f;
+    }
+    const float cost = rounds * c.bm * c.bn / c.eff;
+    if (best < 0 || cost < best_cost) best = c.id, best_cost = cost;
+  }
+  return best;
+}
+
 constexpr int MAX_TILE_SPLIT = 8;
 
 bool tile_dims(int tile, int& bm, int& bn);
@@ -395,7 +422,7 @@ int llmmm_fp16_gemm_ex(int dtype, const void* A, const void* B, void* C, int M, 
   if (tile == LLMMM_TILE_AUTO) {
     if (!lookup_fp16_tile(M, N, K, &tile)) tile = LLMMM_TILE_AUTO;
     if (tile == LLMMM_TILE_AUTO) {
-      tile = heuristic_tile(M, N);
+      tile = heuristic_tile_fp16(M, N);
       // small problems: 128 x 128 tiles on at most half of the CUs -> twice as many 64 x 128 tiles of four 16-row
       // waves (1024^3: 8.0 instead of 11.3 us; from 160 tiles of 128 x 128 on, the larger tile wins again)
       if (tile == LLMMM_TILE_128x128 && (long)(M / 128) * (N / 128) <= NUM_CUS / 2) tile = LLMMM_TILE_64x128;

@@ -61,8 +61,13 @@ static const TileTune kTileTune[] = {
 
 // FP16/BF16 MFMA tile kernels.
 static const TileTune kFp16TileTune[] = {
-  {4096, 4096, 4096, 0, 1},
   {1024, 1024, 1024, 4, 1},
+  {2048, 2048, 2048, 3, 1},
+  {4096, 4096, 4096, 0, 1},
+  {4096, 6144, 2048, 0, 1},
+  {4096, 2048, 12288, 1, 1},
+  {2048, 19456, 2560, 0, 1},
+  {2048, 2560, 9728, 1, 1},
 };
 
 }  // namespace llmmm

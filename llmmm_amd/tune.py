@@ -98,6 +98,29 @@ def tune_shape(M, N, K, iters=40, rotate_bytes=768 << 20, verbose=True):
     return best[0], best[1], results
 
 
+FP16_SHAPES = [(1024, 1024, 1024), (2048, 2048, 2048), (4096, 4096, 4096), (4096, 6144, 2048), (4096, 2048, 12288), (2048, 19456, 2560),
+               (2048, 2560, 9728)]  # the benchmark shapes, those of test/fp16_mm_test.cc:96-103 and two Qwen3-4B prefill projections
+FP16_TILES = {_lib.TILE_256x256: (256, 256), _lib.TILE_128x256: (128, 256), _lib.TILE_256x128: (256, 128), _lib.TILE_128x128: (128, 128),
+              _lib.TILE_64x128: (64, 128)}
+
+
+def tune_fp16_shape(M, N, K, iters=40, dtype=torch.float16, verbose=True):
+    """The FP16 / BF16 GEMM's tile for one shape: (best_tile, {tile: ms}) over the tiles that divide it."""
+    g = torch.Generator(device="cuda").manual_seed(2)
+    A = torch.randn((M, K), generator=g, device="cuda").to(dtype)
+    B = (torch.randn((K, N), generator=g, device="cuda") * 0.02).to(dtype)
+    C = torch.empty((M, N), dtype=dtype, device="cuda")
+    results = {}
+    for tile, (bm, bn) in FP16_TILES.items():
+        if M % bm or N % bn:
+            continue
+        results[tile] = _time_ms(lambda: mm.fp16_gemm(A, B, C, tile=tile), iters, graph=True)
+    best = min(results, key=results.get)
+    if verbose:
+        print("fp16 M=%d N=%d K=%d:" % (M, N, K), " ".join("%d:%.1fus" % (t, v * 1e3) for t, v in sorted(results.items())), "-> best", best, flush=True)
+    return best, results
+
+
 def render_table(skinny_rows, tile_rows, fp16_rows):
     out = ["// Offline auto-tune results, compiled in.  Regenerate with `python -m llmmm_amd.tune --write` on an",
            "// MI355X; shapes that are not listed fall back to the heuristics in capi.cpp.",
@@ -125,6 +148,17 @@ def render_file(skinny_rows, tile_rows, fp16_rows):
     return "\n".join(out) + "\n"
 
 
+def parse_header(text):
+    """The rows of a rendered tune_table.h: (skinny_rows, tile_rows, fp16_rows)."""
+    import re
+    out = {"kSkinnyTune": [], "kTileTune": [], "kFp16TileTune": []}
+    for name in out:
+        body = re.search(r"%s\[\] = \{(.*?)\};" % name, text, re.S)
+        if body:
+            out[name] = [tuple(int(v) for v in row.split(",")) for row in re.findall(r"\{([-\d, ]+)\}", body.group(1))]
+    return out["kSkinnyTune"], out["kTileTune"], out["kFp16TileTune"]
+
+
 def parse_file(text):
     """Inverse of render_file: (skinny_rows, tile_rows, fp16_rows); lines that are not entries are skipped, as the library does."""
     skinny, tile, fp16 = [], [], []
@@ -149,6 +183,8 @@ def main():
     ap.add_argument("--iters", type=int, default=40)
     ap.add_argument("--write-file", metavar="PATH", help="write the results as a run-time tune file (LLMMM_TUNE_FILE)")
     ap.add_argument("--shape", action="append", metavar="N,K", help="tune this weight shape instead of the Qwen3-4B projections (repeatable)")
+    ap.add_argument("--fp16-shape", action="append", metavar="M,N,K", help="tune the FP16 / BF16 GEMM's tile for this shape instead of the built-in list (repeatable)")
+    ap.add_argument("--fp16-only", action="store_true", help="tune only the FP16 / BF16 shapes (the FP8 rows keep the compiled-in values)")
     args = ap.parse_args()
     torch.cuda.set_device(0)
     ms = [int(x) for x in args.m.split(",")]
@@ -156,6 +192,9 @@ def main():
     if args.shape:
         shapes = {"%sx%s" % tuple(x.split(",")): tuple(int(v) for v in x.split(",")) for x in args.shape}
     skinny_rows, tile_rows = [], ([] if args.shape else [(4096, 4096, 4096, _lib.TILE_256x256, 1)])
+    if args.fp16_only:
+        skinny_rows, tile_rows, _ = parse_header(open(os.path.join(HERE, "csrc", "tune_table.h")).read())
+        shapes = {}
     for name, (N, K) in shapes.items():
         for M in ms:
             tile, split, _ = tune_shape(M, N, K, iters=args.iters)
@@ -167,7 +206,8 @@ def main():
                 tile_rows.append((M, N, K, tile, split))
             torch.cuda.empty_cache()
     skinny_rows.sort(key=lambda r: (r[1], r[2], r[0]))
-    fp16_rows = [] if args.shape else [(4096, 4096, 4096, _lib.TILE_256x256, 1), (1024, 1024, 1024, _lib.TILE_64x128, 1)]
+    fp16_shapes = [tuple(int(v) for v in x.split(",")) for x in args.fp16_shape] if args.fp16_shape else ([] if args.shape else FP16_SHAPES)
+    fp16_rows = [(M, N, K, tune_fp16_shape(M, N, K, iters=args.iters)[0], 1) for M, N, K in fp16_shapes]
     text = render_table(skinny_rows, tile_rows, fp16_rows)
     print(text)
     if args.write_file:

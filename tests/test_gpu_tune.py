@@ -28,3 +28,18 @@ def test_tune_shape_returns_a_runnable_candidate(lib, oracle, M, N, K):
     assert_fused_close(oracle, Cq.cpu().numpy(), Cs.cpu().numpy(), rq, rs, "tuned candidate")
     rows = ([(M, N, K, split)], []) if tile == _lib.TILE_SKINNY else ([], [(M, N, K, tile, split)])
     assert tune.parse_file(tune.render_file(rows[0], rows[1], []))[:2] == rows
+
+
+def test_tune_fp16_shape_returns_a_runnable_tile(lib, oracle):
+    """The FP16 side of the driver: every tile that divides the shape is timed, the winner runs and meets the Kahan oracle."""
+    import numpy as np
+    from helpers import assert_fp16_close, fp16_inputs_uniform
+    from llmmm_amd import tune
+    M, N, K = 256, 512, 544
+    best, results = tune.tune_fp16_shape(M, N, K, iters=5, verbose=False)
+    assert best in results and len(results) == 5 and results[best] == min(results.values())
+    A, B = fp16_inputs_uniform(M, N, K, seed=9)
+    C = lib.fp16_gemm(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), tile=best)
+    torch.cuda.synchronize()
+    assert_fp16_close(C.cpu().numpy(), oracle.kahan_gemm(A, B), "tuned fp16 tile")
+    assert tune.parse_file(tune.render_file([], [], [(M, N, K, best, 1)]))[2] == [(M, N, K, best, 1)]

@@ -68,3 +68,14 @@ def test_shapes_near_a_tuned_one_inherit_its_tile():
     assert q(1536, 2560, 9728)[0] == _lib.TILE_128x128       # between the entries at 1024 and 2048 (both 128 x 128)
     assert q(128, 6144, 2560)[0] == _lib.TILE_SKINNY         # M = 128 stays with its weight-streaming entry, not the tile tuned at 256
     assert q(96, 6144, 2560)[0] == _lib.TILE_SKINNY
+
+
+def test_the_compiled_in_header_parses_back_to_what_renders_it():
+    """--fp16-only keeps the FP8 rows of csrc/tune_table.h: parse_header must read exactly what render_table wrote."""
+    import os
+    from llmmm_amd import tune
+    path = os.path.join(os.path.dirname(tune.__file__), "csrc", "tune_table.h")
+    text = open(path).read()
+    skinny, tile, fp16 = tune.parse_header(text)
+    assert skinny and tile and fp16 and all(len(r) == 4 for r in skinny) and all(len(r) == 5 for r in tile + fp16)
+    assert tune.render_table(skinny, tile, fp16).rstrip() == text.rstrip()
