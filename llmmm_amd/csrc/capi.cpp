@@ -262,12 +262,12 @@ bool lookup_tile(int M, int N, int K, int* tile, int* split, bool exact_only = f
   if (lookup_tile_in(llmmm::kTileTune, M, N, K, &t2, &s2, &best2) && best2 < best) *tile = t2, *split = s2, best = best2;
   return best < limit;
 }
-bool lookup_skinny(int M, int N, int K, int* split)
+bool lookup_skinny(int M, int N, int K, int* split, int* m_max = nullptr)
 {
   for (const auto& e : tune_override().skinny)
-    if (e.N == N && e.K == K && M <= e.m_max) return *split = e.split_k, true;
+    if (e.N == N && e.K == K && M <= e.m_max) return *split = e.split_k, (m_max ? *m_max = e.m_max : 0), true;
   for (const auto& e : llmmm::kSkinnyTune)
-    if (e.N == N && e.K == K && M <= e.m_max) return *split = e.split_k, true;
+    if (e.N == N && e.K == K && M <= e.m_max) return *split = e.split_k, (m_max ? *m_max = e.m_max : 0), true;
   return false;
 }
 bool lookup_fp16_tile(int M, int N, int K, int* tile)
@@ -287,9 +287,15 @@ int choose_fp8(int M, int N, int K, llmmm_gemm_cfg* cfg)
   cfg->split_k  = 0;
   cfg->b_layout = LLMMM_FP8_B_ROWS;
   cfg->a_layout = LLMMM_FP8_A_QUANTISED;
-  if (M % 128 == 0) {
-    int t, sp;
-    if (lookup_tile(M, N, K, &t, &sp, true)) cfg->tile = t, cfg->split_k = sp;
+  {
+    int t, sp;  // an entry for exactly this shape (one for fewer than 128 rows can only name the 128 x 128 tile: a row tail)
+    if (lookup_tile(M, N, K, &t, &sp, true) && (M % 128 == 0 || (M < 128 && t == LLMMM_TILE_128x128))) cfg->tile = t, cfg->split_k = sp;
+  }
+  // 64 < M < 128 with a weight-streaming entry measured in that range (m_max < 128): it was timed against the row-tail
+  // tiles below and won (2560 x 9728 up to 96 rows: 13.0 us in four splits of 32-row groups, 14.5 us in tiles)
+  if (cfg->tile < 0 && M > 64 && M < 128) {
+    int sp, mm;
+    if (lookup_skinny(M, N, K, &sp, &mm) && mm < 128) cfg->tile = LLMMM_TILE_SKINNY, cfg->split_k = sp;
   }
   // 64 < M < 128: where the table gives M = 128 to 128 x 128 tiles, the same tiles take the shorter matrix too (the
   // rows of the tile beyond M are computed and not stored) -- 96 x 19456 x 2560: 20 us instead of 33 us in the

@@ -26,6 +26,7 @@ static const SkinnyTune kSkinnyTune[] = {
   {1, 2560, 9728, 10},
   {16, 2560, 9728, 10},
   {64, 2560, 9728, 10},
+  {96, 2560, 9728, 4},
   {1, 6144, 2560, 5},
   {16, 6144, 2560, 5},
   {64, 6144, 2560, 5},
@@ -33,7 +34,6 @@ static const SkinnyTune kSkinnyTune[] = {
   {1, 19456, 2560, 1},
   {16, 19456, 2560, 1},
   {32, 19456, 2560, 1},
-  {64, 19456, 2560, 3},
 };
 
 // FP8 MFMA tile kernels (M % 128 == 0).
@@ -41,6 +41,7 @@ static const TileTune kTileTune[] = {
   {4096, 4096, 4096, 0, 1},
   {2048, 6144, 2560, 0, 1},
   {2048, 2560, 4096, 3, 1},
+  {64, 19456, 2560, 3, 1},
   {128, 19456, 2560, 3, 1},
   {2048, 19456, 2560, 0, 1},
   {128, 2560, 9728, 3, 8},

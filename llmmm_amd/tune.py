@@ -4,8 +4,9 @@ of shapes on the GPU at hand and writes ``csrc/tune_table.h`` (compiled into ``l
     python -m llmmm_amd.tune [--write] [--write-file PATH] [--m 1,16,128,2048] [--shape N,K ...]
 
 The reference only hints at such an interface (``tune(N, K)`` in src/mm/fp32/impl.h:20-23, a
-stub that throws).  Candidates: for M <= 128 the split-K factor of the weight-streaming kernel;
-for M % 128 == 0 the MFMA tile (M = 128 tries both).  Timing: HIP events around a HIP graph of back-to-back launches
+stub that throws).  Candidates: for M <= 128 the split-K factor of the weight-streaming kernel; for 32 < M < 128 also a
+single row of 128 x 128 tiles (a row tail) and its splits; for M % 128 == 0 the MFMA tiles (M = 128 tries both); for the
+FP16 / BF16 GEMM all five tiles.  Timing: HIP events around a HIP graph of back-to-back launches
 that rotate over enough weight copies to defeat the caches (decode shapes) -- the same method
 ``bench.py`` uses.  Without ``--write`` the table is only printed.  ``--write-file PATH`` writes the same
 results as a text file that the library reads at run time when ``LLMMM_TUNE_FILE=PATH`` is set (its entries come
@@ -77,6 +78,8 @@ def tune_shape(M, N, K, iters=40, rotate_bytes=768 << 20, verbose=True):
     if skinny:
         kb = K // 128
         cands = [(_lib.TILE_SKINNY, s) for s in sorted({1, 2, 3, 4, 5, 6, 8, 10, 12, 16, 19, 20, 24, 32, kb, kb // 2}) if 1 <= s <= min(32, kb)]
+    if 32 < M < 128:  # a single row of 128 x 128 tiles whose last rows are not stored
+        cands += [(_lib.TILE_128x128, x) for x in tile_splits if x == 1 or (N // 128) * x <= 640]
     if M % 128 == 0:
         dims = {_lib.TILE_256x256: (256, 256), _lib.TILE_128x256: (128, 256), _lib.TILE_256x128: (256, 128), _lib.TILE_128x128: (128, 128)}
         cands = (cands if skinny else []) + [(t, x) for t, (bm, bn) in dims.items() if M % bm == 0 and N % bn == 0
@@ -199,9 +202,7 @@ def main():
         for M in ms:
             tile, split, _ = tune_shape(M, N, K, iters=args.iters)
             if tile == _lib.TILE_SKINNY:
-                below = [m for m in ms if m < 128]
-                # the largest tuned M below 128 speaks for every M up to 127
-                skinny_rows.append((127 if below and M == max(below) and M > 64 else M, N, K, split))
+                skinny_rows.append((M, N, K, split))  # speaks for every M up to this one that no smaller entry covers
             else:
                 tile_rows.append((M, N, K, tile, split))
             torch.cuda.empty_cache()

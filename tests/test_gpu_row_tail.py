@@ -64,8 +64,12 @@ def test_table_routes_64_to_127_rows_like_128(lib):
     for n, k in ((19456, 2560), (2560, 9728)):
         want = lib.query_config(_lib.OUT_FP8Q, 128, n, k)
         assert want[0] == T128
-        for m in (65, 96, 127):
+        for m in (65, 96, 127) if n == 19456 else (97, 112, 127):
             assert lib.query_config(_lib.OUT_FP8Q, m, n, k) == want
+    # ... unless the table holds a weight-streaming entry measured between 65 and 127 rows (down up to 96 rows: four splits of
+    # 32-row groups beat the tiles)
+    for m in (65, 80, 96):
+        assert lib.query_config(_lib.OUT_FP8Q, m, 2560, 9728) == (SKINNY, 4)
     # an unsplit entry (gate_up: enough column groups to fill the chip) already takes 33 .. 64 rows; a split one (down) does not
     for m in (33, 48, 64):
         assert lib.query_config(_lib.OUT_FP8Q, m, 19456, 2560) == lib.query_config(_lib.OUT_FP8Q, 128, 19456, 2560)
@@ -125,7 +129,8 @@ def test_add_rmsnorm_quant_on_tail_rows_with_the_queried_workspace(lib, oracle, 
     (one unsplit row of 128 x 128 tiles, which has no epilogue of its own and needs one plane), with exactly the
     workspace its query function asks for: hidden == T(C32 + residual), codes and scales == the oracle's on that."""
     from llmmm_amd import _lib
-    assert lib.query_config(_lib.OUT_F32, M, N, K)[0] == T128
+    # (the down projection up to 96 rows: the table sends it to the weight-streaming kernel in four splits -- the same property)
+    assert lib.query_config(_lib.OUT_F32, M, N, K)[0] == (SKINNY if (N, K) == (2560, 9728) and M <= 96 else T128)
     need = _lib.lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K)
     assert need >= M * N * 4
     Aq, As, Bq, Bs = _inputs(oracle, M, N, K, 5)
