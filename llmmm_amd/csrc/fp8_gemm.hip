@@ -196,9 +196,13 @@ __device__ __forceinline__ void fp8_compute_stage(const char LLMMM_LDS* lds, int
   const char LLMMM_LDS*   ldsB = lds + TC::A_BYTES;
   i32x8                   a[MF], b[2];
   f32x4                   p[2][MF];
+  // the first MFMA needs b[0] and a[0] only: they are requested first (pinned: the scheduler would otherwise put all of A
+  // in front), so that it waits for four LDS reads instead of eleven while all eight waves read at once behind the barrier
   b[0] = fp8_read_frag(ldsB, b_rd0, b_rd1, 0);
+  a[0] = fp8_read_frag(ldsA, a_rd0, a_rd1, 0);
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int mf = 0; mf < MF; ++mf) a[mf] = fp8_read_frag(ldsA, a_rd0, a_rd1, mf * 2048);
+  for (int mf = 1; mf < MF; ++mf) a[mf] = fp8_read_frag(ldsA, a_rd0, a_rd1, mf * 2048);
 #pragma unroll
   for (int nf = 0; nf < NF; ++nf) {
     const int cur = nf & 1;
