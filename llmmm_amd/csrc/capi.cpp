@@ -241,7 +241,10 @@ bool lookup_tile_in(const Table& table, int M, int N, int K, int* tile, int* spl
   for (const auto& e : table) {
     if (e.N != N || e.K != K) continue;
     int bm, bn;
-    if (!tile_dims(e.tile, bm, bn) || M % bm || N % bn) continue;
+    if (!tile_dims(e.tile, bm, bn) || N % bn) continue;
+    // (an entry for fewer than 128 rows is a row tail of 128 x 128 tiles and speaks for exactly its M)
+    if (M % bm && !(M < 128 && e.M == M && e.tile == LLMMM_TILE_128x128)) continue;
+    if (e.M < 128 && e.M != M) continue;
     const double ratio = e.M > M ? (double)e.M / M : (double)M / e.M;
     if (ratio < *best_ratio) {
       *best_ratio = ratio, *tile = e.tile, *split = e.M == M ? e.split_k : 0;

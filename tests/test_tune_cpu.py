@@ -79,3 +79,23 @@ def test_the_compiled_in_header_parses_back_to_what_renders_it():
     skinny, tile, fp16 = tune.parse_header(text)
     assert skinny and tile and fp16 and all(len(r) == 4 for r in skinny) and all(len(r) == 5 for r in tile + fp16)
     assert tune.render_table(skinny, tile, fp16).rstrip() == text.rstrip()
+
+
+def test_entries_for_fewer_than_128_rows(tmp_path):
+    """A tile entry with M < 128 names a row tail of 128 x 128 tiles for exactly that M; a weight-streaming entry whose m_max
+    lies between 65 and 127 goes before the row-tail tiles that M = 128 would hand down."""
+    path = tmp_path / "tune.txt"
+    path.write_text("tile 80 4096 4096 3 2\ntile 128 4096 4096 3 1\ntile 72 4096 4096 0 1\nskinny 100 8192 4096 3\ntile 128 8192 4096 3 1\n")
+    prog = textwrap.dedent("""
+        import sys
+        sys.path.insert(0, %r)
+        import llmmm_amd
+        from llmmm_amd import _lib
+        q = lambda *a: llmmm_amd.query_config(_lib.OUT_FP8Q, *a)
+        print(q(80, 4096, 4096), q(96, 4096, 4096), q(72, 4096, 4096), q(128, 4096, 4096), q(256, 4096, 4096)[0], q(90, 8192, 4096), q(110, 8192, 4096))
+    """ % ROOT)
+    res = subprocess.run([sys.executable, "-c", prog], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=dict(os.environ, LLMMM_TUNE_FILE=str(path)))
+    assert res.returncode == 0, res.stderr
+    # 80 rows: its own entry; 96 and 72 rows: what M = 128 hands down (the 256 x 256 entry for 72 rows cannot be a row tail);
+    # 256 rows: not the 80-row entry; 90 rows of the other shape: the streaming entry, 110 rows: beyond its m_max -> tiles
+    assert res.stdout.strip() == "(3, 2) (3, 1) (3, 1) (3, 1) 3 (8, 3) (3, 1)", res.stdout
