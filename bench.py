@@ -883,6 +883,16 @@ def main():
             nb = m * 2560 * 3.0 + m * 20 * 4.0
             shapes.append({"name": "rmsnorm_quant_bf16_m%d_k2560" % m, "M": m, "K": 2560, "us": ms_ * 1e3, "hbm_gbs": nb / ms_ * 1e-6,
                            "frac_of_hbm_peak": nb / ms_ * 1e-6 / PEAK_HBM_GBS})
+        # The blockwise quantiser (examples/005.fp8.mm.cu:439-563) on the 4096^2 operands of the FP8 workload: activations
+        # 1x128 with transposed scales, weights 128x128.  Algorithmic bytes: 4 read + 1 written per element, plus the scales.
+        xq = torch.randn((4096, 4096), device="cuda")
+        qq = torch.empty((4096, 4096), device="cuda", dtype=torch.uint8)
+        for qname, qm, ns in (("quant_1x128_4096x4096", 1, 32 * 4096), ("quant_128x128_4096x4096", 128, 32 * 32)):
+            sq = torch.empty(ns, device="cuda")
+            ms_, _ = _events_ms(lambda: llmmm_amd.fp8_blockwise_symmetric_quantization(xq, qq, sq, 4096, 4096, qm, 128, qm == 1), s2, w2, graph=True)
+            nb = 4096.0 * 4096.0 * 5.0 + ns * 4.0
+            shapes.append({"name": qname, "us": ms_ * 1e3, "hbm_gbs": nb / ms_ * 1e-6, "frac_of_hbm_peak": nb / ms_ * 1e-6 / PEAK_HBM_GBS})
+        del xq, qq
         # One decoder MLP block as three launches: RMSNorm+quant -> gate_up GEMM with fused SwiGLU output -> down GEMM
         # (bf16 output), weights pre-shuffled and rotated over distinct copies so that they stream from HBM.
         for m in (1, 16):
