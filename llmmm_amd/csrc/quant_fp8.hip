@@ -67,25 +67,37 @@ __global__ void __launch_bounds__(256) quant_1x128_kernel(const float* __restric
   const int mbeg  = blockIdx.y * rows_per_wg;
   const int mend  = min(M, mbeg + rows_per_wg);
   const bool live = n < N;
-  for (int m = mbeg + sub; m < mend; m += 8) {
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    if (live) v = __builtin_nontemporal_load((const f32x4*)(x + (size_t)m * N + n));
-    float a = QUANT_AMAX_SEED;
-    if (live) a = amax4(a, v);
-    a       = wave_xor_max(a, 1);
-    a       = wave_xor_max(a, 2);
-    a       = wave_xor_max(a, 4);
-    a       = wave_xor_max(a, 8);
-    a       = wave_xor_max(a, 16);
-    const float s = a / 448.f;
-    uint32_t    c = 0;
-    if (s != 0.f) c = q_pack_quotients_e4m3x4(v, s);
-    if (live) *(uint32_t*)(q + (size_t)m * N + n) = c;
-    if (l32 == 0) {
-      if (TRANSPOSE)
-        scale[(size_t)nb * M + m] = s;
-      else
-        scale[(size_t)m * nbn + nb] = s;
+  // four rows per thread and pass: their loads go out together, before the first row's cross-lane amax and divisions
+  constexpr int U = 4;
+  for (int m0 = mbeg + sub; m0 < mend; m0 += 8 * U) {
+    f32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int m = m0 + 8 * u;
+      v[u]        = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (live && m < mend) v[u] = __builtin_nontemporal_load((const f32x4*)(x + (size_t)m * N + n));
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int m = m0 + 8 * u;
+      if (m >= mend) break;  // uniform over the half-wavefront that shares the row
+      float a = QUANT_AMAX_SEED;
+      if (live) a = amax4(a, v[u]);
+      a       = wave_xor_max(a, 1);
+      a       = wave_xor_max(a, 2);
+      a       = wave_xor_max(a, 4);
+      a       = wave_xor_max(a, 8);
+      a       = wave_xor_max(a, 16);
+      const float s = a / 448.f;
+      uint32_t    c = 0;
+      if (s != 0.f) c = q_pack_quotients_e4m3x4(v[u], s);
+      if (live) *(uint32_t*)(q + (size_t)m * N + n) = c;
+      if (l32 == 0) {
+        if (TRANSPOSE)
+          scale[(size_t)nb * M + m] = s;
+        else
+          scale[(size_t)m * nbn + nb] = s;
+      }
     }
   }
 }
