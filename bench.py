@@ -923,15 +923,16 @@ def main():
             ms_, _ = _events_ms(lambda: torch.matmul(A, B, out=C), max(10, args.steps // 2), max(3, args.warmup // 2), graph=True)
             comp["torch_matmul_fp16_%d_tflops" % m] = 2.0 * m * n * k / ms_ * 1e-9
             comp["torch_matmul_fp16_%d_us" % m] = ms_ * 1e3
-        # a shape whose 256 x 256 tiles end in a partly filled round (608 tiles): the two-shape launch beside the vendor library
-        m, n, k = 2048, 19456, 2560
-        A, B = fp16_inputs(m, n, k)
-        C = torch.empty((m, n), dtype=torch.float16, device="cuda")
-        ms_, _ = _events_ms(lambda: llmmm_amd.fp16_gemm(A, B, C), max(10, args.steps // 5), max(3, args.warmup // 5), graph=True)
-        comp["fp16_gemm_2048x19456x2560_tflops"] = 2.0 * m * n * k / ms_ * 1e-9
-        ms_, _ = _events_ms(lambda: torch.matmul(A, B, out=C), max(10, args.steps // 5), max(3, args.warmup // 5), graph=True)
-        comp["torch_matmul_fp16_2048x19456x2560_tflops"] = 2.0 * m * n * k / ms_ * 1e-9
-        del A, B, C
+        # a shape whose 256 x 256 tiles end in a partly filled round (608 tiles: the two-shape launch), the two non-square shapes
+        # of the reference's own test (test/fp16_mm_test.cc:98-103) and a long-K projection, beside the vendor library
+        for m, n, k in ((2048, 19456, 2560), (4096, 6144, 2048), (4096, 2048, 12288), (2048, 2560, 9728)):
+            A, B = fp16_inputs(m, n, k)
+            C = torch.empty((m, n), dtype=torch.float16, device="cuda")
+            ms_, _ = _events_ms(lambda: llmmm_amd.fp16_gemm(A, B, C), max(10, args.steps // 5), max(3, args.warmup // 5), graph=True)
+            comp["fp16_gemm_%dx%dx%d_tflops" % (m, n, k)] = 2.0 * m * n * k / ms_ * 1e-9
+            ms_, _ = _events_ms(lambda: torch.matmul(A, B, out=C), max(10, args.steps // 5), max(3, args.warmup // 5), graph=True)
+            comp["torch_matmul_fp16_%dx%dx%d_tflops" % (m, n, k)] = 2.0 * m * n * k / ms_ * 1e-9
+            del A, B, C
         try:
             # the vendor library's FP8 GEMM (one scale per tensor, bf16 out: a simpler contract than 1x128 / 128x128 blocks)
             g8 = torch.Generator(device="cuda").manual_seed(7)
