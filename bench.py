@@ -6,13 +6,15 @@
 A "step" is one GEMM launch through the C ABI (``libllmmm.so``) on inputs already resident in
 HBM.  The headline workload is the FP16 GEMM at M=N=K=4096 (A ~ N(0,1), B ~ N(0,0.02), seed 2,
 fp32 accumulation, fp16 output, one kernel, no split-K); ``value`` is its TFLOP/s
-(2*M*N*K / time).  One JSON line is printed, carrying as well
+(2*M*N*K / time).  The LAST line of stdout is the record: one compact strict-JSON object (a few KB) with
   * ``roofline``: the dominant kernel against MI355X's published dense MFMA peak (or HBM peak
     for the decode shapes), from HIP events recorded on the launch stream around the timed
-    region;
+    region; ``roofline.targets``: FP16 4096^3, FP8 fused 4096^3 and the decode projections at M = 1 and 16,
+    each with its microseconds and fraction of the published peak;
   * ``cpu_baseline``: the CPU oracle (a port of the reference's Kahan GEMM, test/kahan.cu:16-26)
-    timed on this host's cores on a bounded sample of the same workload;
-  * ``shapes``: TFLOP/s (and GB/s for M <= 16) of the other benchmark shapes, measured the same way.
+    timed on this host's cores on a bounded sample of the same workload.
+The lines before it, one JSON object each with a ``detail`` key, carry the per-shape table (``shapes``), the
+side-by-side vendor-library comparison, the measured peaks, the other CPU baselines and the full target rows.
 """
 import argparse
 import json
@@ -27,12 +29,43 @@ PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "fp8": 5000.0}  # MI355X dense MFM
 PEAK_HBM_GBS = 8000.0
 PREHEAT_S = 0.25  # seconds of untimed launches before the warm-up steps of every measurement
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE + WRITE_SIZE counter runs of
-# these same workloads, each scaled by the counter's reading for a 1 GiB device copy (FETCH_SIZE x 2.0 KiB,
-# WRITE_SIZE x 1.0 KiB per count).  Counters cannot be read from inside this process, so the figures are
-# carried here; the summaries they come from are kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"fp16_gemm_4096": 235.1e6, "fp8_gemm_fused_4096": 119.2e6, "decode_gate_up_m1": 50.0e6,
-                          "decode_gate_up_m1_pre": 50.0e6, "decode_o_m1_bf16_pre": 10.6e6}
+# HBM bytes per launch of the dominant kernel come from rocprofv3 FETCH_SIZE + WRITE_SIZE counter runs of these same
+# workloads (counters cannot be read from inside this process).  The summaries under profiles/ carry the result
+# ("traffic = X MB per launch") and the SHA-256 of the kernel source file they were taken on; a summary whose hash is
+# not that of the source in this tree is stale and yields traffic = null.
+HERE = os.path.dirname(os.path.abspath(__file__))
+TRAFFIC_PROFILES = {
+    "fp16_gemm_4096": ("fp16_gemm_kernel_4096.txt", "fp16_gemm.hip"),
+    "fp8_gemm_fused_4096": ("fp8_gemm_kernel_fused_4096.txt", "fp8_gemm.hip"),
+    "decode_gate_up_m1": ("fp8_skinny_kernel_gate_up_m1.txt", "fp8_skinny.hip"),
+    "decode_gate_up_m1_pre": ("fp8_skinny_kernel_gate_up_m1_preshuffled.txt", "fp8_skinny.hip"),
+}
+
+
+def source_sha256(name):
+    import hashlib
+    with open(os.path.join(HERE, "llmmm_amd", "csrc", name), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()
+
+
+def measured_traffic(workload):
+    """(bytes per launch, note) from the counter summary of this workload, or (None, why not)."""
+    import re
+    if workload not in TRAFFIC_PROFILES:
+        return None, "no counter summary for this workload"
+    fname, src = TRAFFIC_PROFILES[workload]
+    try:
+        text = open(os.path.join(HERE, "profiles", fname)).read()
+    except OSError:
+        return None, "profiles/%s missing" % fname
+    mt = re.search(r"traffic = ([0-9.]+) MB per launch", text)
+    mh = re.search(r"sha256\(%s\) = ([0-9a-f]{64})" % re.escape(src), text)
+    if not mt or not mh:
+        return None, "profiles/%s carries no traffic figure or no source hash" % fname
+    if mh.group(1) != source_sha256(src):
+        return None, "profiles/%s was taken on another version of %s" % (fname, src)
+    return float(mt.group(1)) * 1e6, "profiles/%s" % fname
+
 
 QWEN3_4B = {"qkv": (6144, 2560), "o": (2560, 4096), "gate_up": (19456, 2560), "down": (2560, 9728)}
 
@@ -136,6 +169,24 @@ def sample_clock_power(step, seconds=1.2):
     mhz = sorted(x[0] for x in samples if x[0] is not None)
     watts = sorted(x[1] for x in samples if x[1] is not None)
     return {"sclk_mhz": mhz[len(mhz) // 2] if mhz else None, "power_w": watts[len(watts) // 2] if watts else None, "samples": len(samples)}
+
+
+def _finite(x):
+    """x with every float that strict JSON cannot carry (NaN, +-Inf) replaced by None."""
+    if isinstance(x, float):
+        return x if np.isfinite(x) else None
+    if isinstance(x, dict):
+        return {k: _finite(v) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [_finite(v) for v in x]
+    if isinstance(x, (np.floating, np.integer)):
+        return _finite(x.item())
+    return x
+
+
+def emit_detail(name, obj):
+    """One JSON object on a line of its own, ahead of the final record."""
+    print(json.dumps(_finite({"detail": name, **obj}), allow_nan=False), flush=True)
 
 
 def fp16_inputs(M, N, K, dtype=torch.float16, seed=2):
@@ -811,7 +862,10 @@ def main():
         print("unknown workload", w, file=sys.stderr)
         sys.exit(2)
 
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(w) if not mk else None
+    if mk:
+        roof["traffic"], roof["traffic_source"] = None, "no counter summary for this workload"
+    else:
+        roof["traffic"], roof["traffic_source"] = measured_traffic(w)
     roof["algorithmic_bytes"] = r["bytes"]
     clk = r.get("clock") if isinstance(r, dict) else None
     if clk and clk.get("sclk_mhz") and roof["bound"] == "mfma":
@@ -822,7 +876,7 @@ def main():
     line = {
         "metric": "TFLOPS (% of MI355X FP8/FP16 MFMA peak) at 4096\u00b3; HBM GB/s at M\u226416 decode",
         "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms"],
-        "wall_ms_per_step": r["wall_ms"], "timing": "median of %d batches of `steps` launches (one HIP-graph replay each), events per batch; min %.5f max %.5f ms per step"
+        "wall_ms_per_step": r["wall_ms"], "timing": "median of %d HIP-graph replays of `steps` launches, events per replay; min %.5f max %.5f ms per step"
         % (TIMED_BATCHES, r.get("ms_min") or r["ms"], r.get("ms_max") or r["ms"]), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
         "data": "synthetic", "config": cfg, "roofline": roof,
     }
@@ -911,7 +965,7 @@ def main():
         for m, cs in ((1, False), (1, True), (2, True), (16, False)):
             shapes.append(bench_decoder_layer(m, sd, w2, consumer_side=cs))
             torch.cuda.empty_cache()
-        line["shapes"] = shapes
+        emit_detail("shapes", {"shapes": shapes})
 
     if not args.no_shapes:
         # Side-by-side comparison only (never part of the product or of `value`): the vendor library behind torch.matmul
@@ -947,24 +1001,31 @@ def main():
             comp["torch_scaled_mm_fp8_tensorwise_4096_tflops"] = None
             comp["torch_scaled_mm_error"] = str(e)[:160]
         comp["note"] = "hipBLASLt via torch.matmul / torch._scaled_mm, same timing method; reported for comparison only"
-        line["comparison"] = comp
+        emit_detail("comparison", comp)
     if not args.no_peaks:
         # the same kernel against what this very part sustains: random-operand MFMA rate / streaming read rate
         mp = measured_peaks()
-        line["measured_peaks"] = mp
+        emit_detail("measured_peaks", mp)
         key = {"f16": "mfma_f16_random_operands_tflops", "bf16": "mfma_bf16_random_operands_tflops", "fp8": "mfma_fp8_random_operands_tflops"}[dtype]
         roof["peak_measured"] = mp["hbm_read_1gib_gbs"] if roof["bound"] == "hbm" else mp[key]
         roof["frac_of_measured"] = roof["achieved"] / roof["peak_measured"]
     if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline(4096, 4096, 4096, args.cpu_rows)
+        cb = cpu_baseline(4096, 4096, 4096, args.cpu_rows)
+        emit_detail("cpu_baseline_others", {"others": cb.pop("others")})
+        line["cpu_baseline"] = cb
     else:
         line["cpu_baseline"] = None
     if not args.no_targets:
-        # last key of the line, and inside `roofline` as well: all three figures of the metric in one place
+        # all three figures of the metric, measured in this run: the full rows (read ceilings, GB/s, kernels) go out as a
+        # detail line, the final line keeps microseconds, the fraction of the published peak and the number of kernels
         tg = bench_targets(max(20, args.steps), max(3, args.warmup), headline=r if w == "fp16_gemm_4096" else None)
-        roof["targets"] = tg
-        line["targets"] = tg
-    print(json.dumps(line))
+        emit_detail("targets", tg)
+        roof["targets"] = {k: {"us": v["us"], "frac": v["frac"], "target": v["target"], "kernels": v["kernel"].count("+") + 1}
+                           for k, v in tg.items() if isinstance(v, dict)}
+        roof["targets_note"] = "frac = achieved / published peak (2500 TFLOP/s f16, 5000 fp8, 8000 GB/s for decode_*); _pre = pre-shuffled weights, _bf16 = bf16 output"
+    # The last line of stdout is the record: strict JSON, a few KB.  Everything else was printed above it, one JSON
+    # object per line, each with a "detail" key.
+    print(json.dumps(_finite(line), allow_nan=False), flush=True)
 
 
 if __name__ == "__main__":

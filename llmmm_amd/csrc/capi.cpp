@@ -2,6 +2,7 @@
 // Mirrors the reference's host launchers: no allocation, no synchronisation, work enqueued on
 // the caller's stream (src/mm/fp16/mm.cu:6-42, examples/005.fp8.mm.cu:2466-2500).
 #include "../../include/llmmm.h"
+#include "../../include/llmmm_probe.h"
 #include "kernels.h"
 #include "tune_table.h"
 
@@ -209,6 +210,13 @@ const TuneOverride& tune_override()
     int  lineno = 0;
     while (fgets(line, sizeof(line), f)) {
       ++lineno;
+      if (!strchr(line, '\n') && !feof(f)) {
+        // longer than the buffer: no entry is, so the whole line is dropped (its tail must not be read as a new entry)
+        int ch;
+        while ((ch = fgetc(f)) != EOF && ch != '\n') {}
+        fprintf(stderr, "llmmm: %s:%d: line too long, ignored\n", path, lineno);
+        continue;
+      }
       if (char* h = strchr(line, '#')) *h = 0;
       char kind[16];
       int  a, b, c, d, e;
@@ -217,10 +225,12 @@ const TuneOverride& tune_override()
       int bm, bn;
       if (n == 5 && !strcmp(kind, "skinny") && a >= 1 && a <= SKINNY_MAX_M && b > 0 && c > 0 && d >= 1 && d <= MAX_SPLIT_K)
         o.skinny.push_back({a, b, c, d});
+      // (a tile must divide the shape it is entered for -- an entry that does not would turn a call the heuristic serves
+      // into "not aligned"; the one exception is a row tail: fewer than 128 rows in 128 x 128 tiles)
       else if (n == 6 && !strcmp(kind, "tile") && a > 0 && b > 0 && c > 0 && tile_dims(d, bm, bn) && d != LLMMM_TILE_64x128 && d != LLMMM_TILE_128x160 && e >= 0 &&
-               e <= MAX_SPLIT_K)
+               e <= MAX_SPLIT_K && b % bn == 0 && (a % bm == 0 || (a < 128 && d == LLMMM_TILE_128x128)))
         o.tile.push_back({a, b, c, d, e});
-      else if (n == 5 && !strcmp(kind, "fp16") && a > 0 && b > 0 && c > 0 && tile_dims(d, bm, bn) && d != LLMMM_TILE_128x160)
+      else if (n == 5 && !strcmp(kind, "fp16") && a > 0 && b > 0 && c > 0 && tile_dims(d, bm, bn) && d != LLMMM_TILE_128x160 && a % bm == 0 && b % bn == 0)
         o.fp16.push_back({a, b, c, d, 1});
       else
         fprintf(stderr, "llmmm: %s:%d: not a tune entry, ignored\n", path, lineno);
@@ -275,10 +285,15 @@ bool lookup_skinny(int M, int N, int K, int* split, int* m_max = nullptr)
 }
 bool lookup_fp16_tile(int M, int N, int K, int* tile)
 {
+  // (an entry whose tile does not divide the shape is no entry: the heuristic decides)
+  auto fits = [&](int t) {
+    int bm, bn;
+    return tile_dims(t, bm, bn) && M % bm == 0 && N % bn == 0;
+  };
   for (const auto& e : tune_override().fp16)
-    if (e.M == M && e.N == N && e.K == K) return *tile = e.tile, true;
+    if (e.M == M && e.N == N && e.K == K && fits(e.tile)) return *tile = e.tile, true;
   for (const auto& e : llmmm::kFp16TileTune)
-    if (e.M == M && e.N == N && e.K == K) return *tile = e.tile, true;
+    if (e.M == M && e.N == N && e.K == K && fits(e.tile)) return *tile = e.tile, true;
   return false;
 }
 
@@ -373,6 +388,18 @@ int skinny_split_for(int M, int N, int K)
   return lookup_skinny(M, N, K, &sp) ? sp : heuristic_split(M, N, K);
 }
 
+// Planes a strip-capable shape needs when the call turns out not to run in strips after all: activations the kernel makes
+// itself (cfg.a_layout) and explicit splits belong to the split-K form, and generated activations need a split whose K
+// range fits the staging buffer.  The size queries cannot see the caller's cfg, so they answer for this case.
+size_t strip_fallback_plane_bytes(int M, int N, int K)
+{
+  int s = skinny_split_for(M, N, K);
+  const int kb = K / 128, min_split = (kb + 31) / 32;  // = agen_min_split(K)
+  if (s < min_split) s = min_split;
+  if (s > max_split_for(K)) s = max_split_for(K);
+  return (size_t)(s < 1 ? 1 : s) * M * N * sizeof(float);
+}
+
 int choose_fp8_out(int out_kind, int M, int N, int K, llmmm_gemm_cfg* cfg)
 {
   const int rc = choose_fp8(M, N, K, cfg);
@@ -462,6 +489,7 @@ size_t llmmm_fp8_gemm_workspace(int out_kind, int M, int N, int K)
   if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
   llmmm_gemm_cfg cfg;
   if (choose_fp8_out(out_kind, M, N, K, &cfg) != LLMMM_OK) return 0;
+  if (cfg.tile == LLMMM_TILE_STRIP) return strip_fallback_plane_bytes(M, N, K);  // strips need none; a call with generated activations leaves them
   const int  s       = cfg.split_k;  // the split the library would pick (an explicit cfg->split_k = S needs S planes)
   const bool narrow  = cfg.tile == LLMMM_TILE_256x128 || cfg.tile == LLMMM_TILE_128x128;
   const bool a_plane = out_kind == LLMMM_OUT_FP8Q_SWIGLU && (cfg.tile == LLMMM_TILE_SKINNY || narrow);  // SwiGLU outside a 256-column tile
@@ -500,7 +528,9 @@ size_t llmmm_fp8_planes_rmsnorm_a_workspace(int M, int N, int K)
 {
   llmmm_gemm_cfg cfg;
   if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
-  if (cfg.tile == LLMMM_TILE_SKINNY && M <= AGEN2_MAX_M && K <= AGEN2_MAX_K) return 0;
+  // (the generating kernel writes fp32 only: any other output kind goes through one fp32 plane and the reduce kernel, and
+  // an unsplit call has no plane in llmmm_fp8_gemm_workspace's answer -- this one covers it)
+  if (cfg.tile == LLMMM_TILE_SKINNY && M <= AGEN2_MAX_M && K <= AGEN2_MAX_K) return (size_t)M * N * sizeof(float);
   return swiglu_a_bytes(M, K);  // the same codes + scales block
 }
 
@@ -757,7 +787,7 @@ static size_t plane_route_workspace(int M, int N, int K, bool wide_ok)
   llmmm_gemm_cfg cfg;
   if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
   if (wide_ok) prefer_wide_tile(&cfg, M, N), prefer_strip(&cfg, M, N, K);
-  if (cfg.tile == LLMMM_TILE_STRIP) return 0;  // epilogue inside the strip kernel
+  if (cfg.tile == LLMMM_TILE_STRIP) return strip_fallback_plane_bytes(M, N, K);  // strips need none (epilogue inside the kernel); a call with generated activations leaves them
   int split = cfg.split_k < 1 ? 1 : cfg.split_k;
   if (split > max_split_for(K)) split = max_split_for(K);
   int bm = 0, bn = 0;
@@ -913,8 +943,13 @@ size_t llmmm_fp8_gemm_planes_bytes(int M, int N, int K)
   if (M <= 0 || N <= 0 || K <= 0 || N % 128 || K % 128) return 0;
   llmmm_gemm_cfg cfg;
   if (choose_fp8(M, N, K, &cfg) != LLMMM_OK) return 0;
-  prefer_strip(&cfg, M, N, K);  // (one plane then: split_k = 1)
-  return (size_t)(cfg.split_k < 1 ? 1 : cfg.split_k) * M * N * sizeof(float);
+  const size_t own = (size_t)(cfg.split_k < 1 ? 1 : cfg.split_k) * M * N * sizeof(float);
+  prefer_strip(&cfg, M, N, K);  // (strips write one plane; a call with generated activations leaves them for the split-K form)
+  if (cfg.tile == LLMMM_TILE_STRIP) {
+    const size_t fb = strip_fallback_plane_bytes(M, N, K);
+    return fb > own ? fb : own;
+  }
+  return own;
 }
 
 int llmmm_fp8_gemm_planes(const void* A, const float* As, const void* Bt, const float* Bs, int M, int N, int K, float* planes, size_t planes_bytes,

@@ -190,6 +190,17 @@ __device__ __forceinline__ uint32_t pack_e4m3x4_sat(float a, float b, float c, f
   return ((uint32_t)v & ~nan) | (0x7F7F7F7Fu & nan);
 }
 
+// 448 / amax of the fused re-quantisation (examples/005.fp8.mm.opt.cu:439-446), or 0 where that quotient is not finite: a
+// group of zeros (the reference multiplies by 448 / 0 and writes NaN codes) and a group so small -- amax below 2^-119 --
+// that the reciprocal overflows (the reference then writes +-448 for every non-zero element and NaN for the zeros).
+// Such a group gets codes 0 (a NaN element stays NaN, 0x7F) next to its scale amax / 448; with a finite reciprocal every
+// product lies within +-448 (1 + 2^-20), which is what pack_e4m3x4_in_range asks for.
+__device__ __forceinline__ float requant_inv(float amax)
+{
+  const float inv = 448.f / amax;
+  return inv < __builtin_inff() ? inv : 0.f;
+}
+
 // Four consecutive row elements of type float / bf16 / fp16 <-> fp32 (one 16- or 8-byte access).
 template <typename IN_T>
 __device__ __forceinline__ f32x4 load_row4(const IN_T* p);

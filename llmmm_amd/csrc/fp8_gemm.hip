@@ -285,7 +285,7 @@ __device__ __forceinline__ void swiglu_finish(const f32x4 (&acc)[8][MF], const f
     amax              = wave_xor_max(amax, 16);
     amax              = wave_xor_max(amax, 32);
     const float scale = amax / 448.f;
-    const float inv   = amax > 0.f ? 448.f / amax : 0.f;
+    const float inv   = requant_inv(amax);
     const int   r     = h * 16 + li;
 #pragma unroll
     for (int nf = 0; nf < 8; ++nf)
@@ -745,7 +745,7 @@ __device__ __forceinline__ void fp8_gemm_body(const uint8_t* __restrict__ A, con
       amax              = wave_xor_max(amax, 16);
       amax              = wave_xor_max(amax, 32);
       const float scale = amax / 448.f;
-      const float inv   = amax > 0.f ? 448.f / amax : 0.f;
+      const float inv   = requant_inv(amax);
       const int   r     = mf * 16 + li;
 #pragma unroll
       for (int nf = 0; nf < 8; ++nf) {
@@ -877,7 +877,7 @@ fp8_splitk_reduce_kernel(const float* __restrict__ planes, int S, void* __restri
       a       = wave_xor_max(a, 8);
       a       = wave_xor_max(a, 16);
       const float scale = a / 448.f;
-      const float inv   = a > 0.f ? 448.f / a : 0.f;
+      const float inv   = requant_inv(a);
       *(uint32_t*)((uint8_t*)Cv + (size_t)m * ldc + n) = pack_e4m3x4_in_range(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
       if (l32 == 0) Cs[(size_t)nb * M + m] = scale;
     }
@@ -952,7 +952,7 @@ fp8_planes_qk_norm_rope_kernel(const float* __restrict__ planes, int S, void* __
 #pragma unroll
       for (int step = 1; step <= 16; step <<= 1) a = wave_xor_max(a, step);
       const float scale = a / 448.f;
-      const float inv   = a > 0.f ? 448.f / a : 0.f;
+      const float inv   = requant_inv(a);
       *(uint32_t*)((uint8_t*)Cv + (size_t)m * N + n) = pack_e4m3x4_in_range(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
       if (l32 == 0) Cs[(size_t)head * M + m] = scale;
     }

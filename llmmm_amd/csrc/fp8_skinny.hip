@@ -314,15 +314,25 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
     const bool   live   = rsel < M;
     for (int x = tid; x < nsl * 128; x += 512) *(i32x4 LLMMM_LDS*)((char LLMMM_LDS*)a_stage + x * 16) = i32x4{0, 0, 0, 0};
     for (int x = tid; x < nsl * 16; x += 512) a_scale[x] = 0.f;
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * LOADS) : "memory");  // the operand's loads are in; the ring's stay in flight
+    // The operand's loads are in once at most the ring's D * LOADS loads are outstanding.  Every destination register of
+    // those early loads is an in/out operand of the wait itself, so the values the code below reads are, to the compiler,
+    // results of this instruction: nothing that uses them can be placed in front of it.  (One statement per chunk column:
+    // twelve 128-bit operands each; the second and third find the count already met.)
+    static_assert(GP == 10, "the operand list below names ten planes");
 #pragma unroll
     for (int u = 0; u < 3; ++u) {
       if constexpr (sizeof(HT) == 4)
-        asm volatile("" : "+v"(g_res[u]), "+v"(g_w[u]));
+        asm volatile("s_waitcnt vmcnt(%12)"
+                     : "+v"(g_res[u]), "+v"(g_w[u]), "+v"(g_p[0][u]), "+v"(g_p[1][u]), "+v"(g_p[2][u]), "+v"(g_p[3][u]), "+v"(g_p[4][u]), "+v"(g_p[5][u]),
+                       "+v"(g_p[6][u]), "+v"(g_p[7][u]), "+v"(g_p[8][u]), "+v"(g_p[9][u])
+                     : "n"(D * LOADS)
+                     : "memory");
       else
-        asm volatile("" : "+v"(g_res2[u]), "+v"(g_w[u]));
-#pragma unroll
-      for (int v = 0; v < GP; ++v) asm volatile("" : "+v"(g_p[v][u]));
+        asm volatile("s_waitcnt vmcnt(%12)"
+                     : "+v"(g_res2[u]), "+v"(g_w[u]), "+v"(g_p[0][u]), "+v"(g_p[1][u]), "+v"(g_p[2][u]), "+v"(g_p[3][u]), "+v"(g_p[4][u]), "+v"(g_p[5][u]),
+                       "+v"(g_p[6][u]), "+v"(g_p[7][u]), "+v"(g_p[8][u]), "+v"(g_p[9][u])
+                     : "n"(D * LOADS)
+                     : "memory");
     }
     f32x4 held[3], rv[3], wv[3];
 #pragma unroll
@@ -401,9 +411,11 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
     // (row, slice) tasks are dealt round-robin to the 16 half-waves: for M = 1 every half-wave has one slice to make.
     // The first batch was requested in front of the ring prologue: once at most D * LOADS loads are outstanding it is in.
     const int nsl = kb1 - kb0, rows = min(M, 16), tasks = nsl * rows;
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * LOADS) : "memory");
-#pragma unroll
-    for (int u = 0; u < 4; ++u) asm volatile("" : "+v"(g_gate[u]), "+v"(g_up[u]));
+    // (the early loads' destinations are in/out operands of the wait: what is read below is, to the compiler, its result)
+    asm volatile("s_waitcnt vmcnt(%8)"
+                 : "+v"(g_gate[0]), "+v"(g_up[0]), "+v"(g_gate[1]), "+v"(g_up[1]), "+v"(g_gate[2]), "+v"(g_up[2]), "+v"(g_gate[3]), "+v"(g_up[3])
+                 : "n"(D * LOADS)
+                 : "memory");
     for (int t0 = tid >> 5; t0 < tasks; t0 += 16 * 4) {  // four tasks of a half-wave per batch
       f32x4 gv[4], uv[4];
       if (t0 < 16) {
@@ -431,7 +443,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
 #pragma unroll
           for (int step = 1; step <= 16; step <<= 1) a = wave_xor_max(a, step);
           const float scale = a / 448.f;
-          const float inv   = a > 0.f ? 448.f / a : 0.f;
+          const float inv   = requant_inv(a);
           *(uint32_t LLMMM_LDS*)((char LLMMM_LDS*)a_stage + j * 2048 + kmajor_offset<SWZ_ROWS16>(r, l32 >> 2) + (l32 & 3) * 4) =
             pack_e4m3x4_in_range(h[0] * inv, h[1] * inv, h[2] * inv, h[3] * inv);
           if (l32 == 0) a_scale[j * 16 + r] = scale;
@@ -520,7 +532,7 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
 #pragma unroll
       for (int w = 0; w < 8; ++w) amax = fmaxf(amax, wave_amax[w][mb][i]);
       const float scale = amax / 448.f;
-      const float inv   = amax > 0.f ? 448.f / amax : 0.f;
+      const float inv   = requant_inv(amax);
       if (m < M) {
         *(uint32_t*)(C + (size_t)m * N + ncol) =
           pack_e4m3x4_in_range(acc[mb][0] * inv, acc[mb][1] * inv, acc[mb][2] * inv, acc[mb][3] * inv);

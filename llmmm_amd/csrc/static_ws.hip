@@ -57,10 +57,12 @@ extern "C" int llmmm_fp8_gemm_static_ws(int out_kind, const void* A, const float
   if (need > (size_t)LLMMM_STATIC_WS_BYTES)
     return llmmm::report_error(LLMMM_ERR_WORKSPACE, "M = %d, N = %d, K = %d needs %zu bytes of split-K planes, the built-in array holds %zu: use llmmm_fp8_gemm with a workspace",
                                M, N, K, need, (size_t)LLMMM_STATIC_WS_BYTES);
-  void* ws = nullptr;
-  if (need) {
-    const int rcs = scratch_on_current_device(&ws);
-    if (rcs) return rcs;
-  }
-  return llmmm_fp8_gemm_ex(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, ws, need, nullptr, stream);
+  // The two runtime queries of this path -- the array's address and the device's CU count -- are made on every call,
+  // whatever the shape needs: both are answered from memory after the first, so any warm-up call on a device makes
+  // every later call on it free of runtime queries, as stream capture requires.
+  void*     ws  = nullptr;
+  const int rcs = scratch_on_current_device(&ws);
+  if (rcs) return rcs;
+  (void)llmmm::num_cus();
+  return llmmm_fp8_gemm_ex(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, need ? ws : nullptr, need, nullptr, stream);
 }

@@ -172,6 +172,13 @@ def _a_operand(A, As, M, K, a_swiglu):
     return _ptr(A, "A", _FP8_DTYPES, M * K), _ptr(As, "A_scale_transposed", (torch.float32,), kb * M), _lib.FP8_A_QUANTISED, None
 
 
+def _a_workspace_bytes(A, M, N, K, a_swiglu):
+    """Workspace bytes the A operand adds to a call's own: 0 for quantised codes, the library's answer for an operand it makes."""
+    if isinstance(A, PlanesRmsnorm):
+        return int(lib.llmmm_fp8_planes_rmsnorm_a_workspace(M, N, K))
+    return int(lib.llmmm_fp8_swiglu_a_workspace(M, N, K)) if a_swiglu else 0
+
+
 def _fp8_gemm(out_kind, A, As, Bt, Bs, C, Cs, M, N, K, workspace, tile, split_k, stream, b_preshuffled=False, a_swiglu=False):
     kb = K // 128 if K % 128 == 0 else 0
     c_dtypes = {_lib.OUT_F32: (torch.float32,), _lib.OUT_BF16: (torch.bfloat16,), _lib.OUT_FP8Q: _FP8_DTYPES, _lib.OUT_FP8Q_SWIGLU: _FP8_DTYPES}[out_kind]
@@ -236,7 +243,7 @@ def fp8_gemm_add_rmsnorm_quant(A, A_scale_transposed, B_transposed, B_scale_tran
         raise RuntimeError("T is not supported.")
     kb = K // 128 if K % 128 == 0 else 0
     if workspace is None:
-        n = int(lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K)) + (int(lib.llmmm_fp8_swiglu_a_workspace(M, N, K)) if a_swiglu else 0)
+        n = int(lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K)) + _a_workspace_bytes(A, M, N, K, a_swiglu)
         workspace = torch.empty(max(n, 16), dtype=torch.uint8, device=residual.device)
     q = torch.empty((M, N), dtype=torch.uint8, device=residual.device)
     s = torch.empty(((N + 127) // 128, M), dtype=torch.float32, device=residual.device)
@@ -259,6 +266,8 @@ def fp8_gemm_planes(A, A_scale_transposed, B_transposed, B_scale_transposed, M, 
         planes = torch.empty(max(int(lib.llmmm_fp8_gemm_planes_bytes(M, N, K)) // 4, max(split_k, 1) * M * N), dtype=torch.float32,
                              device=B_transposed.device)
     kb = K // 128 if K % 128 == 0 else 0
+    if workspace is None and _a_workspace_bytes(A, M, N, K, a_swiglu):
+        workspace = torch.empty(_a_workspace_bytes(A, M, N, K, a_swiglu), dtype=torch.uint8, device=B_transposed.device)
     a_p, as_p, a_layout, _keep = _a_operand(A, A_scale_transposed, M, K, a_swiglu)
     cfg = GemmCfg(tile, split_k, _lib.FP8_B_PRESHUFFLED if b_preshuffled else _lib.FP8_B_ROWS, a_layout)
     splits = ctypes.c_int(0)
@@ -279,7 +288,7 @@ def fp8_gemm_qkv_rope(A, A_scale_transposed, B_transposed, B_scale_transposed, q
     dev = B_transposed.device
     kb = K // 128 if K % 128 == 0 else 0
     if workspace is None:
-        n = int(lib.llmmm_fp8_gemm_qkv_rope_workspace(M, N, K))
+        n = int(lib.llmmm_fp8_gemm_qkv_rope_workspace(M, N, K)) + _a_workspace_bytes(A, M, N, K, False)
         workspace = torch.empty(max(n, 16), dtype=torch.uint8, device=dev)
     out = torch.empty((M, N), dtype=torch.uint8 if out_fp8 else torch.bfloat16, device=dev)
     sc = torch.empty(((N + 127) // 128, M), dtype=torch.float32, device=dev) if out_fp8 else None

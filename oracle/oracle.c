@@ -385,8 +385,10 @@ ORACLE_API int oracle_fp8_gemm(const uint8_t* A, const float* As, const uint8_t*
  * reciprocal != 0: Cq = e4m3(C * (448.f/amax))  (opt.cu:439-454)
  * reciprocal == 0: Cq = e4m3(C / scale)         (examples/005.fp8.mm.cu:759-769)
  * Cs[nb*M + m] = scale (opt.cu:458-461).
- * zero_guard != 0: an all-zero group gives codes 0 and scale 0 (this repository's kernels);
- * zero_guard == 0: the reference's unguarded arithmetic (0 * inf = NaN -> 0x7F).
+ * zero_guard != 0 (this repository's kernels): a group whose 448.f/amax is not finite -- all zeros, or amax below
+ *                  2^-119 so that the reciprocal overflows -- gives codes 0 next to its scale amax/448;
+ * zero_guard == 0: the reference's unguarded arithmetic (0 * inf = NaN -> 0x7F; with an overflowing reciprocal
+ *                  +-448 for every non-zero element).
  * Non-finite C: a NaN element never enters the maximum.  (In the reference a thread's chain
  * `max_val > |c| ? max_val : |c|`, opt.cu:413, keeps a NaN only when it is the last value that thread compares, and the
  * cross-lane `max()` steps behind it, opt.cu:415-416 and :432, drop it again: fmaxf semantics.  Only a group that holds
@@ -411,8 +413,8 @@ ORACLE_API void oracle_requant_c_1x128(const float* C, uint8_t* Cq, float* Cs, i
       for (int n = n0; n < n1; ++n) {
         float v = C[(size_t)m * N + n];
         float r;
-        if (zero_guard && amax == 0.0f)
-          r = v * 0.0f; /* zeros stay zeros, a NaN stays a NaN (code 0x7F) */
+        if (zero_guard && !(inv < INFINITY))
+          r = v * 0.0f; /* amax == 0, or so small that 448 / amax overflows: zeros, a NaN stays a NaN (code 0x7F) */
         else
           r = reciprocal ? v * inv : v / scale;
         Cq[(size_t)m * N + n] = oracle_e4m3_encode(r);

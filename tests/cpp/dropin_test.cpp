@@ -6,6 +6,7 @@
 #include "llmmm/base/base.h"
 #include "llmmm/mm/fp8/mm.h"
 
+#include <hip/hip_fp8.h>
 #include <hip/hip_runtime.h>
 #include <cstdio>
 #include <cstring>
@@ -286,6 +287,25 @@ int main()
       CHECK(hipMemcpy(h0.data(), dc0, h0.size(), hipMemcpyDeviceToHost)); CHECK(hipMemcpy(h1.data(), dc1, h1.size(), hipMemcpyDeviceToHost));
       if (memcmp(h0.data(), h1.data(), h0.size()) != 0) ++fw;
     }
+    // the same call from a caller that holds HIP's own OCP e4m3 type -- the natural port of the reference's __nv_fp8_e4m3*
+    // (examples/005.fp8.mm.cu:217-225, :2467-2476): the pointers go in as they are
+    {
+      static_assert(sizeof(__hip_fp8_e4m3) == 1, "one byte");
+      const __hip_fp8_e4m3* a8 = reinterpret_cast<const __hip_fp8_e4m3*>(daq);
+      const __hip_fp8_e4m3* b8 = reinterpret_cast<const __hip_fp8_e4m3*>(dbq);
+      __hip_fp8_e4m3*       c8 = reinterpret_cast<__hip_fp8_e4m3*>(dc0);
+      CHECK(hipMemsetAsync(dc0, 0x55, (size_t)m * n, st));
+      LLMMM::fp8_blockwise_symmetric_quantization<1, 128, true>(dx, reinterpret_cast<__hip_fp8_e4m3*>(daq), das, m, k, st);  // the same codes and scales again
+      LLMMM::fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(a8, das, b8, dbs, c8, dcs0, m, n, k, st);
+      CHECK(hipStreamSynchronize(st));
+      std::vector<unsigned char> h0((size_t)m * n), h1((size_t)m * n);
+      CHECK(hipMemcpy(h0.data(), dc0, h0.size(), hipMemcpyDeviceToHost));
+      if (llmmm_fp8_gemm(LLMMM_OUT_FP8Q, daq, das, dbq, dbs, dc1, dcs1, m, n, k, ws1, wsz, nullptr) != LLMMM_OK) ++fw;
+      CHECK(hipDeviceSynchronize());
+      CHECK(hipMemcpy(h1.data(), dc1, h1.size(), hipMemcpyDeviceToHost));
+      if (memcmp(h0.data(), h1.data(), h0.size()) != 0) { ++fw; printf("__hip_fp8_e4m3 pointers: FAIL\n"); }
+    }
+    LLMMM::release_fp8_workspace(st);  // before the handle goes away: a later stream with the same handle must not inherit the entry
     CHECK(hipGraphExecDestroy(exec)); CHECK(hipGraphDestroy(graph)); CHECK(hipStreamDestroy(st));
     printf("caller-supplied workspace: first call captured into a graph, too-small and withdrawn workspaces: %s\n", fw ? "FAIL" : "ok");
     fails += fw;

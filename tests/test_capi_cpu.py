@@ -10,10 +10,20 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "llmmm.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"LLMMM_API\s+[\w\s\*]+?\b(llmmm_\w+)\s*\(", text)))
+def _declared_symbols(headers=("llmmm.h", "llmmm_probe.h")):
+    names = set()
+    for h in headers:
+        text = open(os.path.join(ROOT, "include", h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names.update(re.findall(r"LLMMM_API\s+[\w\s\*]+?\b(llmmm_\w+)\s*\(", text))
+    return sorted(names)
+
+
+def test_probes_are_declared_apart_from_the_drop_in_surface():
+    """The boundary header declares no instrumentation: every llmmm_probe_* lives in llmmm_probe.h, nothing else does."""
+    assert not [n for n in _declared_symbols(("llmmm.h",)) if n.startswith("llmmm_probe_")]
+    probes = _declared_symbols(("llmmm_probe.h",))
+    assert probes and all(n.startswith("llmmm_probe_") for n in probes)
 
 
 def test_library_exports_every_declared_symbol():
@@ -23,7 +33,7 @@ def test_library_exports_every_declared_symbol():
     raw = ctypes.CDLL(_lib.LIB_PATH)
     for n in names:
         assert hasattr(raw, n), "libllmmm.so does not export " + n
-    assert sorted(_lib.SIGNATURES) == names, "llmmm_amd._lib.SIGNATURES and include/llmmm.h disagree"
+    assert sorted(_lib.SIGNATURES) == names, "llmmm_amd._lib.SIGNATURES and include/llmmm.h + llmmm_probe.h disagree"
 
 
 def test_error_strings_are_the_reference_texts():
@@ -305,7 +315,7 @@ def test_planes_and_planes_rmsnorm_validation_without_device():
     assert call(_lib.APlanesRmsnorm(**dict(good, hidden_dtype=9))) == _lib.ERR_UNSUPPORTED_TYPE
     assert call(_lib.APlanesRmsnorm(**dict(good, eps=-1.0))) == _lib.ERR_INVALID_ARGUMENT
     assert call(_lib.APlanesRmsnorm(**dict(good, residual=0x2004))) == _lib.ERR_INVALID_ARGUMENT
-    assert lib.llmmm_fp8_planes_rmsnorm_a_workspace(2, N2, K2) == 0
+    assert lib.llmmm_fp8_planes_rmsnorm_a_workspace(2, N2, K2) == 2 * N2 * 4  # the kernel generates: one fp32 plane for outputs other than fp32
     assert lib.llmmm_fp8_planes_rmsnorm_a_workspace(16, N2, K2) > 0
 
 
@@ -392,3 +402,54 @@ def test_planes_rmsnorm_descriptor_needs_no_16_byte_alignment():
     rc = lib.llmmm_fp8_gemm_qkv_rope(_lib.OUT_BF16, ctypes.c_void_p(addr), None, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, ctypes.c_float(1e-6), FAKE, FAKE, 64, FAKE,
                                      32, 8, M, N, K, FAKE, 1 << 20, ctypes.byref(cfg), None)
     assert rc == _lib.ERR_INVALID_ARGUMENT and b"splits" in lib.llmmm_last_error()
+
+
+@pytest.mark.skipif(not _no_gpu_here(), reason="passes validation with made-up pointers: only where no device can be reached")
+@pytest.mark.parametrize("N,K", [(2560, 9728), (2560, 4096), (6144, 2560), (19456, 2560), (4096, 14336)])
+@pytest.mark.parametrize("M", [1, 2, 4, 8, 16, 32, 128])
+@pytest.mark.parametrize("a_layout", [1, 2])
+def test_queried_sizes_hold_for_generated_activations(M, N, K, a_layout):
+    """A call whose activations the library makes itself (cfg.a_layout = SWIGLU_F32 or PLANES_RMSNORM) never runs in
+    column strips, so the size queries -- which cannot see cfg -- must cover the split-K form of a strip-capable shape
+    (2560 x 9728 at M <= 4 needs three planes for generated activations).  Each entry point gets exactly the queried
+    sizes and must get as far as the launch (LLMMM_ERR_RUNTIME without a device)."""
+    from llmmm_amd import _lib
+    lib = _lib.lib
+    eps = ctypes.c_float(1e-6)
+    if a_layout == _lib.FP8_A_PLANES_RMSNORM and K > 10240:
+        pytest.skip("the fused norm handles rows of at most 10240 columns")
+    a_ws = (lib.llmmm_fp8_swiglu_a_workspace if a_layout == _lib.FP8_A_SWIGLU_F32 else lib.llmmm_fp8_planes_rmsnorm_a_workspace)(M, N, K)
+    cfg = _lib.GemmCfg(_lib.TILE_AUTO, 0, 0, a_layout)
+    if a_layout == _lib.FP8_A_PLANES_RMSNORM:
+        d = _lib.APlanesRmsnorm()
+        d.planes, d.splits, d.hidden_dtype, d.residual, d.hidden_out, d.norm_weight, d.eps = 0x1000, 4, _lib.DTYPE_BF16, 0x2000, 0x3000, 0x4000, 1e-6
+        A = ctypes.cast(ctypes.pointer(d), ctypes.c_void_p)
+    else:
+        A = FAKE
+
+    def ws(n):
+        return (FAKE if n else None), n
+
+    # the plain GEMM, every output kind
+    for out in (_lib.OUT_F32, _lib.OUT_BF16, _lib.OUT_FP8Q):
+        need = lib.llmmm_fp8_gemm_workspace(out, M, N, K) + a_ws
+        rc = lib.llmmm_fp8_gemm_ex(out, A, None, FAKE, FAKE, FAKE, FAKE, M, N, K, *ws(need), ctypes.byref(cfg), None)
+        assert rc == _lib.ERR_RUNTIME, (out, lib.llmmm_last_error())
+    # planes only
+    pb = lib.llmmm_fp8_gemm_planes_bytes(M, N, K)
+    splits = ctypes.c_int(0)
+    rc = lib.llmmm_fp8_gemm_planes(A, None, FAKE, FAKE, M, N, K, FAKE, pb, ctypes.byref(splits), *ws(a_ws), ctypes.byref(cfg), None)
+    assert rc == _lib.ERR_RUNTIME, lib.llmmm_last_error()
+    # projection + residual add + RMSNorm + quantiser
+    if N <= 10240:
+        need = lib.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(M, N, K) + a_ws
+        rc = lib.llmmm_fp8_gemm_add_rmsnorm_quant(A, None, FAKE, FAKE, _lib.DTYPE_BF16, FAKE, FAKE, FAKE, eps, FAKE, FAKE, M, N, K, *ws(need),
+                                                  ctypes.byref(cfg), None)
+        assert rc == _lib.ERR_RUNTIME, lib.llmmm_last_error()
+    # QKV + per-head norm + rope
+    heads = N // 128
+    nkv = 1 if heads < 12 else 8
+    need = lib.llmmm_fp8_gemm_qkv_rope_workspace(M, N, K) + a_ws
+    rc = lib.llmmm_fp8_gemm_qkv_rope(_lib.OUT_BF16, A, None, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, eps, FAKE, FAKE, 64, FAKE, heads - 2 * nkv, nkv, M, N, K,
+                                     *ws(need), ctypes.byref(cfg), None)
+    assert rc == _lib.ERR_RUNTIME, lib.llmmm_last_error()

@@ -309,3 +309,32 @@ def test_non_finite_operands(lib, oracle, tile, split):
     assert (Cq == oq).all(), what + ": fused codes differ from requant(own fp32) at %s" % np.argwhere(Cq != oq)[:5].tolist()
     assert (Cs.view(np.uint32) == os_.view(np.uint32)).all()
     assert (Cq[3] == 0x7F).all() and (Cq[:, 200] == 0x7F).all()
+
+
+@pytest.mark.parametrize("tile,split", [("256x256", 0), ("128x128", 0), ("128x128", 2), (8, 1), (8, 2)])
+def test_groups_whose_reciprocal_scale_overflows(lib, oracle, tile, split):
+    """Rows whose results are so small (|C| <= 2^-120) that 448 / amax is not a finite fp32 number: every epilogue that
+    multiplies by the reciprocal -- the tile kernels' own, the split-K reduce kernel, the weight-streaming kernel's -- must
+    treat such a group like a group of zeros (codes 0, scale amax / 448) instead of writing NaN codes; the rows next to
+    them are quantised as usual.  Bit for bit against the oracle's re-quantisation of the kernel's own fp32 result."""
+    skinny = tile == 8
+    M, N, K = (16 if skinny else 256), 256, 256
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=91)
+    rng = np.random.default_rng(5)
+    k0 = 37
+    Bq[:, k0] = rng.choice(np.array([0x00, 0x01, 0x81, 0x02, 0x82], np.uint8), N)  # 0, +-2^-9, +-2^-8
+    Bs[:] = np.float32(2.0 ** -44)
+    for m in (0, 5):  # one non-zero activation (2^-9) with scale 2^-60: |C| in {0, 2^-122, 2^-121}
+        Aq[m] = 0
+        Aq[m, k0] = 0x01
+        As[:, m] = np.float32(2.0 ** -60)
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    assert 0 < np.abs(ref[0]).max() <= 2.0 ** -120 and np.abs(ref[1]).max() > 2.0 ** -100
+    C, Cb, Cq, Cs = _run_all(lib, Aq, As, Bq, Bs, tile=tile if skinny else TILES[tile], split_k=split)[:4]
+    what = "tile %s split %d" % (tile, split)
+    assert (C[[0, 5]] == ref[[0, 5]]).all(), what + ": one product per sum, nothing to round"
+    oq, os_ = oracle.requant_c_1x128(C)
+    assert (Cq == oq).all(), what + ": fused codes differ from requant(own fp32) at %s" % np.argwhere(Cq != oq)[:5].tolist()
+    assert (Cs.view(np.uint32) == os_.view(np.uint32)).all(), what + ": scales"
+    assert ((Cq[[0, 5]] & 0x7F) == 0).all() and (Cs[:, [0, 5]] > 0).all()
+    assert (np.abs(oracle.e4m3_decode(Cq[1])).reshape(-1, 128).max(-1) == 448).all()

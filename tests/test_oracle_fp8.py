@@ -157,3 +157,23 @@ def test_requant_zero_guard_versus_reference_nan(oracle):
     q_ref, _ = oracle.requant_c_1x128(C, zero_guard=False)
     assert (q_guard == 0).all() and (s == 0).all()
     assert (q_ref == 0x7F).all()  # the reference's unguarded 0 * inf = NaN
+
+
+def test_requant_overflowing_reciprocal(oracle):
+    """A group whose amax lies below 448 / FLT_MAX (about 2^-119): 448.f / amax is +inf.  The reference's arithmetic then
+    writes +-448 for every non-zero element and NaN for the zeros; under the guard the group's codes are 0 next to the
+    scale amax / 448 (v * 0: a negative element gives -0, code 0x80), and a group just above the limit is quantised as usual (its amax element reaches 448)."""
+    tiny = np.float32(2.0 ** -121)
+    C = np.zeros((3, 128), np.float32)
+    C[0, :4] = [tiny, -tiny / 2, 0.0, tiny / 4]
+    C[1, :3] = [np.float32(1e-36), np.float32(-5e-37), 0.0]      # also below 1.3166e-36
+    C[2, :3] = [np.float32(2.0 ** -118), np.float32(-2.0 ** -119), 0.0]  # reciprocal finite
+    with np.errstate(over="ignore", invalid="ignore", divide="ignore"):
+        q_ref, _ = oracle.requant_c_1x128(C, zero_guard=False)
+        q, s = oracle.requant_c_1x128(C, zero_guard=True)
+    assert list(q_ref[0, :4]) == [0x7E, 0xFE, 0x7F, 0x7E]
+    assert ((q[0] & 0x7F) == 0).all() and ((q[1] & 0x7F) == 0).all()  # signed zeros: v * 0
+    assert q[0, 1] == 0x80 and q[0, 0] == 0
+    assert s[0, 0] == np.float32(tiny) / np.float32(448.0) and s[0, 1] == np.float32(1e-36) / np.float32(448.0)
+    assert q[2, 0] == 0x7E and q[2, 1] == 0xF6 and q[2, 2] == 0  # 448 and -224
+    assert (q[2] == q_ref[2]).all()

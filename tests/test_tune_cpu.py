@@ -99,3 +99,31 @@ def test_entries_for_fewer_than_128_rows(tmp_path):
     # 80 rows: its own entry; 96 and 72 rows: what M = 128 hands down (the 256 x 256 entry for 72 rows cannot be a row tail);
     # 256 rows: not the 80-row entry; 90 rows of the other shape: the streaming entry, 110 rows: beyond its m_max -> tiles
     assert res.stdout.strip() == "(3, 2) (3, 1) (3, 1) (3, 1) 3 (8, 3) (3, 1)", res.stdout
+
+
+def test_bad_file_entries_are_dropped_not_obeyed(tmp_path):
+    """An entry whose tile does not divide its shape, and a line longer than the parser's buffer (whose tail looks like an
+    entry of its own), are ignored with a warning: the shapes they name are served by the built-in table or the heuristic
+    as if the file did not mention them."""
+    import torch
+    path = tmp_path / "tune.txt"
+    long_line = "tile 128 4096 4096 3 1" + " " * 280 + "skinny 16 4096 4096 9"
+    path.write_text("fp16 384 384 256 0\ntile 384 4096 4096 0 1\n" + long_line + "\nskinny 16 5120 4096 6\n")
+    prog = textwrap.dedent("""
+        import ctypes, sys
+        sys.path.insert(0, %r)
+        import llmmm_amd
+        from llmmm_amd import _lib
+        q = lambda *a: llmmm_amd.query_config(_lib.OUT_FP8Q, *a)
+        fake = ctypes.c_void_p(0x1000)
+        rc = _lib.lib.llmmm_fp16_gemm(0, fake, fake, fake, 384, 384, 256, 0, None) if not __import__("torch").cuda.is_available() else -1
+        print(q(8, 4096, 4096)[1] != 9, q(384, 4096, 4096)[0] != _lib.TILE_256x256, q(8, 5120, 4096), rc)
+    """ % ROOT)
+    res = subprocess.run([sys.executable, "-c", prog], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=dict(os.environ, LLMMM_TUNE_FILE=str(path)))
+    assert res.returncode == 0, res.stderr
+    out = res.stdout.split()
+    assert out[:2] == ["True", "True"], res.stdout
+    assert "(8, 6)" in res.stdout            # the entry behind the long line is still read
+    assert "line too long" in res.stderr and res.stderr.count("not a tune entry") == 2
+    if not torch.cuda.is_available():
+        assert out[-1] == "5", res.stdout    # the FP16 call gets as far as the launch (no device here): not "not aligned"

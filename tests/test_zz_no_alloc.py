@@ -71,3 +71,53 @@ def test_static_workspace_rejects_what_does_not_fit():
     fake = ctypes.c_void_p(0x1000)
     rc = raw.llmmm_fp8_gemm_static_ws(_lib.OUT_FP8Q, fake, fake, fake, fake, fake, fake, M, N, K, None)
     assert rc == _lib.ERR_WORKSPACE and b"built-in array" in raw.llmmm_last_error()
+
+
+def test_static_workspace_call_is_capturable_and_allocates_nothing(oracle):
+    """After one warm-up call on a shape that needs no planes at all (so the warm-up itself cannot have been what resolved
+    the array for a split-K shape), a split-K call is captured into a HIP graph: the capture must succeed (torch captures in the
+    mode in which an allocation or a synchronising runtime query on any thread fails the capture), an eager call must leave
+    the device's free memory where it was, and every replay -- with eager
+    work and synchronisations between them -- must reproduce the eager call's bits."""
+    from llmmm_amd import _lib
+    raw = _lib.lib
+    M, N, K = 16, 2560, 4096
+    assert raw.llmmm_fp8_gemm_workspace(_lib.OUT_FP8Q, M, N, K) > 0
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=21)
+    t = [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in (Aq, As, Bq, Bs)]
+    wM, wN, wK = 256, 256, 256  # one unsplit tile: no planes
+    assert raw.llmmm_fp8_gemm_workspace(_lib.OUT_FP8Q, wM, wN, wK) == 0
+    wa, was, wb, wbs = [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in fp8_inputs(oracle, wM, wN, wK, seed=22)]
+    wc = torch.empty((wM, wN), dtype=torch.uint8, device="cuda")
+    wcs = torch.empty((wN // 128, wM), dtype=torch.float32, device="cuda")
+    C = torch.full((M, N), 0x55, dtype=torch.uint8, device="cuda")
+    Cs = torch.full((N // 128, M), -1.0, dtype=torch.float32, device="cuda")
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        st = ctypes.c_void_p(side.cuda_stream)
+        assert raw.llmmm_fp8_gemm_static_ws(_lib.OUT_FP8Q, _p(wa), _p(was), _p(wb), _p(wbs), _p(wc), _p(wcs), wM, wN, wK, st) == 0  # warm-up
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            rc = raw.llmmm_fp8_gemm_static_ws(_lib.OUT_FP8Q, _p(t[0]), _p(t[1]), _p(t[2]), _p(t[3]), _p(C), _p(Cs), M, N, K,
+                                              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, raw.llmmm_last_error().decode()
+    torch.cuda.synchronize()
+    # an eager call of the same shape leaves the device's free memory where it was (hipMemGetInfo around it)
+    free0 = torch.cuda.mem_get_info()[0]
+    assert raw.llmmm_fp8_gemm_static_ws(_lib.OUT_FP8Q, _p(t[0]), _p(t[1]), _p(t[2]), _p(t[3]), _p(C), _p(Cs), M, N, K, None) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "device memory was allocated by the call"
+    # the eager result, through the caller's-workspace form
+    need = raw.llmmm_fp8_gemm_workspace(_lib.OUT_FP8Q, M, N, K)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    Ce, Cse = torch.empty_like(C), torch.empty_like(Cs)
+    assert raw.llmmm_fp8_gemm(_lib.OUT_FP8Q, _p(t[0]), _p(t[1]), _p(t[2]), _p(t[3]), _p(Ce), _p(Cse), M, N, K, _p(ws), need, None) == 0
+    torch.cuda.synchronize()
+    for rep in range(3):
+        C.fill_(0x55)
+        Cs.fill_(-1.0)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(C, Ce) and torch.equal(Cs.view(torch.int32), Cse.view(torch.int32)), "replay %d differs from the eager call" % rep
