@@ -82,3 +82,45 @@ def test_residual_add_rmsnorm_quant_on_o_and_down(lib, oracle, seed):
         assert (np.abs(h - want) <= tol).all(), what + ": hidden state"
         rq, rs = oracle.rmsnorm_quant(h, w, 1e-6)  # bit-exact on the stored hidden state
         assert np.array_equal(q.cpu().numpy(), rq) and np.array_equal(s.cpu().numpy().view(np.uint32), rs.view(np.uint32)), what
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 8, 16, 32])
+@pytest.mark.parametrize("N,K", [(2560, 9728), (2560, 4096)])
+def test_generated_activations_with_the_queried_workspaces(lib, oracle, M, N, K):
+    """The down projection on silu(gate) * up made by the library (a_swiglu) through every entry point that takes it, each
+    with exactly the buffers its size queries ask for -- the Python mirror's defaults.  These shapes run in column strips
+    with quantised activations and in the split-K form with generated ones; the queries must cover the latter."""
+    from llmmm_amd import _lib
+    rng = np.random.default_rng(100 + M + K)
+    G = (rng.standard_normal((M, 2 * K)) * 1.5).astype(np.float32)
+    W = (rng.standard_normal((N, K)) * 0.03).astype(np.float32)
+    Bq, Bs = oracle.quant_fp8(W, 128, False)
+    hq, hs = oracle.swiglu_requant(G)
+    ref = oracle.fp8_gemm(hq, hs, Bq, Bs, promote=128)
+    dG, dB, dBs = torch.from_numpy(G).cuda(), torch.from_numpy(Bq).cuda(), torch.from_numpy(Bs).cuda()
+    raw = _lib.lib
+    a_ws = int(raw.llmmm_fp8_swiglu_a_workspace(M, N, K))
+    # plain GEMM, fp32 output: llmmm_fp8_gemm_workspace + llmmm_fp8_swiglu_a_workspace bytes
+    need = int(raw.llmmm_fp8_gemm_workspace(_lib.OUT_F32, M, N, K)) + a_ws
+    ws = torch.full((max(need, 16),), 0xFF, dtype=torch.uint8, device="cuda")[:max(need, 1)] if need else None
+    C = torch.full((M, N), float("nan"), device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(dG, None, dB, dBs, C, M, N, K, workspace=ws, a_swiglu=True)
+    torch.cuda.synchronize()
+    assert_fp8_gemm_close(C.cpu().numpy(), ref, "a_swiglu fp32, M %d" % M)
+    # planes only: the defaults of the mirror are the queried sizes
+    planes, splits = lib.fp8_gemm_planes(dG, None, dB, dBs, M, N, K, a_swiglu=True)
+    torch.cuda.synchronize()
+    assert splits >= 1 and planes.numel() * 4 == int(raw.llmmm_fp8_gemm_planes_bytes(M, N, K))
+    assert_fp8_gemm_close(planes.view(-1)[:splits * M * N].view(splits, M, N).sum(0).cpu().numpy(), ref, "a_swiglu planes, M %d" % M)
+    # projection + residual add + RMSNorm + quantiser
+    res = torch.from_numpy(rng.standard_normal((M, N)).astype(np.float32)).cuda().to(torch.bfloat16)
+    w = rng.uniform(0.5, 1.5, N).astype(np.float32)
+    hidden = torch.empty_like(res)
+    q, s = lib.fp8_gemm_add_rmsnorm_quant(dG, None, dB, dBs, res, hidden, torch.from_numpy(w).cuda(), 1e-6, M, N, K, a_swiglu=True)
+    torch.cuda.synchronize()
+    h = hidden.float().cpu().numpy()
+    want = ref + res.float().cpu().numpy()
+    tol = 2e-2 * np.maximum(np.abs(ref), np.abs(ref).reshape(M, N // 128, 128).max(-1).repeat(128, axis=1) * 2.0 ** -7) + 2.0 ** -8 * np.abs(want) + 1e-6
+    assert (np.abs(h - want) <= tol).all(), "a_swiglu hidden state, M %d" % M
+    rq, rs = oracle.rmsnorm_quant(h, w, 1e-6)
+    assert np.array_equal(q.cpu().numpy(), rq) and np.array_equal(s.cpu().numpy().view(np.uint32), rs.view(np.uint32))
