@@ -40,6 +40,13 @@ LLMMM_API int    llmmm_probe_fp8_gemm_phases(const void* A, const float* As, con
 LLMMM_API int    llmmm_probe_fp16_gemm_phases(int dtype, const void* A, const void* B, void* C, int M, int N, int K, void* stamps, size_t stamps_bytes,
                                               void* stream);
 
+/* The decode-sized fused-quantisation GEMM in column strips (M <= 16 on the few-column-group projections) lets the eight
+ * workgroups of a 128-column group exchange their row maxima through device memory and wait for each other, with a bound
+ * on the wait (20 ms).  *count = waves that ever hit that bound since the library was loaded: 0 on a healthy device; a
+ * non-zero value means results of such calls are not to be trusted.  Synchronises the device.  No counterpart in the
+ * reference (its kernels never split K, README.md:22). */
+LLMMM_API int llmmm_probe_strip_exchange_timeouts(unsigned* count);
+
 #ifdef __cplusplus
 }
 #endif

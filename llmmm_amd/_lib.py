@@ -65,6 +65,7 @@ SIGNATURES = {
     "llmmm_probe_mfma": (_i, [_i, _vp, _fp, _i, _i, _vp]),
     "llmmm_probe_mfma_flops": (_c.c_double, [_i, _i, _i]),
     "llmmm_probe_hbm_read": (_i, [_vp, _sz, _fp, _i, _vp]),
+    "llmmm_probe_strip_exchange_timeouts": (_i, [_c.POINTER(_c.c_uint)]),
     "llmmm_probe_phases_bytes": (_sz, [_i, _i]),
     "llmmm_probe_fp8_gemm_phases": (_i, [_vp, _fp, _vp, _fp, _vp, _fp, _i, _i, _i, _vp, _sz, _vp]),
     "llmmm_probe_fp16_gemm_phases": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _vp, _sz, _vp]),

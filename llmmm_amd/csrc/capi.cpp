@@ -12,6 +12,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
 #include <vector>
 
 namespace {
@@ -381,6 +382,37 @@ void prefer_strip(llmmm_gemm_cfg* cfg, int M, int N, int K)
     cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
 }
 
+// The fused 1x128 output in column strips (one launch; the eight strips of a column group exchange their row maxima
+// through device memory, fp8_skinny.hip): M <= 16 and few enough column groups for the exchange area.  The hand-off
+// costs 1.4 - 1.6 us (a store and a load through memory; the same strips with bf16 output are that much faster), a
+// little less than the reduce launch it removes, so what decides is the strips' own cost: every strip reads all M
+// activation rows over all of K, and more strips than CUs run in two rounds.  Measured with pre-shuffled weights, us,
+// strips / split-K + reduce: 2560 x 4096 (160 strips) 5.4 / 6.5 (M = 1), 5.7 / 6.6 (4), 6.1 / 6.9 (8), 6.6 / 7.0 (16);
+// 2560 x 9728 8.0 / 8.4, 8.6 / 8.5, 9.1 / 9.0, 11.0 / 9.3; 6144 x 2560 (384 strips) 6.6 / 6.7, 6.8 / 6.6, 7.5 / 6.7, 8.2 / 7.0.
+bool strip_fp8q_fits(int M, int N, int K) { return strip_fits(M, N, K) && M <= 16 && N % 128 == 0 && N / 128 <= llmmm::STRIP_XCH_MAX_GROUPS; }
+void prefer_strip_fp8q(llmmm_gemm_cfg* cfg, int M, int N, int K)
+{
+  if (cfg->tile != LLMMM_TILE_SKINNY || cfg->split_k <= 1 || !strip_fp8q_fits(M, N, K)) return;
+  const bool one_round = N / 16 <= NUM_CUS;
+  if (one_round ? (long)M * K <= 65536 : M <= 1) cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
+}
+
+// The exchange area of a stream (0 .. STRIP_XCH_AREAS - 1): launches on one stream are ordered, so they may share an
+// area; every stream the library meets gets one of its own, for the life of the process, and streams beyond the number
+// of areas get -1 -- their calls keep the split-K form.  Host bookkeeping only: nothing here touches the device.
+int strip_exchange_area(void* stream)
+{
+  static std::mutex mu;
+  static void*      owner[llmmm::STRIP_XCH_AREAS];
+  static int        used = 0;
+  std::lock_guard<std::mutex> lock(mu);
+  for (int i = 0; i < used; ++i)
+    if (owner[i] == stream) return i;
+  if (used == llmmm::STRIP_XCH_AREAS) return -1;
+  owner[used] = stream;
+  return used++;
+}
+
 // The split the weight-streaming kernel runs this shape in when it is the split-K form after all (tune table, then heuristic).
 int skinny_split_for(int M, int N, int K)
 {
@@ -405,6 +437,7 @@ int choose_fp8_out(int out_kind, int M, int N, int K, llmmm_gemm_cfg* cfg)
   const int rc = choose_fp8(M, N, K, cfg);
   if (rc) return rc;
   if (out_kind == LLMMM_OUT_F32 || out_kind == LLMMM_OUT_BF16) prefer_wide_tile(cfg, M, N), prefer_strip(cfg, M, N, K);
+  if (out_kind == LLMMM_OUT_FP8Q) prefer_strip_fp8q(cfg, M, N, K);
   if (out_kind == LLMMM_OUT_FP8Q_SWIGLU) {
     if (N % 256) return fail(LLMMM_ERR_NOT_ALIGNED, "M or N or K are not aligned.");
     if (cfg->tile != LLMMM_TILE_SKINNY && cfg->split_k <= 1) {
@@ -633,10 +666,25 @@ int llmmm_fp8_gemm_ex(int out_kind, const void* A, const float* As, const void* 
     cfg.tile = LLMMM_TILE_SKINNY;
     if (!(user && user->split_k > 0)) cfg.split_k = skinny_split_for(M, N, K);
   }
+  int xarea = -1;
+  if (cfg.tile == LLMMM_TILE_STRIP && out_kind == LLMMM_OUT_FP8Q && strip_fp8q_fits(M, N, K) && (xarea = strip_exchange_area(stream)) < 0 &&
+      !(user && user->tile == LLMMM_TILE_STRIP)) {
+    // more streams than exchange areas: a strip the library picked itself gives way to the split-K form
+    cfg.tile    = LLMMM_TILE_SKINNY;
+    cfg.split_k = skinny_split_for(M, N, K);
+  }
   if (cfg.tile == LLMMM_TILE_STRIP) {
-    if (out_kind != LLMMM_OUT_F32 && out_kind != LLMMM_OUT_BF16) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel has fp32 and bf16 outputs only (a strip holds an eighth of a 1x128 group)");
-    if (!strip_fits(M, N, K)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel handles M <= %d and K >= 1024", llmmm::STRIP_MAX_M);
-    e = llmmm::fp8_strip_launch(out_kind, cfg.b_layout, A, As, Bt, Bs, C, M, N, K, (hipStream_t)stream);
+    if (out_kind == LLMMM_OUT_FP8Q) {
+      if (!strip_fp8q_fits(M, N, K))
+        return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel quantises C for M <= 16, K >= 1024 and at most %d column groups", llmmm::STRIP_XCH_MAX_GROUPS);
+      if (xarea < 0) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel's fp8 output serves %d streams per process", llmmm::STRIP_XCH_AREAS);
+      e = llmmm::fp8_strip_fp8q_launch(cfg.b_layout, A, As, Bt, Bs, C, Cs, M, N, K, xarea, (hipStream_t)stream);
+    }
+    else {
+      if (out_kind != LLMMM_OUT_F32 && out_kind != LLMMM_OUT_BF16) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel has fp32, bf16 and fp8 (1x128) outputs only");
+      if (!strip_fits(M, N, K)) return fail(LLMMM_ERR_INVALID_ARGUMENT, "the column-strip kernel handles M <= %d and K >= 1024", llmmm::STRIP_MAX_M);
+      e = llmmm::fp8_strip_launch(out_kind, cfg.b_layout, A, As, Bt, Bs, C, M, N, K, (hipStream_t)stream);
+    }
   }
   else if (cfg.tile == LLMMM_TILE_SKINNY) {
     int split = cfg.split_k;
@@ -793,6 +841,14 @@ static size_t plane_route_workspace(int M, int N, int K, bool wide_ok)
   int bm = 0, bn = 0;
   if (cfg.tile != LLMMM_TILE_SKINNY && tile_dims(cfg.tile, bm, bn) && M % bm == 0 && split == 1) return 0;  // epilogue inside the tile kernel
   return (size_t)split * M * N * sizeof(float);
+}
+
+int llmmm_probe_strip_exchange_timeouts(unsigned* count)
+{
+  if (!count) return fail(LLMMM_ERR_INVALID_ARGUMENT, "null pointer");
+  const hipError_t e = llmmm::strip_exchange_timeouts(count);
+  if (e != hipSuccess) return fail(LLMMM_ERR_RUNTIME, "reading the exchange's time-out counter: %s", hipGetErrorString(e));
+  return LLMMM_OK;
 }
 
 size_t llmmm_probe_phases_bytes(int M, int N)

@@ -552,13 +552,43 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
 // split kernel did.  A strip holds an eighth of a 1x128 quantisation group, so this form serves the outputs without
 // such groups: fp32, bf16, and hidden = T(C + residual) for the projections that end a decoder block.
 // The activations come straight from global memory (L2) into the operand registers, slice by slice (M <= 32 rows).
-enum { ST_OUT_F32 = 0, ST_OUT_BF16 = 1, ST_OUT_ADD = 2 };
+//
+// The fused 1x128 re-quantisation (ST_OUT_FP8Q, M <= 16) needs the row maximum over a whole 128-column group, i.e. over
+// the eight strips -- eight workgroups -- that share the group.  They exchange just that: every strip publishes the
+// maxima of its 16 columns (16 rows x 4 bytes) in a small exchange area in device memory and reads the other seven
+// strips' back, all with device-scope atomic stores and loads and no fence (nothing else is shared, and the values carry
+// their own "written" mark), then quantises its own columns with the group's scale.  Against the split-K form this
+// saves the second launch and the fp32 planes' round trip; it costs one store -> load hand-off through memory.
+//
+// The exchange area: g_strip_xch[area][buffer][group][strip][row], zero when the library is loaded.  A slot holds
+// (bits of the maximum) + 1 -- never 0, the maxima being non-negative floats and never NaN -- or 0 for "not written
+// in this launch".  Two buffers take turns: a launch works in the buffer that holds zeros and, first of all, every
+// strip zeroes its own 16 slots of the other buffer (which its previous launch filled), so the next launch finds
+// that one clean.  Which buffer is which, a strip reads off its own row-0 slots at kernel entry -- written by no one
+// but itself, and all strips of a group are always launched together, so they agree.  Nothing is reset from the host,
+// nothing counts arrivals, and a captured graph can be replayed at will.  Launches that share an area must not overlap:
+// the host gives every stream an area of its own (llmmm::strip_exchange_area) and keeps the split-K form for streams
+// beyond the number of areas.
+//
+// Waiting for other workgroups is safe here because workgroups are dispatched in the order of their ids and the eight
+// strips of a group have consecutive ids: whenever a strip waits, all strips with smaller ids have been dispatched, so
+// the group with the smallest id that is still incomplete can always make progress.  The wait is bounded all the same
+// (XCH_SPIN_TICKS of the 100 MHz clock): a wave that gives up counts itself in g_strip_xch_timeouts, which the host
+// can read (llmmm_probe_strip_exchange_timeouts), and finishes with whatever it has -- every wave always reaches the
+// end of the kernel.
+constexpr int                XCH_AREAS = STRIP_XCH_AREAS, XCH_GROUPS = STRIP_XCH_MAX_GROUPS;
+constexpr unsigned long long XCH_SPIN_TICKS = 2000000ull;  // 20 ms
+static __device__ unsigned   g_strip_xch[XCH_AREAS][2][XCH_GROUPS][8][16];
+static __device__ unsigned   g_strip_xch_timeouts;
+
+enum { ST_OUT_F32 = 0, ST_OUT_BF16 = 1, ST_OUT_ADD = 2, ST_OUT_FP8Q = 3 };
 
 template <int MBLK, int OUT, int D, bool TAIL, typename HT>
 __global__ void __launch_bounds__(512)
 fp8_strip_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt, const float* __restrict__ Bs,
-                 void* __restrict__ Cv, const HT* __restrict__ residual, int M, int N, int K, int bpre)
+                 void* __restrict__ Cv, const HT* __restrict__ residual, int M, int N, int K, int bpre, float* __restrict__ Cs, int xarea)
 {
+  static_assert(OUT != ST_OUT_FP8Q || MBLK == 1, "the exchange handles one 16-row block");
   constexpr int LOADS = SKINNY_LOADS_PER_SLOT_BASE + 3 * MBLK;
   static_assert((D + (TAIL ? 1 : 0)) * LOADS < 64, "vmcnt is a 6-bit counter");
   static_assert(D >= 2 && D <= 4, "ring depths in use");
@@ -613,6 +643,15 @@ fp8_strip_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, co
 #pragma unroll
   for (int mb = 0; mb < MBLK; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // ST_OUT_FP8Q: the strip's own row-0 slot of exchange buffer 0 (non-zero: the strip's last launch worked in buffer 0),
+  // requested before everything else (the oldest load in flight: it has landed whenever a ring slot has) and looked at
+  // in the epilogue
+  unsigned own_mark = 0u;
+  if constexpr (OUT == ST_OUT_FP8Q) {
+    const int grp = n0 >> 7, strip = (n0 >> 4) & 7;
+    asm volatile("global_load_dword %0, %1, off sc1" : "=v"(own_mark) : "v"(&g_strip_xch[xarea][0][grp][strip][0]) : "memory");
+  }
+
   // the tail slice first (the oldest loads in flight: landed whenever a ring slot has), then the wave's q slices through
   // its ring, D in flight (the pipeline of fp8_skinny_kernel)
   SkinnySlot<MBLK, false> tslot;
@@ -659,6 +698,47 @@ fp8_strip_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, co
 #pragma unroll
   for (int w = 1; w < 8; ++w) v += part[w][mb][lane];  // wave order: the same sum whatever the waves' timing
   const int m = mb * 16 + i, ncol = n0 + 4 * g;  // lane (g, i): row m, columns ncol .. ncol + 3
+  if constexpr (OUT == ST_OUT_FP8Q) {
+    // (wave 0 only; rows beyond M take part with whatever their sums are: their maxima are exchanged and never used)
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(own_mark)::"memory");  // long landed; ties the register to this point
+    const int grp = n0 >> 7, strip = (n0 >> 4) & 7;
+    const int cur = own_mark != 0u ? 1 : 0;  // the buffer this strip did not fill last time (both clean: buffer 0)
+    unsigned* mine_cur  = &g_strip_xch[xarea][cur][grp][strip][0];
+    unsigned* mine_prev = &g_strip_xch[xarea][cur ^ 1][grp][strip][0];
+    float     a         = fmaxf(fmaxf(fmaxf(0.f, __builtin_fabsf(v[0])), __builtin_fabsf(v[1])), fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
+    a                   = wave_xor_max(a, 16);
+    a                   = wave_xor_max(a, 32);  // the strip's maximum of row i, in all four lanes that hold the row
+    if (g == 0) {
+      __hip_atomic_store(mine_prev + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(mine_cur + i, __builtin_bit_cast(unsigned, a) + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    // lane l polls rows 2 (l % 8), 2 (l % 8) + 1 of strip l / 8: the group's 128 slots, 8 bytes per lane
+    const unsigned long long* src = (const unsigned long long*)&g_strip_xch[xarea][cur][grp][0][0] + lane;
+    unsigned long long        w;
+    const unsigned long long  t0 = __builtin_amdgcn_s_memrealtime();
+    for (;;) {
+      w = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool missing = (unsigned)w == 0u || (unsigned)(w >> 32) == 0u;
+      if (__builtin_amdgcn_ballot_w64(missing) == 0ull) break;
+      if (__builtin_amdgcn_s_memrealtime() - t0 > XCH_SPIN_TICKS) {  // (uniform: one clock reading per wave)
+        if (lane == 0) atomicAdd(&g_strip_xch_timeouts, 1u);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    float r0 = __builtin_bit_cast(float, (unsigned)w - 1u), r1 = __builtin_bit_cast(float, (unsigned)(w >> 32) - 1u);
+#pragma unroll
+    for (int step = 8; step <= 32; step <<= 1) r0 = wave_xor_max(r0, step), r1 = wave_xor_max(r1, step);  // over the eight strips
+    const float e0 = __shfl(r0, i >> 1, 64), e1 = __shfl(r1, i >> 1, 64);
+    const float amax = (i & 1) ? e1 : e0;  // the group's maximum of row i
+    const float scale = amax / 448.f;
+    const float inv   = requant_inv(amax);
+    if (m < M) {
+      *(uint32_t*)((uint8_t*)Cv + (size_t)m * N + ncol) = pack_e4m3x4_in_range(v[0] * inv, v[1] * inv, v[2] * inv, v[3] * inv);
+      if (strip == 0 && g == 0) Cs[(size_t)grp * M + m] = scale;
+    }
+    return;
+  }
   if (m >= M) return;
   if constexpr (OUT == ST_OUT_F32)
     *(f32x4*)((float*)Cv + (size_t)m * N + ncol) = v;
@@ -675,7 +755,7 @@ fp8_strip_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, co
 // wave: 8.3 us with an 8-deep ring, 6.5 us with a 2-deep one); the deeper ring on ties.
 template <int MBLK, int OUT, typename HT>
 static hipError_t launch_strip(const void* A, const float* As, const void* Bt, const float* Bs, void* C, const void* residual, int M, int N, int K, int bpre,
-                               hipStream_t stream)
+                               hipStream_t stream, float* Cs = nullptr, int xarea = 0)
 {
   const int  q = (K / 128) / 8;
   const dim3 grid(N / 16), block(512);
@@ -688,10 +768,10 @@ static hipError_t launch_strip(const void* A, const float* As, const void* Bt, c
 #define LLMMM_GO(D)                                                                                                                                         \
   if (tail)                                                                                                                                                 \
     hipLaunchKernelGGL((fp8_strip_kernel<MBLK, OUT, D, true, HT>), grid, block, 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, (const HT*)residual, \
-                       M, N, K, bpre);                                                                                                                      \
+                       M, N, K, bpre, Cs, xarea);                                                                                                           \
   else                                                                                                                                                      \
     hipLaunchKernelGGL((fp8_strip_kernel<MBLK, OUT, D, false, HT>), grid, block, 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, (const HT*)residual, \
-                       M, N, K, bpre)
+                       M, N, K, bpre, Cs, xarea)
   if (best == 4) {
     LLMMM_GO(4);
   }
@@ -717,6 +797,21 @@ hipError_t fp8_strip_launch(int out_kind, int b_layout, const void* A, const flo
     return M <= 16 ? launch_strip<1, ST_OUT_BF16, float>(A, As, Bt, Bs, C, nullptr, M, N, K, bpre, stream)
                    : launch_strip<2, ST_OUT_BF16, float>(A, As, Bt, Bs, C, nullptr, M, N, K, bpre, stream);
   return hipErrorInvalidValue;
+}
+
+// The fused 1x128 re-quantisation in column strips (M <= 16, at most STRIP_XCH_MAX_GROUPS column groups): one launch, the
+// eight strips of a group agreeing on the row maxima through exchange area `xarea` (see above the kernel).
+hipError_t fp8_strip_fp8q_launch(int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K,
+                                 int xarea, hipStream_t stream)
+{
+  if (M < 1 || M > 16 || N % 128 || N / 128 > XCH_GROUPS || K % 128 || K / 128 < 8 || xarea < 0 || xarea >= XCH_AREAS || !Cs) return hipErrorInvalidValue;
+  return launch_strip<1, ST_OUT_FP8Q, float>(A, As, Bt, Bs, C, nullptr, M, N, K, b_layout == LLMMM_FP8_B_PRESHUFFLED, stream, Cs, xarea);
+}
+
+// Waves that gave up waiting in the exchange since the library was loaded (0 on a healthy device); synchronises.
+hipError_t strip_exchange_timeouts(unsigned* out)
+{
+  return hipMemcpyFromSymbol(out, HIP_SYMBOL(g_strip_xch_timeouts), sizeof(unsigned), 0, hipMemcpyDeviceToHost);
 }
 
 template <typename HT>

@@ -179,6 +179,23 @@ def parse_file(text):
     return skinny, tile, fp16
 
 
+def merge_rows(base, additions):
+    """base and every element of additions: (skinny_rows, tile_rows, fp16_rows).  Rows are keyed by (m_max | M, N, K); a later
+    row replaces an earlier one with the same key.  Weight-streaming rows come out ordered by (N, K, m_max), as the lookup
+    (first entry with M <= m_max) needs them; the other tables keep their order, new keys behind the old ones."""
+    out = []
+    for idx in range(3):
+        rows = {}
+        for src in [base] + list(additions):
+            for r in src[idx]:
+                rows[tuple(r[:3])] = tuple(r)
+        vals = list(rows.values())
+        if idx == 0:
+            vals.sort(key=lambda r: (r[1], r[2], r[0]))
+        out.append(vals)
+    return tuple(out)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--write", action="store_true", help="rewrite csrc/tune_table.h with the results")
@@ -188,7 +205,17 @@ def main():
     ap.add_argument("--shape", action="append", metavar="N,K", help="tune this weight shape instead of the Qwen3-4B projections (repeatable)")
     ap.add_argument("--fp16-shape", action="append", metavar="M,N,K", help="tune the FP16 / BF16 GEMM's tile for this shape instead of the built-in list (repeatable)")
     ap.add_argument("--fp16-only", action="store_true", help="tune only the FP16 / BF16 shapes (the FP8 rows keep the compiled-in values)")
+    ap.add_argument("--merge-file", metavar="PATH", action="append",
+                    help="no measurement: merge the entries of this tune file (as --write-file wrote it; repeatable) into csrc/tune_table.h, "
+                         "an entry of the file replacing the table's entry for the same key")
     args = ap.parse_args()
+    if args.merge_file:
+        path = os.path.join(HERE, "csrc", "tune_table.h")
+        merged = merge_rows(parse_header(open(path).read()), [parse_file(open(f).read()) for f in args.merge_file])
+        with open(path, "w") as f:
+            f.write(render_table(*merged))
+        print("merged %s into csrc/tune_table.h -- rebuild with `python llmmm_amd/build.py`" % ", ".join(args.merge_file), file=sys.stderr)
+        return
     torch.cuda.set_device(0)
     ms = [int(x) for x in args.m.split(",")]
     shapes = QWEN3_4B

@@ -1,0 +1,135 @@
+"""The fused 1x128 re-quantisation of C from column strips (decode-sized M on the projections with few column groups):
+one launch, in which the eight workgroups of a 128-column group exchange their row maxima through device memory.
+Codes and scales must be the oracle's re-quantisation of the strip kernel's own fp32 result bit for bit -- launch after
+launch on one stream with changing inputs (a stale maximum from an earlier launch would show as a wrong scale), in
+replayed graphs, on several streams at once -- and no wave may ever have hit the bound on its wait."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_fused_close, fp8_inputs
+
+pytestmark = pytest.mark.gpu
+STRIP, SKINNY = 9, 8
+
+
+def _dev(*arrs):
+    return [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in arrs]
+
+
+def _timeouts():
+    from llmmm_amd import _lib
+    n = ctypes.c_uint(99)
+    assert _lib.lib.llmmm_probe_strip_exchange_timeouts(ctypes.byref(n)) == 0
+    return n.value
+
+
+def _fused(lib, t, M, N, K, pre=False, tile=STRIP, guard=2):
+    Cq = torch.full((M + guard, N), 0x55, dtype=torch.uint8, device="cuda")
+    Cs = torch.full((N // 128, M), -1.0, dtype=torch.float32, device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(*t, Cq[:M], Cs, M, N, K, tile=tile, b_preshuffled=pre)
+    return Cq, Cs
+
+
+def _check(oracle, lib, t, M, N, K, Cq, Cs, what, pre=False):
+    C32 = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__output_fp32(*t, C32, M, N, K, tile=STRIP, b_preshuffled=pre)
+    torch.cuda.synchronize()
+    assert (Cq[M:] == 0x55).all(), what + ": rows behind M were written"
+    oq, os_ = oracle.requant_c_1x128(C32.cpu().numpy())
+    got_q, got_s = Cq[:M].cpu().numpy(), Cs.cpu().numpy()
+    assert (got_s.view(np.uint32) == os_.view(np.uint32)).all(), what + ": scales differ from amax / 448 of the kernel's own fp32 result"
+    assert (got_q == oq).all(), what + ": codes differ from requant(own fp32) at %s" % np.argwhere(got_q != oq)[:5].tolist()
+
+
+# K / 128 from 8 (one slice per wave) over uneven shares (20, 76 slices: tail slices) to 80; one, three and 48 column groups
+@pytest.mark.parametrize("M,N,K", [(1, 2560, 4096), (16, 2560, 4096), (1, 6144, 2560), (16, 6144, 2560), (1, 2560, 9728), (8, 2560, 9728),
+                                   (5, 128, 1024), (3, 384, 10240), (16, 256, 1152)])
+@pytest.mark.parametrize("pre", [False, True])
+def test_against_oracle(lib, oracle, M, N, K, pre):
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=M + N + K)
+    t = _dev(Aq, As, Bq, Bs)
+    if pre:
+        t[2] = lib.preshuffle_weight(t[2])
+    Cq, Cs = _fused(lib, t, M, N, K, pre)
+    what = "fused strips %dx%dx%d pre %d" % (M, N, K, pre)
+    _check(oracle, lib, t, M, N, K, Cq, Cs, what, pre)
+    ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
+    rq, rs = oracle.requant_c_1x128(ref)
+    assert_fused_close(oracle, Cq[:M].cpu().numpy(), Cs.cpu().numpy(), rq, rs, what)
+    assert _timeouts() == 0
+
+
+def test_back_to_back_launches_with_changing_inputs(lib, oracle):
+    """Twelve launches on one stream with no synchronisation between them, the activations scaled differently for each
+    (so every launch has other row maxima) and two shapes taking turns (groups 0 .. 19 of the exchange area serve both):
+    every launch must deliver the scales of its own inputs."""
+    shapes = [(16, 2560, 4096), (4, 6144, 2560)]
+    cases = []
+    for j in range(12):
+        M, N, K = shapes[j % 2]
+        Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=50 + j % 2)
+        As = (As * np.float32(2.0 ** (j - 6))).astype(np.float32)
+        cases.append((M, N, K, _dev(Aq, As, Bq, Bs)))
+    outs = [_fused(lib, t, M, N, K) for M, N, K, t in cases]
+    torch.cuda.synchronize()
+    for j, ((M, N, K, t), (Cq, Cs)) in enumerate(zip(cases, outs)):
+        _check(oracle, lib, t, M, N, K, Cq, Cs, "launch %d" % j)
+    assert _timeouts() == 0
+
+
+def test_graph_replays_and_two_streams(lib, oracle):
+    """A captured launch replayed four times with the activations rewritten between the replays, eager work and
+    synchronisations in between, and a second stream (an exchange area of its own) running the same shape concurrently."""
+    M, N, K = 16, 2560, 4096
+    base = fp8_inputs(oracle, M, N, K, seed=77)
+    t = _dev(*base)
+    other = _dev(*fp8_inputs(oracle, M, N, K, seed=78))
+    Cq = torch.full((M, N), 0x55, dtype=torch.uint8, device="cuda")
+    Cs = torch.full((N // 128, M), -1.0, dtype=torch.float32, device="cuda")
+    side, side2 = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(*t, Cq, Cs, M, N, K)  # warm-up outside the capture
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(*t, Cq, Cs, M, N, K)
+    torch.cuda.synchronize()
+    for rep in range(4):
+        t[1].copy_(torch.from_numpy((base[1] * np.float32(3.0 ** rep)).astype(np.float32)))
+        Cq.fill_(0x55)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side2):
+            o_q, o_s = _fused(lib, other, M, N, K, guard=0)
+        g.replay()
+        torch.cuda.synchronize()
+        _check(oracle, lib, t, M, N, K, Cq, Cs, "replay %d" % rep)
+        _check(oracle, lib, other, M, N, K, o_q, o_s, "second stream, round %d" % rep)
+    assert _timeouts() == 0
+
+
+def test_library_choice_and_fallbacks(lib, oracle):
+    """Auto configuration takes strips for these shapes; the split-K form named explicitly still works and agrees within
+    the fused bar (other summation order); M = 17 is refused for the strips' fp8 output."""
+    from llmmm_amd import _lib
+    M, N, K = 4, 2560, 9728
+    assert lib.query_config(_lib.OUT_FP8Q, M, N, K) == (STRIP, 1)
+    assert lib.query_config(_lib.OUT_FP8Q, 16, N, K)[0] == SKINNY and lib.query_config(_lib.OUT_FP8Q, 2, 6144, 2560)[0] == SKINNY
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=5)
+    t = _dev(Aq, As, Bq, Bs)
+    Cq = torch.full((M, N), 0x55, dtype=torch.uint8, device="cuda")
+    Cs = torch.full((N // 128, M), -1.0, dtype=torch.float32, device="cuda")
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(*t, Cq, Cs, M, N, K)  # auto, no workspace needed
+    _check(oracle, lib, t, M, N, K, Cq, Cs, "auto")
+    ws = lib.make_workspace(_lib.OUT_FP8Q, M, N, K)
+    Sq, Ss = torch.empty_like(Cq), torch.empty_like(Cs)
+    lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(*t, Sq, Ss, M, N, K, tile=SKINNY, workspace=ws)
+    torch.cuda.synchronize()
+    assert_fused_close(oracle, Sq.cpu().numpy(), Ss.cpu().numpy(), Cq.cpu().numpy(), Cs.cpu().numpy(), "split-K form vs strips")
+    with pytest.raises(RuntimeError):
+        lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(*_dev(*fp8_inputs(oracle, 17, 256, 1024, seed=1)),
+                                                                             torch.empty((17, 256), dtype=torch.uint8, device="cuda"),
+                                                                             torch.empty((2, 17), dtype=torch.float32, device="cuda"), 17, 256, 1024, tile=STRIP)
+    assert _timeouts() == 0

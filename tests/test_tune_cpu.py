@@ -46,7 +46,8 @@ def test_tune_file_round_trip_and_override(tmp_path):
         import llmmm_amd
         from llmmm_amd import _lib
         q = lambda *a: llmmm_amd.query_config(_lib.OUT_FP8Q, *a)
-        print(q(8, 4096, 14336), q(100, 4096, 14336), q(2048, 4096, 14336), q(256, 2560, 4096), q(16, 2560, 4096), q(3072, 4096, 14336)[0])
+        # (M = 12 and 24: beyond the sizes that run in column strips, where the split of the weight-streaming kernel shows)
+        print(q(12, 4096, 14336), q(100, 4096, 14336), q(2048, 4096, 14336), q(256, 2560, 4096), q(24, 2560, 4096), q(3072, 4096, 14336)[0])
     """ % ROOT)
     env = dict(os.environ, LLMMM_TUNE_FILE=str(path))
     res = subprocess.run([sys.executable, "-c", prog], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=env)
@@ -107,8 +108,8 @@ def test_bad_file_entries_are_dropped_not_obeyed(tmp_path):
     as if the file did not mention them."""
     import torch
     path = tmp_path / "tune.txt"
-    long_line = "tile 128 4096 4096 3 1" + " " * 280 + "skinny 16 4096 4096 9"
-    path.write_text("fp16 384 384 256 0\ntile 384 4096 4096 0 1\n" + long_line + "\nskinny 16 5120 4096 6\n")
+    long_line = "tile 128 4096 4096 3 1" + " " * 280 + "skinny 32 4096 4096 9"
+    path.write_text("fp16 384 384 256 0\ntile 384 4096 4096 0 1\n" + long_line + "\nskinny 32 5120 4096 6\n")
     prog = textwrap.dedent("""
         import ctypes, sys
         sys.path.insert(0, %r)
@@ -117,7 +118,7 @@ def test_bad_file_entries_are_dropped_not_obeyed(tmp_path):
         q = lambda *a: llmmm_amd.query_config(_lib.OUT_FP8Q, *a)
         fake = ctypes.c_void_p(0x1000)
         rc = _lib.lib.llmmm_fp16_gemm(0, fake, fake, fake, 384, 384, 256, 0, None) if not __import__("torch").cuda.is_available() else -1
-        print(q(8, 4096, 4096)[1] != 9, q(384, 4096, 4096)[0] != _lib.TILE_256x256, q(8, 5120, 4096), rc)
+        print(q(24, 4096, 4096)[1] != 9, q(384, 4096, 4096)[0] != _lib.TILE_256x256, q(24, 5120, 4096), rc)
     """ % ROOT)
     res = subprocess.run([sys.executable, "-c", prog], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=dict(os.environ, LLMMM_TUNE_FILE=str(path)))
     assert res.returncode == 0, res.stderr
