@@ -73,7 +73,11 @@ int max_split_for(int K) { return (K / 128) < MAX_SPLIT_K ? (K / 128) : MAX_SPLI
 int heuristic_split(int M, int N, int K)
 {
   const int groups = N / 128, kb = K / 128;
-  int       s      = (240 + groups / 2) / groups;
+  // whole workgroups per CU, never more workgroups than CUs (96 column groups in three splits are 288 workgroups, a
+  // second round: 16 x 12288 x 4096 took 18.6 us so, 13.1 us in two splits), and no more than eight splits: beyond that
+  // the planes and the reduce kernel cost more than the shorter streams give (3072 x 8192 at M = 16: 9.8 us in ten, 8.5 in eight)
+  int s = NUM_CUS / groups;
+  if (s > 8) s = 8;
   if (s > kb / 2) s = kb / 2;
   const int mblk = M <= 16 ? 1 : M <= 32 ? 2 : M <= 64 ? 4 : 8;
   const int cap  = 32 / mblk;  // slices whose rows fit the staging area
@@ -378,6 +382,9 @@ bool strip_fits(int M, int N, int K) { return M >= 1 && M <= llmmm::STRIP_MAX_M 
 // 9.4 / 7.3; down 6.7 / 8.2, 7.7 / 8.9, 9.4 / 9.1, 13.7 / 9.7.
 void prefer_strip(llmmm_gemm_cfg* cfg, int M, int N, int K)
 {
+  // (more strips than CUs run in two rounds: only while the weight matrix is small -- 6144 x 2560 above; 5120 x 13824 at
+  // M = 1 takes 14.8 us in six splits + reduce and 19.5 us in 320 strips with the fused quantisation, 1.5 us less without)
+  if (N / 16 > NUM_CUS && (long)N * K > (16L << 20)) return;
   if (cfg->tile == LLMMM_TILE_SKINNY && cfg->split_k > 1 && strip_fits(M, N, K) && (M <= 8 || (M <= 16 && K <= 4096)))
     cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
 }
@@ -393,8 +400,10 @@ bool strip_fp8q_fits(int M, int N, int K) { return strip_fits(M, N, K) && M <= 1
 void prefer_strip_fp8q(llmmm_gemm_cfg* cfg, int M, int N, int K)
 {
   if (cfg->tile != LLMMM_TILE_SKINNY || cfg->split_k <= 1 || !strip_fp8q_fits(M, N, K)) return;
+  // (more strips than CUs: only the smallest such matrix at M = 1, where it ties with the split form and needs no workspace;
+  // 5120 x 13824 at M = 1: 19.5 us in 320 strips, 14.8 us in six splits)
   const bool one_round = N / 16 <= NUM_CUS;
-  if (one_round ? (long)M * K <= 65536 : M <= 1) cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
+  if (one_round ? (long)M * K <= 65536 : (M <= 1 && (long)N * K <= (16L << 20))) cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
 }
 
 // The exchange area of a stream (0 .. STRIP_XCH_AREAS - 1): launches on one stream are ordered, so they may share an

@@ -43,3 +43,37 @@ def test_tune_fp16_shape_returns_a_runnable_tile(lib, oracle):
     torch.cuda.synchronize()
     assert_fp16_close(C.cpu().numpy(), oracle.kahan_gemm(A, B), "tuned fp16 tile")
     assert tune.parse_file(tune.render_file([], [], [(M, N, K, best, 1)]))[2] == [(M, N, K, best, 1)]
+
+
+@pytest.mark.parametrize("N,K,tuned", [(4096, 14336, True), (5120, 5120, True), (8192, 8192, True),
+                                       (3072, 8192, False), (12288, 4096, False), (9216, 3072, False)])
+def test_the_library_choice_is_close_to_the_measured_best(lib, N, K, tuned):
+    """Decode-sized M on projections of model families other than the one the kernels were developed on: three shapes the
+    compiled-in table lists (a table hit) and three it has never seen (the heuristics).  The configuration the library
+    picks by itself must run within 15 % of the best of the split counts timed here, on this GPU, in the same process --
+    weights rotated over more copies than the caches hold, as the tune driver times them."""
+    from llmmm_amd import _lib, mm, tune
+    M = 16
+    tile, split = lib.query_config(_lib.OUT_FP8Q, M, N, K)
+    assert tile in (_lib.TILE_SKINNY, _lib.TILE_STRIP)
+    rows = [r for r in tune.parse_header(open(tune.os.path.join(tune.HERE, "csrc", "tune_table.h")).read())[0] if r[1:3] == (N, K)]
+    assert bool(rows) == tuned, "the test's idea of what the table lists is out of date"
+    copies = max(2, -(-(512 << 20) // (N * K)))
+    Aq, As, weights = tune._inputs(M, N, K, copies)
+    Cq = torch.empty((M, N), dtype=torch.uint8, device="cuda")
+    Cs = torch.empty((N // 128, M), dtype=torch.float32, device="cuda")
+    ws = torch.empty(16 * M * N * 4, dtype=torch.uint8, device="cuda")
+
+    def time_of(**cfg):
+        state = {"i": 0}
+
+        def step():
+            Bq, Bs = weights[state["i"] % copies]
+            state["i"] += 1
+            mm.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(Aq, As, Bq, Bs, Cq, Cs, M, N, K, workspace=ws, **cfg)
+        return min(tune._time_ms(step, 30, graph=True) for _ in range(2))
+
+    auto = time_of()
+    cands = {s: time_of(tile=_lib.TILE_SKINNY, split_k=s) for s in (1, 2, 3, 4, 5, 6, 8, 10) if s <= K // 256}
+    best = min(cands, key=cands.get)
+    assert auto <= 1.15 * cands[best], "M %d N %d K %d: the library's %s takes %.2f us, %d splits %.2f us" % (M, N, K, (tile, split), auto * 1e3, best, cands[best] * 1e3)
