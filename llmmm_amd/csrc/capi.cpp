@@ -400,10 +400,10 @@ bool strip_fp8q_fits(int M, int N, int K) { return strip_fits(M, N, K) && M <= 1
 void prefer_strip_fp8q(llmmm_gemm_cfg* cfg, int M, int N, int K)
 {
   if (cfg->tile != LLMMM_TILE_SKINNY || cfg->split_k <= 1 || !strip_fp8q_fits(M, N, K)) return;
-  // (more strips than CUs: only the smallest such matrix at M = 1, where it ties with the split form and needs no workspace;
-  // 5120 x 13824 at M = 1: 19.5 us in 320 strips, 14.8 us in six splits)
-  const bool one_round = N / 16 <= NUM_CUS;
-  if (one_round ? (long)M * K <= 65536 : (M <= 1 && (long)N * K <= (16L << 20))) cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
+  // (more strips than CUs never pay with the exchange behind them: 6144 x 2560 at M = 1 ties from pre-shuffled weights,
+  // 6.7 us either way, and loses from row-major ones, 7.0 against 6.65 us; 5120 x 13824 at M = 1: 19.5 us in 320 strips,
+  // 14.8 us in six splits)
+  if (N / 16 <= NUM_CUS && (long)M * K <= 65536) cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
 }
 
 // The exchange area of a stream (0 .. STRIP_XCH_AREAS - 1): launches on one stream are ordered, so they may share an

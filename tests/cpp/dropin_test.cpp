@@ -193,7 +193,9 @@ int main()
   // per-stream cached buffer) and must give the bits of the C API with an explicit workspace
   {
     int fd = 0;
-    const int shapes[2][3] = {{16, 2560, 4096}, {5, 2560, 9728}};  // the second needs a larger buffer: the cache grows
+    // (shapes that still split K over workgroups -- the smallest M on these projections run in column strips, one launch, no scratch;
+    // the second needs a larger buffer: the cache grows)
+    const int shapes[2][3] = {{16, 6144, 2560}, {24, 2560, 9728}};
     for (const auto& sh : shapes) {
       const int m = sh[0], n = sh[1], k = sh[2];
       llmmm_gemm_cfg qc;
@@ -231,7 +233,7 @@ int main()
   // fresh stream can be captured into a graph; replayed, it gives the bits of the eager C-API call
   {
     int fw = 0;
-    const int m = 16, n = 2560, k = 4096;
+    const int m = 16, n = 6144, k = 2560;  // splits K over workgroups: the planes live in the workspace
     std::vector<float> fx((size_t)m * k), fwt((size_t)n * k);
     for (auto& v : fx) { s = s * 1664525u + 1013904223u; v = ((s >> 8) / 16777216.0f) * 4.f - 2.f; }
     for (auto& v : fwt) { s = s * 1664525u + 1013904223u; v = ((s >> 8) / 16777216.0f) * 0.1f - 0.05f; }
