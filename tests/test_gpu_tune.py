@@ -46,7 +46,7 @@ def test_tune_fp16_shape_returns_a_runnable_tile(lib, oracle):
 
 
 @pytest.mark.parametrize("N,K,tuned", [(4096, 14336, True), (5120, 5120, True), (8192, 8192, True),
-                                       (3072, 8192, False), (12288, 4096, False), (9216, 3072, False)])
+                                       (6144, 6144, False), (12288, 4096, False), (9216, 3072, False)])
 def test_the_library_choice_is_close_to_the_measured_best(lib, N, K, tuned):
     """Decode-sized M on projections of model families other than the one the kernels were developed on: three shapes the
     compiled-in table lists (a table hit) and three it has never seen (the heuristics).  The configuration the library
