@@ -80,7 +80,7 @@ hipError_t fp8_strip_launch(int out_kind, int b_layout, const void* A, const flo
 // The fused 1x128 re-quantisation from column strips (M <= 16, N % 128 == 0, at most STRIP_XCH_MAX_GROUPS column groups): one
 // launch; the eight strips of a group exchange their row maxima through area `xarea` (0 .. STRIP_XCH_AREAS - 1) of a small
 // array in the library's device image.  Launches that use the same area must not overlap.
-constexpr int STRIP_XCH_AREAS = 8, STRIP_XCH_MAX_GROUPS = 256;
+constexpr int STRIP_XCH_AREAS = 32, STRIP_XCH_MAX_GROUPS = 256;
 hipError_t fp8_strip_fp8q_launch(int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K,
                                  int xarea, hipStream_t stream);
 hipError_t strip_exchange_timeouts(unsigned* out);  // waves that ever gave up waiting in that exchange (synchronises)

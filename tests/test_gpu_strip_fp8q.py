@@ -133,3 +133,31 @@ def test_library_choice_and_fallbacks(lib, oracle):
                                                                              torch.empty((17, 256), dtype=torch.uint8, device="cuda"),
                                                                              torch.empty((2, 17), dtype=torch.float32, device="cuda"), 17, 256, 1024, tile=STRIP)
     assert _timeouts() == 0
+
+
+def test_more_streams_than_exchange_areas(lib, oracle):
+    """Every stream the library meets gets an exchange area of its own; there are 32.  Forty streams, one call each with the
+    caller's workspace at hand: the calls beyond the areas take the split-K form (two kernels) -- every result meets the
+    fused bar, and those that ran in strips equal the first stream's bit for bit."""
+    from llmmm_amd import _lib
+    M, N, K = 8, 2560, 4096
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=123)
+    t = _dev(Aq, As, Bq, Bs)
+    ws = lib.make_workspace(_lib.OUT_FP8Q, M, N, K)
+    assert ws is not None
+    rq, rs = oracle.requant_c_1x128(oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128))
+    streams = [torch.cuda.Stream() for _ in range(40)]
+    outs = []
+    for st in streams:
+        Cq = torch.full((M, N), 0x55, dtype=torch.uint8, device="cuda")
+        Cs = torch.full((N // 128, M), -1.0, dtype=torch.float32, device="cuda")
+        with torch.cuda.stream(st):
+            lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(*t, Cq, Cs, M, N, K, workspace=ws)
+        st.synchronize()  # the calls beyond the areas share the one workspace: one after the other
+        outs.append((Cq.cpu().numpy(), Cs.cpu().numpy()))
+    same = 0
+    for q, s in outs:
+        assert_fused_close(oracle, q, s, rq, rs, "stream")
+        same += int((q == outs[0][0]).all() and (s.view(np.uint32) == outs[0][1].view(np.uint32)).all())
+    assert same >= 1  # (how many streams found an area depends on what ran in this process before)
+    assert _timeouts() == 0
