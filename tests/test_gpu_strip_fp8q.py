@@ -161,3 +161,32 @@ def test_more_streams_than_exchange_areas(lib, oracle):
         same += int((q == outs[0][0]).all() and (s.view(np.uint32) == outs[0][1].view(np.uint32)).all())
     assert same >= 1  # (how many streams found an area depends on what ran in this process before)
     assert _timeouts() == 0
+
+
+def test_non_finite_operands_and_tiny_groups(lib, oracle):
+    """NaN codes in A and B, an infinite activation scale, a row of zeros and a row whose results are so small that
+    448 / amax overflows: the exchanged maxima never become NaN (fmaxf drops it), an infinite maximum travels as it is,
+    and codes and scales are the oracle's re-quantisation of the strip kernel's own fp32 result bit for bit."""
+    M, N, K = 16, 384, 1024
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=31)
+    Aq[3, 130] = 0x7F        # row 3: NaN in every column
+    Bq[200, 300] = 0xFF      # column 200: NaN in every row
+    As[1, 9] = np.inf        # row 9, second slice
+    As[0, 13] = 1e38         # row 13: some sums overflow
+    Aq[5] = 0                # row 5: all zeros
+    k0 = 37
+    Bq[:, k0] = np.random.default_rng(2).choice(np.array([0x00, 0x01, 0x81, 0x02], np.uint8), N)
+    Bs[:] = np.float32(2.0 ** -44)
+    Aq[7] = 0
+    Aq[7, k0] = 0x01
+    As[:, 7] = np.float32(2.0 ** -60)   # row 7: |C| <= 2^-121
+    t = _dev(Aq, As, Bq, Bs)
+    Cq, Cs = _fused(lib, t, M, N, K)
+    _check(oracle, lib, t, M, N, K, Cq, Cs, "non-finite operands")
+    q, s = Cq[:M].cpu().numpy(), Cs.cpu().numpy()
+    assert (q[3] == 0x7F).all() and (q[:, 200] == 0x7F).all()
+    keep = np.arange(N) != 200  # (0 * NaN = NaN in column 200)
+    assert (q[5, keep] == 0).all() and (s[:, 5] == 0).all()
+    assert ((q[7, keep] & 0x7F) == 0).all() and (s[:, 7] > 0).all() and (s[:, 7] < 1e-38).all()
+    assert np.isinf(s[:, 9]).any()
+    assert _timeouts() == 0
