@@ -376,34 +376,39 @@ void prefer_wide_tile(llmmm_gemm_cfg* cfg, int M, int N)
 // The weight-streaming kernel in column strips (one launch, the K split inside the workgroup) takes what the split-K
 // form of that kernel would otherwise do in two launches, for the outputs it has: no 1x128 groups.
 bool strip_fits(int M, int N, int K) { return M >= 1 && M <= llmmm::STRIP_MAX_M && N % 16 == 0 && K % 128 == 0 && K / 128 >= 8; }
-// Every strip reads all M activation rows over all of K, so next to the weights a launch moves M / 16 of their bytes again
-// from L2 into the CUs, whose load path is what bounds it.  Measured against the split form (bf16 out, us, strips /
-// split + reduce): O 4.0 / 6.2 (M = 1), 4.9 / 6.5 (8), 5.6 / 6.8 (16), 7.7 / 7.3 (32); QKV 5.0 / 6.5, 5.7 / 6.6, 6.8 / 6.8,
-// 9.4 / 7.3; down 6.7 / 8.2, 7.7 / 8.9, 9.4 / 9.1, 13.7 / 9.7.
+// Where strips beat the split-K form with its second kernel (measured, pre-shuffled weights; `fused` = with the 1x128
+// quantisation, whose exchange between the strips of a column group costs 1.4 - 1.6 us, about what the reduce launch did).
+// Every strip reads all M activation rows over all of K, so the strips' cost grows with M while the split form's hardly does.
+//  * at most one 16-column strip per CU (2560 and 4096 columns): plain outputs up to M = 8, up to 16 for K <= 4096; fused
+//    while M * K <= 65536 (2560 x 4096, us, strips / split + reduce: 5.4 / 6.5 at M = 1, 6.6 / 7.0 at 16; 2560 x 9728: 8.0 / 8.4
+//    at M = 1, 9.1 / 9.0 at 8);
+//  * more, but 32-column strips fit one round and the matrix is small (llmmm::strip_fragments; 6144 x 2560, 6144 x 4096,
+//    5120 x 5120): plain outputs as above (6144 x 4096 at M = 16: 7.5 / 8.8), fused up to M = 4 (6144 x 2560: 6.2 / 6.65 at M = 1,
+//    7.0 / 6.7 at 8; 6144 x 4096: 7.2 / 8.65 and 7.8 / 8.7; 5120 x 5120: 7.9 / 8.4 and 8.7 / 8.55);
+//  * exactly two 16-column strips per CU (8192 x 8192: 13.2 / 15.1 fused at M = 1, 14.3 / 15.3 at 8, 16.5 / 15.3 at 16);
+//  * otherwise not: 5120 x 13824 at M = 1 takes 19.5 us in 320 strips, a round and a quarter, and 14.8 us in six splits.
+bool strips_pay(int M, int N, int K, bool fused)
+{
+  const long cus = NUM_CUS, s16 = N / 16;
+  const bool plain_ok = M <= 8 || (M <= 16 && K <= 4096);
+  if (s16 <= cus) return fused ? (long)M * K <= 65536 : plain_ok;
+  if (llmmm::strip_fragments(N, K) == 2) return fused ? M <= 4 : plain_ok;
+  if (s16 == 2 * cus) return fused ? M <= 8 : M <= 16;
+  return false;
+}
+// Plain outputs, one 16-column strip per CU, measured against the split form (bf16 out, us, strips / split + reduce):
+// O 4.0 / 6.2 (M = 1), 4.9 / 6.5 (8), 5.6 / 6.8 (16), 7.7 / 7.3 (32); down 6.7 / 8.2, 7.7 / 8.9, 9.4 / 9.1, 13.7 / 9.7.
 void prefer_strip(llmmm_gemm_cfg* cfg, int M, int N, int K)
 {
-  // (more strips than CUs run in two rounds: only while the weight matrix is small -- 6144 x 2560 above; 5120 x 13824 at
-  // M = 1 takes 14.8 us in six splits + reduce and 19.5 us in 320 strips with the fused quantisation, 1.5 us less without)
-  if (N / 16 > NUM_CUS && (long)N * K > (16L << 20)) return;
-  if (cfg->tile == LLMMM_TILE_SKINNY && cfg->split_k > 1 && strip_fits(M, N, K) && (M <= 8 || (M <= 16 && K <= 4096)))
-    cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
+  if (cfg->tile == LLMMM_TILE_SKINNY && cfg->split_k > 1 && strip_fits(M, N, K) && strips_pay(M, N, K, false)) cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
 }
 
-// The fused 1x128 output in column strips (one launch; the eight strips of a column group exchange their row maxima
-// through device memory, fp8_skinny.hip): M <= 16 and few enough column groups for the exchange area.  The hand-off
-// costs 1.4 - 1.6 us (a store and a load through memory; the same strips with bf16 output are that much faster), a
-// little less than the reduce launch it removes, so what decides is the strips' own cost: every strip reads all M
-// activation rows over all of K, and more strips than CUs run in two rounds.  Measured with pre-shuffled weights, us,
-// strips / split-K + reduce: 2560 x 4096 (160 strips) 5.4 / 6.5 (M = 1), 5.7 / 6.6 (4), 6.1 / 6.9 (8), 6.6 / 7.0 (16);
-// 2560 x 9728 8.0 / 8.4, 8.6 / 8.5, 9.1 / 9.0, 11.0 / 9.3; 6144 x 2560 (384 strips) 6.6 / 6.7, 6.8 / 6.6, 7.5 / 6.7, 8.2 / 7.0.
+// The fused 1x128 output in column strips (one launch; the strips of a column group exchange their row maxima through
+// device memory, fp8_skinny.hip): M <= 16 and few enough column groups for the exchange area.
 bool strip_fp8q_fits(int M, int N, int K) { return strip_fits(M, N, K) && M <= 16 && N % 128 == 0 && N / 128 <= llmmm::STRIP_XCH_MAX_GROUPS; }
 void prefer_strip_fp8q(llmmm_gemm_cfg* cfg, int M, int N, int K)
 {
-  if (cfg->tile != LLMMM_TILE_SKINNY || cfg->split_k <= 1 || !strip_fp8q_fits(M, N, K)) return;
-  // (more strips than CUs never pay with the exchange behind them: 6144 x 2560 at M = 1 ties from pre-shuffled weights,
-  // 6.7 us either way, and loses from row-major ones, 7.0 against 6.65 us; 5120 x 13824 at M = 1: 19.5 us in 320 strips,
-  // 14.8 us in six splits)
-  if (N / 16 <= NUM_CUS && (long)M * K <= 65536) cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
+  if (cfg->tile == LLMMM_TILE_SKINNY && cfg->split_k > 1 && strip_fp8q_fits(M, N, K) && strips_pay(M, N, K, true)) cfg->tile = LLMMM_TILE_STRIP, cfg->split_k = 1;
 }
 
 // The exchange area of a stream (0 .. STRIP_XCH_AREAS - 1): launches on one stream are ordered, so they may share an

@@ -552,30 +552,32 @@ fp8_skinny_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, c
 // split kernel did.  A strip holds an eighth of a 1x128 quantisation group, so this form serves the outputs without
 // such groups: fp32, bf16, and hidden = T(C + residual) for the projections that end a decoder block.
 // The activations come straight from global memory (L2) into the operand registers, slice by slice (M <= 32 rows).
+// With CF = 2 a workgroup owns two adjacent 16-column fragments (a 32-column strip): waves 2 ks and 2 ks + 1 take K range ks
+// of 4 for fragment 0 and 1 -- half the workgroups, for shapes whose 16-column strips would outnumber the CUs.
 //
 // The fused 1x128 re-quantisation (ST_OUT_FP8Q, M <= 16) needs the row maximum over a whole 128-column group, i.e. over
-// the eight strips -- eight workgroups -- that share the group.  They exchange just that: every strip publishes the
-// maxima of its 16 columns (16 rows x 4 bytes) in a small exchange area in device memory and reads the other seven
-// strips' back, all with device-scope atomic stores and loads and no fence (nothing else is shared, and the values carry
+// the eight 16-column fragments -- eight workgroups, or four of two fragments -- that share the group.  They exchange just
+// that: the wave that finishes a fragment publishes the maxima of its 16 columns (16 rows x 4 bytes) in a small exchange
+// area in device memory and reads the other seven fragments' back, all with device-scope atomic stores and loads and no fence (nothing else is shared, and the values carry
 // their own "written" mark), then quantises its own columns with the group's scale.  Against the split-K form this
 // saves the second launch and the fp32 planes' round trip; it costs one store -> load hand-off through memory.
 //
-// The exchange area: g_strip_xch[area][buffer][group][strip][row], zero when the library is loaded.  A slot holds
+// The exchange area: g_strip_xch[area][buffer][group][fragment][row], zero when the library is loaded.  A slot holds
 // (bits of the maximum) + 1 -- never 0, the maxima being non-negative floats and never NaN -- or 0 for "not written
 // in this launch".  Two buffers take turns: a launch works in the buffer that holds zeros and, first of all, every
-// strip zeroes its own 16 slots of the other buffer (which its previous launch filled), so the next launch finds
-// that one clean.  Which buffer is which, a strip reads off its own row-0 slots at kernel entry -- written by no one
-// but itself, and all strips of a group are always launched together, so they agree.  Nothing is reset from the host,
-// nothing counts arrivals, and a captured graph can be replayed at will.  Launches that share an area must not overlap:
-// the host gives every stream an area of its own (llmmm::strip_exchange_area) and keeps the split-K form for streams
-// beyond the number of areas.
+// fragment zeroes its own 16 slots of the other buffer (which its previous launch filled), so the next launch finds
+// that one clean.  Which buffer is which, a fragment's wave reads off the fragment's own row-0 slot at kernel entry --
+// written by no one but that fragment's wave, and all eight fragments of a group take part in every launch that touches
+// the group, whatever the strip width, so they agree.  Nothing is reset from the host, nothing counts arrivals, and a
+// captured graph can be replayed at will.  Launches that share an area must not overlap: the host gives every stream an
+// area of its own (llmmm::strip_exchange_area) and keeps the split-K form for streams beyond the number of areas.
 //
-// Waiting for other workgroups is safe here because workgroups are dispatched in the order of their ids and the eight
-// strips of a group have consecutive ids: whenever a strip waits, all strips with smaller ids have been dispatched, so
-// the group with the smallest id that is still incomplete can always make progress.  The wait is bounded all the same
-// (XCH_SPIN_TICKS of the 100 MHz clock): a wave that gives up counts itself in g_strip_xch_timeouts, which the host
-// can read (llmmm_probe_strip_exchange_timeouts), and finishes with whatever it has -- every wave always reaches the
-// end of the kernel.
+// Waiting for other workgroups is safe here because workgroups are dispatched in the order of their ids and the
+// workgroups of a group have consecutive ids: whenever a wave waits, all workgroups with smaller ids have been
+// dispatched, so the group with the smallest id that is still incomplete can always make progress.  The wait is bounded
+// all the same (XCH_SPIN_TICKS of the 100 MHz clock): a wave that gives up counts itself in g_strip_xch_timeouts, which
+// the host can read (llmmm_probe_strip_exchange_timeouts), and finishes with whatever it has -- every wave always
+// reaches the end of the kernel.
 constexpr int                XCH_AREAS = STRIP_XCH_AREAS, XCH_GROUPS = STRIP_XCH_MAX_GROUPS;
 constexpr unsigned long long XCH_SPIN_TICKS = 2000000ull;  // 20 ms
 static __device__ unsigned   g_strip_xch[XCH_AREAS][2][XCH_GROUPS][8][16];
@@ -583,12 +585,17 @@ static __device__ unsigned   g_strip_xch_timeouts;
 
 enum { ST_OUT_F32 = 0, ST_OUT_BF16 = 1, ST_OUT_ADD = 2, ST_OUT_FP8Q = 3 };
 
-template <int MBLK, int OUT, int D, bool TAIL, typename HT>
+// CF = 16-column fragments of a strip (1 or 2): with CF = 2 a workgroup owns 32 columns -- wave w takes fragment w % 2 and
+// the K range (w / 2) of four -- so that N / 32 workgroups cover outputs whose N / 16 strips would be more than the CUs
+// (a second round of workgroups costs more than the narrower K split: 6144 columns are 384 strips or 192 wide ones).
+template <int MBLK, int OUT, int D, bool TAIL, typename HT, int CF = 1>
 __global__ void __launch_bounds__(512)
 fp8_strip_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, const uint8_t* __restrict__ Bt, const float* __restrict__ Bs,
                  void* __restrict__ Cv, const HT* __restrict__ residual, int M, int N, int K, int bpre, float* __restrict__ Cs, int xarea)
 {
   static_assert(OUT != ST_OUT_FP8Q || MBLK == 1, "the exchange handles one 16-row block");
+  static_assert(CF == 1 || CF == 2, "16 or 32 columns per workgroup");
+  constexpr int KS = 8 / CF;  // K ranges per column fragment
   constexpr int LOADS = SKINNY_LOADS_PER_SLOT_BASE + 3 * MBLK;
   static_assert((D + (TAIL ? 1 : 0)) * LOADS < 64, "vmcnt is a 6-bit counter");
   static_assert(D >= 2 && D <= 4, "ring depths in use");
@@ -604,14 +611,16 @@ fp8_strip_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, co
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int g    = lane >> 4;
   const int i    = lane & 15;
-  const int n0   = blockIdx.x * 16;
+  const int cf   = wave % CF;            // the wave's column fragment
+  const int ks   = wave / CF;            // ... and its K range
+  const int n0   = blockIdx.x * 16 * CF + 16 * cf;  // the wave's first column
   const int KB   = K >> 7;
-  // K is dealt in whole slices: every wave takes q = KB / 8 consecutive slices through its ring (q >= 1: the host checks
-  // KB >= 8), and the KB % 8 slices behind them go one each to the first waves as a "tail" slice, requested before
-  // anything else and consumed last -- so the ring never runs over slices that are not the wave's own.  TAIL = (KB % 8 != 0).
-  const int q    = KB >> 3;
-  const int kb0  = wave * q, kb1 = kb0 + q;
-  const int kbt  = 8 * q + wave;        // the wave's tail slice ...
+  // K is dealt in whole slices: every wave takes q = KB / KS consecutive slices through its ring (q >= 1: the host checks
+  // KB >= 8), and the KB % KS slices behind them go one each to the first K ranges as a "tail" slice, requested before
+  // anything else and consumed last -- so the ring never runs over slices that are not the wave's own.  TAIL = (KB % KS != 0).
+  const int q    = KB / KS;
+  const int kb0  = ks * q, kb1 = kb0 + q;
+  const int kbt  = KS * q + ks;          // the wave's tail slice ...
   const bool has_tail = kbt < KB;        // ... if there is one (otherwise the last slice is fetched in its place and not used)
 
   char LLMMM_LDS* const ring[4] = {(char LLMMM_LDS*)ring0 + wave * 2048, (char LLMMM_LDS*)ring1 + wave * 2048,
@@ -648,8 +657,8 @@ fp8_strip_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, co
   // in the epilogue
   unsigned own_mark = 0u;
   if constexpr (OUT == ST_OUT_FP8Q) {
-    const int grp = n0 >> 7, strip = (n0 >> 4) & 7;
-    asm volatile("global_load_dword %0, %1, off sc1" : "=v"(own_mark) : "v"(&g_strip_xch[xarea][0][grp][strip][0]) : "memory");
+    const int frag = blockIdx.x * CF + cf;  // the 16-column fragment whose epilogue this wave may run: slot frag % 8 of group frag / 8
+    asm volatile("global_load_dword %0, %1, off sc1" : "=v"(own_mark) : "v"(&g_strip_xch[xarea][0][frag >> 3][frag & 7][0]) : "memory");
   }
 
   // the tail slice first (the oldest loads in flight: landed whenever a ring slot has), then the wave's q slices through
@@ -692,27 +701,29 @@ fp8_strip_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, co
 #pragma unroll
   for (int mb = 0; mb < MBLK; ++mb) part[wave][mb][lane] = acc[mb];
   __syncthreads();
-  if (wave >= MBLK) return;  // wave mb finishes the 16-row block mb
-  const int mb = wave;
-  f32x4     v  = part[0][mb][lane];
+  if (wave >= MBLK * CF) return;  // wave mb * CF + c finishes column fragment c of the 16-row block mb
+  const int mb = wave / CF;       // (wave % CF = cf: the fragment whose K ranges this wave summed one of)
+  f32x4     v  = part[cf][mb][lane];
 #pragma unroll
-  for (int w = 1; w < 8; ++w) v += part[w][mb][lane];  // wave order: the same sum whatever the waves' timing
+  for (int w = 1; w < KS; ++w) v += part[w * CF + cf][mb][lane];  // K ranges in order: the same sum whatever the waves' timing
   const int m = mb * 16 + i, ncol = n0 + 4 * g;  // lane (g, i): row m, columns ncol .. ncol + 3
   if constexpr (OUT == ST_OUT_FP8Q) {
-    // (wave 0 only; rows beyond M take part with whatever their sums are: their maxima are exchanged and never used)
+    // (waves 0 .. CF-1 only, each on its own 16-column fragment exactly as a 16-column strip would be -- strips of either
+    // width leave an area in the same state; rows beyond M take part with whatever their sums are: their maxima are
+    // exchanged and never used)
+    float a = fmaxf(fmaxf(fmaxf(0.f, __builtin_fabsf(v[0])), __builtin_fabsf(v[1])), fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
+    a       = wave_xor_max(a, 16);
+    a       = wave_xor_max(a, 32);  // the fragment's maximum of row i, in all four lanes that hold the row
+    const int frag = blockIdx.x * CF + cf, grp = frag >> 3, strip = frag & 7;
     asm volatile("s_waitcnt vmcnt(0)" : "+v"(own_mark)::"memory");  // long landed; ties the register to this point
-    const int grp = n0 >> 7, strip = (n0 >> 4) & 7;
-    const int cur = own_mark != 0u ? 1 : 0;  // the buffer this strip did not fill last time (both clean: buffer 0)
+    const int cur = own_mark != 0u ? 1 : 0;  // the buffer this fragment did not fill last time (both clean: buffer 0)
     unsigned* mine_cur  = &g_strip_xch[xarea][cur][grp][strip][0];
     unsigned* mine_prev = &g_strip_xch[xarea][cur ^ 1][grp][strip][0];
-    float     a         = fmaxf(fmaxf(fmaxf(0.f, __builtin_fabsf(v[0])), __builtin_fabsf(v[1])), fmaxf(__builtin_fabsf(v[2]), __builtin_fabsf(v[3])));
-    a                   = wave_xor_max(a, 16);
-    a                   = wave_xor_max(a, 32);  // the strip's maximum of row i, in all four lanes that hold the row
     if (g == 0) {
       __hip_atomic_store(mine_prev + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(mine_cur + i, __builtin_bit_cast(unsigned, a) + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    // lane l polls rows 2 (l % 8), 2 (l % 8) + 1 of strip l / 8: the group's 128 slots, 8 bytes per lane
+    // lane l polls rows 2 (l % 8), 2 (l % 8) + 1 of fragment l / 8: the group's 128 slots, 8 bytes per lane
     const unsigned long long* src = (const unsigned long long*)&g_strip_xch[xarea][cur][grp][0][0] + lane;
     unsigned long long        w;
     const unsigned long long  t0 = __builtin_amdgcn_s_memrealtime();
@@ -728,7 +739,7 @@ fp8_strip_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, co
     }
     float r0 = __builtin_bit_cast(float, (unsigned)w - 1u), r1 = __builtin_bit_cast(float, (unsigned)(w >> 32) - 1u);
 #pragma unroll
-    for (int step = 8; step <= 32; step <<= 1) r0 = wave_xor_max(r0, step), r1 = wave_xor_max(r1, step);  // over the eight strips
+    for (int step = 8; step <= 32; step <<= 1) r0 = wave_xor_max(r0, step), r1 = wave_xor_max(r1, step);  // over the group's fragments
     const float e0 = __shfl(r0, i >> 1, 64), e1 = __shfl(r1, i >> 1, 64);
     const float amax = (i & 1) ? e1 : e0;  // the group's maximum of row i
     const float scale = amax / 448.f;
@@ -750,27 +761,36 @@ fp8_strip_kernel(const uint8_t* __restrict__ A, const float* __restrict__ As, co
   }
 }
 
-// Ring depth: of 4, 3 and 2 the one that runs over the fewest slices beyond the q = K / 128 / 8 of a wave (a pass past
+// Ring depth: of 4, 3 and 2 the one that runs over the fewest slices beyond the q slices of a wave (a pass past
 // the end re-fetches the last slice: wasted loads cost more here than a shallow ring -- down at M = 1, 9 slices per
 // wave: 8.3 us with an 8-deep ring, 6.5 us with a 2-deep one); the deeper ring on ties.
-template <int MBLK, int OUT, typename HT>
-static hipError_t launch_strip(const void* A, const float* As, const void* Bt, const float* Bs, void* C, const void* residual, int M, int N, int K, int bpre,
-                               hipStream_t stream, float* Cs = nullptr, int xarea = 0)
+// Strip width: 16 columns; 32 when 16-column strips would be more than the CUs, 32-column ones are not, and the weight
+// matrix is small enough that a launch is short (measured, bf16 output at M = 1, us, 16 / 32 columns: 6144 x 2560 5.0 / 4.9,
+// 6144 x 4096 6.2 / 5.9, 5120 x 5120 7.5 / 6.6 -- but 8192 x 8192, 67 MB, 11.8 / 13.3: 512 narrow strips sit two to a
+// CU and pull more between them than one wide strip does).
+int strip_fragments(int N, int K)
 {
-  const int  q = (K / 128) / 8;
-  const dim3 grid(N / 16), block(512);
+  return (N / 16 > num_cus() && N % 32 == 0 && N / 32 <= num_cus() && (long)N * K <= (32L << 20)) ? 2 : 1;
+}
+template <int MBLK, int OUT, typename HT, int CF>
+static hipError_t launch_strip_cf(const void* A, const float* As, const void* Bt, const float* Bs, void* C, const void* residual, int M, int N, int K, int bpre,
+                                  hipStream_t stream, float* Cs, int xarea)
+{
+  constexpr int KS = 8 / CF;
+  const int  q = (K / 128) / KS;
+  const dim3 grid(N / (16 * CF)), block(512);
   int        best = 2, waste = 1 << 30;
   for (int d = 4; d >= 2; --d) {
     const int w = (q + d - 1) / d * d - q;
     if (w < waste) best = d, waste = w;
   }
-  const bool tail = (K / 128) % 8 != 0;
+  const bool tail = (K / 128) % KS != 0;
 #define LLMMM_GO(D)                                                                                                                                         \
   if (tail)                                                                                                                                                 \
-    hipLaunchKernelGGL((fp8_strip_kernel<MBLK, OUT, D, true, HT>), grid, block, 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, (const HT*)residual, \
+    hipLaunchKernelGGL((fp8_strip_kernel<MBLK, OUT, D, true, HT, CF>), grid, block, 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, (const HT*)residual, \
                        M, N, K, bpre, Cs, xarea);                                                                                                           \
   else                                                                                                                                                      \
-    hipLaunchKernelGGL((fp8_strip_kernel<MBLK, OUT, D, false, HT>), grid, block, 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, (const HT*)residual, \
+    hipLaunchKernelGGL((fp8_strip_kernel<MBLK, OUT, D, false, HT, CF>), grid, block, 0, stream, (const uint8_t*)A, As, (const uint8_t*)Bt, Bs, C, (const HT*)residual, \
                        M, N, K, bpre, Cs, xarea)
   if (best == 4) {
     LLMMM_GO(4);
@@ -783,6 +803,13 @@ static hipError_t launch_strip(const void* A, const float* As, const void* Bt, c
   }
 #undef LLMMM_GO
   return hipGetLastError();
+}
+template <int MBLK, int OUT, typename HT>
+static hipError_t launch_strip(const void* A, const float* As, const void* Bt, const float* Bs, void* C, const void* residual, int M, int N, int K, int bpre,
+                               hipStream_t stream, float* Cs = nullptr, int xarea = 0)
+{
+  return strip_fragments(N, K) == 2 ? launch_strip_cf<MBLK, OUT, HT, 2>(A, As, Bt, Bs, C, residual, M, N, K, bpre, stream, Cs, xarea)
+                                 : launch_strip_cf<MBLK, OUT, HT, 1>(A, As, Bt, Bs, C, residual, M, N, K, bpre, stream, Cs, xarea);
 }
 
 hipError_t fp8_strip_launch(int out_kind, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C, int M, int N, int K,
@@ -800,7 +827,7 @@ hipError_t fp8_strip_launch(int out_kind, int b_layout, const void* A, const flo
 }
 
 // The fused 1x128 re-quantisation in column strips (M <= 16, at most STRIP_XCH_MAX_GROUPS column groups): one launch, the
-// eight strips of a group agreeing on the row maxima through exchange area `xarea` (see above the kernel).
+// fragments of a group agreeing on the row maxima through exchange area `xarea` (see above the kernel).
 hipError_t fp8_strip_fp8q_launch(int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C, float* Cs, int M, int N, int K,
                                  int xarea, hipStream_t stream)
 {

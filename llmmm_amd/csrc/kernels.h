@@ -75,6 +75,7 @@ hipError_t fp8_skinny_launch(int out_kind, int b_layout, const void* A, const fl
 // K % 128 == 0, K >= 1024; out_kind LLMMM_OUT_F32 or LLMMM_OUT_BF16 (no 1x128-grouped outputs: a strip holds an eighth
 // of a group).  hipErrorInvalidValue outside these limits.
 constexpr int STRIP_MAX_M = 32;
+int strip_fragments(int N, int K);  // 16-column fragments per strip the launchers below will use for this shape: 1 or 2
 hipError_t fp8_strip_launch(int out_kind, int b_layout, const void* A, const float* As, const void* Bt, const float* Bs, void* C, int M, int N, int K,
                             hipStream_t stream);
 // The fused 1x128 re-quantisation from column strips (M <= 16, N % 128 == 0, at most STRIP_XCH_MAX_GROUPS column groups): one

@@ -1,5 +1,6 @@
-"""The weight-streaming kernel in column strips (LLMMM_TILE_STRIP): a workgroup owns 16 columns over all of K, its eight
-waves split K and add their partial sums in wave order -- one launch, no workspace.  Against the oracle at the GEMM bar;
+"""The weight-streaming kernel in column strips (LLMMM_TILE_STRIP): a workgroup owns 16 columns over all of K (32 where 16-column
+strips would be more than the CUs and the weight matrix is small), its waves split K and add their partial sums in wave
+order -- one launch, no workspace.  Against the oracle at the GEMM bar;
 bit-identical run to run; bf16 == RNE(fp32); pre-shuffled weights give the same bits; rows behind M are never written."""
 import ctypes
 
@@ -28,7 +29,9 @@ def _run(lib, Aq, As, Bq, Bs, M, N, K, pre=False, tile=STRIP, guard=3):
 
 # K / 128 from 8 (one slice per wave) over uneven shares (20 slices: 2 or 3 per wave; 76: 9 or 10) to 8 per wave and more
 @pytest.mark.parametrize("M,N,K", [(1, 2560, 4096), (16, 2560, 9728), (16, 6144, 2560), (5, 256, 1024), (32, 2560, 4096), (17, 128, 1152),
-                                   (1, 128, 8192), (9, 512, 10240), (31, 384, 2560)])
+                                   (1, 128, 8192), (9, 512, 10240), (31, 384, 2560),
+                                   # 32-column strips: 6144 x 2560 above; four waves per fragment with a tail slice, two row blocks, exactly 256 strips
+                                   (3, 4608, 1152), (24, 4608, 1152), (1, 8192, 1024), (16, 6144, 4096)])
 def test_against_oracle(lib, oracle, M, N, K):
     Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=M + N + K)
     ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)
@@ -61,19 +64,30 @@ def test_single_nonzero_slice_is_exact(lib, oracle):
     assert np.abs(C.cpu().numpy() - ref).max() <= 1e-4 * np.abs(ref).max()
 
 
+def _strips_pay(m, n, k, fused):
+    """The library's rule, restated: strips where measured faster than split-K + reduce (256 CUs)."""
+    plain = m <= 8 or (m <= 16 and k <= 4096)
+    if n // 16 <= 256:
+        return m * k <= 65536 and m <= 16 if fused else plain
+    if n % 32 == 0 and n // 32 <= 256 and n * k <= 32 << 20:   # 32-column strips
+        return m <= 4 if fused else plain
+    if n // 16 == 512:                                          # two 16-column strips on every CU
+        return m <= 8 if fused else m <= 16
+    return False
+
+
 def test_the_library_picks_strips_where_it_used_to_split(lib):
     from llmmm_amd import _lib
     for n, k in ((2560, 4096), (2560, 9728), (6144, 2560)):
-        for m in (1, 8, 16, 32):
-            want = (STRIP, 1) if m <= 8 or (m <= 16 and k <= 4096) else None  # every strip re-reads the activations: small M only
+        for m in (1, 4, 8, 16, 32):
+            want = (STRIP, 1) if _strips_pay(m, n, k, False) else None  # every strip re-reads the activations: small M only
             for kind in (_lib.OUT_BF16, _lib.OUT_F32):
                 got = lib.query_config(kind, m, n, k)
                 assert got == want if want else got[0] == SKINNY and got[1] > 1
-            # the 1x128-grouped output takes strips on the same shapes (M <= 16: the strips of a column group exchange their row
-            # maxima); what the split-K form would run in is what the size queries answer for
+            # the 1x128-grouped output takes strips too (M <= 16: the strips of a column group exchange their row maxima; the
+            # exchange costs about what the reduce launch did); what the split-K form would run in is what the size queries answer for
             got8 = lib.query_config(_lib.OUT_FP8Q, m, n, k)
-            want8 = m <= 16 and n // 16 <= 256 and m * k <= 65536  # one round of strips; the exchange costs about what the reduce launch did
-            assert got8 == (STRIP, 1) if want8 else got8[0] == SKINNY and got8[1] > 1
+            assert got8 == (STRIP, 1) if _strips_pay(m, n, k, True) else got8[0] == SKINNY and got8[1] > 1
             split8 = lib.workspace_bytes(_lib.OUT_FP8Q, m, n, k) // (m * n * 4)
             assert split8 > 1
             # the size queries cannot see a call's cfg: they answer for the split-K form, which a strip shape falls back to
@@ -86,6 +100,12 @@ def test_the_library_picks_strips_where_it_used_to_split(lib):
                 assert raw.llmmm_fp8_gemm_add_rmsnorm_quant_workspace(m, n, k) == planes
             assert raw.llmmm_fp8_gemm_qkv_rope_workspace(m, n, k) > 0
     assert lib.query_config(_lib.OUT_BF16, 1, 19456, 2560) == (SKINNY, 1)   # enough column groups: no split to replace
+    # other model families: wide strips on small matrices, paired narrow ones at 8192 columns, none for a round and a quarter
+    for n, k in ((6144, 4096), (5120, 5120), (8192, 8192), (5120, 13824)):
+        for m in (1, 4, 8, 16):
+            for kind, fused in ((_lib.OUT_BF16, False), (_lib.OUT_FP8Q, True)):
+                got = lib.query_config(kind, m, n, k)
+                assert got == (STRIP, 1) if _strips_pay(m, n, k, fused) else got[0] == SKINNY and got[1] > 1, (m, n, k, fused, got)
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 2560, 4096), (8, 2560, 9728), (16, 2560, 4096)])

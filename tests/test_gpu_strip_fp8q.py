@@ -1,5 +1,6 @@
 """The fused 1x128 re-quantisation of C from column strips (decode-sized M on the projections with few column groups):
-one launch, in which the eight workgroups of a 128-column group exchange their row maxima through device memory.
+one launch, in which the workgroups of a 128-column group (eight 16-column strips, or four 32-column ones) exchange their
+row maxima through device memory.
 Codes and scales must be the oracle's re-quantisation of the strip kernel's own fp32 result bit for bit -- launch after
 launch on one stream with changing inputs (a stale maximum from an earlier launch would show as a wrong scale), in
 replayed graphs, on several streams at once -- and no wave may ever have hit the bound on its wait."""
@@ -46,7 +47,9 @@ def _check(oracle, lib, t, M, N, K, Cq, Cs, what, pre=False):
 
 # K / 128 from 8 (one slice per wave) over uneven shares (20, 76 slices: tail slices) to 80; one, three and 48 column groups
 @pytest.mark.parametrize("M,N,K", [(1, 2560, 4096), (16, 2560, 4096), (1, 6144, 2560), (16, 6144, 2560), (1, 2560, 9728), (8, 2560, 9728),
-                                   (5, 128, 1024), (3, 384, 10240), (16, 256, 1152)])
+                                   (5, 128, 1024), (3, 384, 10240), (16, 256, 1152),
+                                   # 32-column strips (6144 x 2560 above): tail slices, exactly 256 strips, a larger K
+                                   (3, 4608, 1152), (16, 4608, 1152), (2, 8192, 1024), (16, 6144, 4096)])
 @pytest.mark.parametrize("pre", [False, True])
 def test_against_oracle(lib, oracle, M, N, K, pre):
     Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=M + N + K)
@@ -64,8 +67,9 @@ def test_against_oracle(lib, oracle, M, N, K, pre):
 
 def test_back_to_back_launches_with_changing_inputs(lib, oracle):
     """Twelve launches on one stream with no synchronisation between them, the activations scaled differently for each
-    (so every launch has other row maxima) and two shapes taking turns (groups 0 .. 19 of the exchange area serve both):
-    every launch must deliver the scales of its own inputs."""
+    (so every launch has other row maxima) and two shapes taking turns -- one in 16-column strips, the other in 32-column
+    ones, groups 0 .. 19 of the exchange area serving both, so a width that left a group's slots in a state the other
+    cannot read would show: every launch must deliver the scales of its own inputs."""
     shapes = [(16, 2560, 4096), (4, 6144, 2560)]
     cases = []
     for j in range(12):
@@ -116,7 +120,7 @@ def test_library_choice_and_fallbacks(lib, oracle):
     from llmmm_amd import _lib
     M, N, K = 4, 2560, 9728
     assert lib.query_config(_lib.OUT_FP8Q, M, N, K) == (STRIP, 1)
-    assert lib.query_config(_lib.OUT_FP8Q, 16, N, K)[0] == SKINNY and lib.query_config(_lib.OUT_FP8Q, 2, 6144, 2560)[0] == SKINNY
+    assert lib.query_config(_lib.OUT_FP8Q, 16, N, K)[0] == SKINNY and lib.query_config(_lib.OUT_FP8Q, 8, 6144, 2560)[0] == SKINNY
     Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=5)
     t = _dev(Aq, As, Bq, Bs)
     Cq = torch.full((M, N), 0x55, dtype=torch.uint8, device="cuda")
