@@ -194,3 +194,33 @@ def test_non_finite_operands_and_tiny_groups(lib, oracle):
     assert ((q[7, keep] & 0x7F) == 0).all() and (s[:, 7] > 0).all() and (s[:, 7] < 1e-38).all()
     assert np.isinf(s[:, 9]).any()
     assert _timeouts() == 0
+
+
+def test_beside_a_kernel_that_fills_the_chip(lib, oracle):
+    """The strips of a group wait for each other, so they rely on all of them being dispatched.  While another stream runs
+    256 x 256-tile GEMMs -- one workgroup per CU, whose LDS leaves no room for a strip beside it -- the strips get CUs only as
+    GEMM workgroups end, a few at a time: every launch must still deliver the bits of an undisturbed one, and no wait may
+    have run into its bound."""
+    M, N, K = 16, 2560, 4096
+    Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=9)
+    t = _dev(Aq, As, Bq, Bs)
+    ref_q, ref_s = _fused(lib, t, M, N, K, guard=0)
+    torch.cuda.synchronize()
+    A = torch.randn(4096, 4096, device="cuda", dtype=torch.float16)
+    B = torch.randn(4096, 4096, device="cuda", dtype=torch.float16)
+    C = torch.empty_like(A)
+    big, small = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = [_fused(lib, t, M, N, K, guard=0) for _ in range(40)]  # buffers made (and filled once) ahead of the contended run
+    for q, s in outs:
+        q.fill_(0x55), s.fill_(-1.0)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(big):
+        for _ in range(30):
+            lib.fp16_mm(A, B, C, 4096, 4096, 4096)
+    with torch.cuda.stream(small):
+        for q, s in outs:
+            lib.fp8_gemm_blockwise_quant_A_1x128__B_128x128__C_1x128__output_fp8(*t, q, s, M, N, K, tile=STRIP)
+    torch.cuda.synchronize()
+    for q, s in outs:
+        assert torch.equal(q, ref_q) and torch.equal(s.view(torch.int32), ref_s.view(torch.int32))
+    assert _timeouts() == 0
