@@ -112,7 +112,16 @@ int heuristic_tile(int M, int N)
       const long tm = M / 256, tn = N / 256, full = tiles / NUM_CUS * NUM_CUS;
       if (tiles > NUM_CUS && tm > 1 && full % tm == 0 && tn - full / tm > 0 && (tn - full / tm) * tm * 2 <= NUM_CUS) waves -= 0.5f;
     }
-    const float cost  = waves * c.per_cu * c.bm * c.bn / c.eff;
+    // More 128 x 128 tiles than CUs put two on some CUs, and on weights that come from HBM -- as a layer's weights do in a
+    // model -- that costs 6-32 % against half as many 256 x 128 tiles, one per CU, whose tile rows re-read the weights half
+    // as often (us, weights rotated over more copies than the caches hold / one copy; 128 x 128 | 256 x 128 | 128 x 256:
+    // 2048 x 2560 x 9728 85.3 / 64.0 | 64.5 / 62.6 | 66.4 / 62.2; 1024 x 6144 x 2560 27.9 / 21.3 | 22.4 / 21.6 | 23.6 / 21.4;
+    // 512 x 10240 x 8192 73.0 / 55.0 | 57.9 / 53.3 | 59.7 / 53.0; 256 x 19456 x 2560 29.1 / 20.5 | 25.8 / 24.0 | 26.0 / 20.9).
+    // Up to one tile per CU the small tile stays ahead (1024 x 4096 x 4096: 26.8 | 31.7 | 30.6 cold).
+    float eff = c.eff;
+    if (c.id == LLMMM_TILE_128x128 && tiles > NUM_CUS) eff = 0.74f;
+    if (c.id == LLMMM_TILE_256x128 && M >= 512) eff = 0.86f;  // (a single tile row of 256 prefers 128 x 256 on cached weights)
+    const float cost  = waves * c.per_cu * c.bm * c.bn / eff;
     if (best < 0 || cost < best_cost) {
       best      = c.id;
       best_cost = cost;
@@ -368,7 +377,9 @@ constexpr size_t SWIGLU_PLANE_LIMIT = 16u << 20;
 // the second a quarter full) against 256 (one).  Measured on O / down at M = 2048: 30.0 -> 26.9 us, 64.0 -> 55.8 us.
 void prefer_wide_tile(llmmm_gemm_cfg* cfg, int M, int N)
 {
-  if (cfg->tile != LLMMM_TILE_128x128 || cfg->split_k > 1 || N % 640 || M % 128) return;
+  // (or 256 x 128 tiles, which the table and the heuristic name where 128 x 128 ones would sit two to a CU: one 128 x 160 tile
+  // per CU is as fast on weights from HBM and faster on cached ones -- 1024 x 5120 x 2560, us: 19.8 / 19.0 against 21.3 / 20.9)
+  if ((cfg->tile != LLMMM_TILE_128x128 && cfg->tile != LLMMM_TILE_256x128) || cfg->split_k > 1 || N % 640 || M % 128) return;
   const long t128 = (long)(M / 128) * (N / 128), t160 = (long)(M / 128) * (N / 160);
   if ((t160 + NUM_CUS - 1) / NUM_CUS < (t128 + NUM_CUS - 1) / NUM_CUS) cfg->tile = LLMMM_TILE_128x160;
 }

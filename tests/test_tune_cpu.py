@@ -57,7 +57,7 @@ def test_tune_file_round_trip_and_override(tmp_path):
     assert res.stdout.split("\n")[0] == "(8, 7) (8, 4) (0, 1) (3, 2) (8, 8) 0", res.stdout
     assert "not a tune entry" in res.stderr
     res = subprocess.run([sys.executable, "-c", prog], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=dict(os.environ, LLMMM_TUNE_FILE=""))
-    assert res.returncode == 0 and "(3, 4) (8, 8)" in res.stdout, res.stdout + res.stderr
+    assert res.returncode == 0 and "(3, 3) (8, 8)" in res.stdout, res.stdout + res.stderr
 
 
 def test_shapes_near_a_tuned_one_inherit_its_tile():
@@ -66,7 +66,7 @@ def test_shapes_near_a_tuned_one_inherit_its_tile():
     q = lambda *a: llmmm_amd.query_config(_lib.OUT_FP8Q, *a)
     assert q(2048, 19456, 2560) == (_lib.TILE_256x256, 1)
     assert q(3072, 19456, 2560)[0] == _lib.TILE_256x256      # 1.5 x the tuned M: the tuned tile, the heuristic's split
-    assert q(1536, 2560, 9728)[0] == _lib.TILE_128x128       # between the entries at 1024 and 2048 (both 128 x 128)
+    assert q(1536, 2560, 9728)[0] == _lib.TILE_256x128       # between the entries at 1024 and 2048 (both 256 x 128)
     assert q(128, 6144, 2560)[0] == _lib.TILE_SKINNY         # M = 128 stays with its weight-streaming entry, not the tile tuned at 256
     assert q(96, 6144, 2560)[0] == _lib.TILE_SKINNY
 
