@@ -66,8 +66,9 @@ extern "C" {
 #define LLMMM_TILE_128x160 5 /* FP8 GEMM only, N % 160 == 0, fp32 / bf16 / residual-add outputs (no 1x128-grouped epilogue):
                               * 2560-column outputs in 16 tiles per row -- one tile per CU at M = 2048 */
 #define LLMMM_TILE_SKINNY 8 /* M <= 128 weight-streaming kernel */
-#define LLMMM_TILE_STRIP 9  /* FP8 GEMM, M <= 32, K >= 1024, fp32 / bf16 / residual-add outputs: the weight-streaming kernel in strips of
-                             * 16 columns over all of K -- the K split happens inside the workgroup, one launch, no workspace */
+#define LLMMM_TILE_STRIP 9  /* FP8 GEMM, M <= 32, K >= 1024, fp32 / bf16 / residual-add outputs, and the 1x128-grouped fp8 output for
+                             * M <= 16: the weight-streaming kernel in strips of 16 or 32 columns over all of K -- the K split
+                             * happens inside the workgroup, one launch, no workspace */
 
 /* Weight layout of the FP8 GEMM's B operand (llmmm_gemm_cfg.b_layout). */
 #define LLMMM_FP8_B_ROWS 0        /* Bt[N,K] row-major, the reference layout (examples/005.fp8.mm.cu:157) */
