@@ -76,4 +76,6 @@ def test_the_library_choice_is_close_to_the_measured_best(lib, N, K, tuned):
     auto = time_of()
     cands = {s: time_of(tile=_lib.TILE_SKINNY, split_k=s) for s in (1, 2, 3, 4, 5, 6, 8, 10) if s <= K // 256}
     best = min(cands, key=cands.get)
+    if auto > 1.15 * cands[best]:  # a timing, not a result: one more look at both before calling it
+        auto, cands[best] = min(auto, time_of()), min(cands[best], time_of(tile=_lib.TILE_SKINNY, split_k=best))
     assert auto <= 1.15 * cands[best], "M %d N %d K %d: the library's %s takes %.2f us, %d splits %.2f us" % (M, N, K, (tile, split), auto * 1e3, best, cands[best] * 1e3)
