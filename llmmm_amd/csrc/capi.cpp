@@ -120,7 +120,7 @@ int heuristic_tile(int M, int N)
     // Up to one tile per CU the small tile stays ahead (1024 x 4096 x 4096: 26.8 | 31.7 | 30.6 cold).
     float eff = c.eff;
     if (c.id == LLMMM_TILE_128x128 && tiles > NUM_CUS) eff = 0.74f;
-    if (c.id == LLMMM_TILE_256x128 && M >= 512) eff = 0.86f;  // (a single tile row of 256 prefers 128 x 256 on cached weights)
+    if (c.id == LLMMM_TILE_256x128) eff = 0.86f;  // (ahead of 128 x 256 on weights from HBM: 256 x 22016 x 4096 34.0 against 40.0 us)
     const float cost  = waves * c.per_cu * c.bm * c.bn / eff;
     if (best < 0 || cost < best_cost) {
       best      = c.id;
