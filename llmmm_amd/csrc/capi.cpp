@@ -396,15 +396,18 @@ bool strip_fits(int M, int N, int K) { return M >= 1 && M <= llmmm::STRIP_MAX_M 
 //  * more, but 32-column strips fit one round and the matrix is small (llmmm::strip_fragments; 6144 x 2560, 6144 x 4096,
 //    5120 x 5120): plain outputs as above (6144 x 4096 at M = 16: 7.5 / 8.8), fused up to M = 4 (6144 x 2560: 6.2 / 6.65 at M = 1,
 //    7.0 / 6.7 at 8; 6144 x 4096: 7.2 / 8.65 and 7.8 / 8.7; 5120 x 5120: 7.9 / 8.4 and 8.7 / 8.55);
-//  * exactly two 16-column strips per CU (8192 x 8192: 13.2 / 15.1 fused at M = 1, 14.3 / 15.3 at 8, 16.5 / 15.3 at 16);
-//  * otherwise not: 5120 x 13824 at M = 1 takes 19.5 us in 320 strips, a round and a quarter, and 14.8 us in six splits.
+//  * two 16-column strips on (nearly) every CU -- between 1.75 and 2 per CU, which share it side by side (8192 x 8192, 512
+//    strips: 13.2 / 15.1 fused at M = 1, 14.3 / 15.3 at 8, 16.5 / 15.3 at 16; 7168 x 5120, 448 strips: 10.3 / 11.7 at M = 1;
+//    8192 x 28672: 39.9 / 39.5 at M = 1 and 40.7 / 37.6 at 4, hence the same M * K bound as above);
+//  * otherwise not: 5120 x 13824 at M = 1 takes 19.5 us in 320 strips, a round and a quarter, and 14.8 us in six splits
+//    (5120 x 17408: 21.4 / 17.5; 10240 x 8192, 640 strips: 17.9 / 18.1).
 bool strips_pay(int M, int N, int K, bool fused)
 {
   const long cus = NUM_CUS, s16 = N / 16;
   const bool plain_ok = M <= 8 || (M <= 16 && K <= 4096);
   if (s16 <= cus) return fused ? (long)M * K <= 65536 : plain_ok;
   if (llmmm::strip_fragments(N, K) == 2) return fused ? M <= 4 : plain_ok;
-  if (s16 == 2 * cus) return fused ? M <= 8 : M <= 16;
+  if (s16 <= 2 * cus && s16 * 8 >= 2 * cus * 7) return (long)M * K <= (fused ? 65536 : 131072);  // (plain: 8192 x 8192 up to M = 16)
   return false;
 }
 // Plain outputs, one 16-column strip per CU, measured against the split form (bf16 out, us, strips / split + reduce):

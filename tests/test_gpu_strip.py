@@ -71,8 +71,8 @@ def _strips_pay(m, n, k, fused):
         return m * k <= 65536 and m <= 16 if fused else plain
     if n % 32 == 0 and n // 32 <= 256 and n * k <= 32 << 20:   # 32-column strips
         return m <= 4 if fused else plain
-    if n // 16 == 512:                                          # two 16-column strips on every CU
-        return m <= 8 if fused else m <= 16
+    if 448 <= n // 16 <= 512:                                   # two 16-column strips on (nearly) every CU
+        return m * k <= (65536 if fused else 131072)
     return False
 
 
@@ -101,7 +101,7 @@ def test_the_library_picks_strips_where_it_used_to_split(lib):
             assert raw.llmmm_fp8_gemm_qkv_rope_workspace(m, n, k) > 0
     assert lib.query_config(_lib.OUT_BF16, 1, 19456, 2560) == (SKINNY, 1)   # enough column groups: no split to replace
     # other model families: wide strips on small matrices, paired narrow ones at 8192 columns, none for a round and a quarter
-    for n, k in ((6144, 4096), (5120, 5120), (8192, 8192), (5120, 13824)):
+    for n, k in ((6144, 4096), (5120, 5120), (8192, 8192), (5120, 13824), (7168, 5120), (8192, 28672)):
         for m in (1, 4, 8, 16):
             for kind, fused in ((_lib.OUT_BF16, False), (_lib.OUT_FP8Q, True)):
                 got = lib.query_config(kind, m, n, k)
