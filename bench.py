@@ -39,6 +39,8 @@ TRAFFIC_PROFILES = {
     "fp8_gemm_fused_4096": ("fp8_gemm_kernel_fused_4096.txt", "fp8_gemm.hip"),
     "decode_gate_up_m1": ("fp8_skinny_kernel_gate_up_m1.txt", "fp8_skinny.hip"),
     "decode_gate_up_m1_pre": ("fp8_skinny_kernel_gate_up_m1_preshuffled.txt", "fp8_skinny.hip"),
+    "decode_o_m16_pre": ("fp8_strip_kernel_fused_quant_o_m16.txt", "fp8_skinny.hip"),
+    "decode_o_m1_bf16_pre": ("fp8_strip_kernel_o_m1.txt", "fp8_skinny.hip"),
 }
 
 
