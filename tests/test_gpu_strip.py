@@ -108,7 +108,7 @@ def test_the_library_picks_strips_where_it_used_to_split(lib):
                 assert got == (STRIP, 1) if _strips_pay(m, n, k, fused) else got[0] == SKINNY and got[1] > 1, (m, n, k, fused, got)
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 2560, 4096), (8, 2560, 9728), (16, 2560, 4096)])
+@pytest.mark.parametrize("M,N,K", [(1, 2560, 4096), (8, 2560, 9728), (16, 2560, 4096), (8, 5120, 5120)])  # (the last: 32-column strips)
 @pytest.mark.parametrize("dt", ["bf16", "f32", "f16"])
 def test_residual_add_and_planes_entry_points_take_strips(lib, oracle, M, N, K, dt):
     """llmmm_fp8_gemm_add_rmsnorm_quant on a strip shape: hidden == T(C32 + residual) with C32 the strip kernel's fp32 output,
