@@ -128,3 +128,12 @@ def test_bad_file_entries_are_dropped_not_obeyed(tmp_path):
     assert "line too long" in res.stderr and res.stderr.count("not a tune entry") == 2
     if not torch.cuda.is_available():
         assert out[-1] == "5", res.stdout    # the FP16 call gets as far as the launch (no device here): not "not aligned"
+
+
+def test_pick_best_prefers_fewer_splits_within_the_noise():
+    """Among candidates within 2 % of the fastest the driver records the one with the fewest splits (fewer fp32 planes)."""
+    from llmmm_amd import tune
+    assert tune.pick_best({(3, 3): 15.7, (3, 4): 15.7, (2, 8): 15.5, (0, 1): 24.0}) == (3, 3)
+    assert tune.pick_best({(0, 1): 196.3, (0, 3): 194.3, (2, 1): 288.0}) == (0, 1)
+    assert tune.pick_best({(3, 1): 85.0, (2, 1): 62.5, (1, 1): 66.5}) == (2, 1)          # a real difference is a real difference
+    assert tune.pick_best({(8, 4): 6.65, (8, 5): 6.60, (8, 8): 7.4}) == (8, 4)
