@@ -31,7 +31,9 @@ def _run(lib, Aq, As, Bq, Bs, M, N, K, pre=False, tile=STRIP, guard=3):
 @pytest.mark.parametrize("M,N,K", [(1, 2560, 4096), (16, 2560, 9728), (16, 6144, 2560), (5, 256, 1024), (32, 2560, 4096), (17, 128, 1152),
                                    (1, 128, 8192), (9, 512, 10240), (31, 384, 2560),
                                    # 32-column strips: 6144 x 2560 above; four waves per fragment with a tail slice, two row blocks, exactly 256 strips
-                                   (3, 4608, 1152), (24, 4608, 1152), (1, 8192, 1024), (16, 6144, 4096)])
+                                   (3, 4608, 1152), (24, 4608, 1152), (1, 8192, 1024), (16, 6144, 4096),
+                                   # 448 16-column strips of a matrix too large for wide ones: two workgroups on most CUs
+                                   (3, 7168, 5120)])
 def test_against_oracle(lib, oracle, M, N, K):
     Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=M + N + K)
     ref = oracle.fp8_gemm(Aq, As, Bq, Bs, promote=128)

@@ -49,7 +49,9 @@ def _check(oracle, lib, t, M, N, K, Cq, Cs, what, pre=False):
 @pytest.mark.parametrize("M,N,K", [(1, 2560, 4096), (16, 2560, 4096), (1, 6144, 2560), (16, 6144, 2560), (1, 2560, 9728), (8, 2560, 9728),
                                    (5, 128, 1024), (3, 384, 10240), (16, 256, 1152),
                                    # 32-column strips (6144 x 2560 above): tail slices, exactly 256 strips, a larger K
-                                   (3, 4608, 1152), (16, 4608, 1152), (2, 8192, 1024), (16, 6144, 4096)])
+                                   (3, 4608, 1152), (16, 4608, 1152), (2, 8192, 1024), (16, 6144, 4096),
+                                   # 448 16-column strips (56 groups) of a matrix too large for wide ones: two workgroups on most CUs
+                                   (2, 7168, 5120)])
 @pytest.mark.parametrize("pre", [False, True])
 def test_against_oracle(lib, oracle, M, N, K, pre):
     Aq, As, Bq, Bs = fp8_inputs(oracle, M, N, K, seed=M + N + K)
